@@ -1,0 +1,203 @@
+"""Exported operators: the callable objects behind ``autort.export`` and
+``autort.ops.<name>``.
+
+The calling convention follows the call sites of the reference's samples:
+tensors are passed positionally in the order of the ``inputs=`` list
+(samples/01_sort_even_first.py:22,27); a tensor of that list which the program
+writes is updated in place; an output that is not in the list is allocated, or
+taken from a trailing positional argument (samples/05_llama2_7b_int4.py:157) or
+from ``out=`` (samples/05_llama2_7b_int4.py:144), and returned.  Outputs may be
+views into larger tensors as long as the view itself is contiguous.  Kernels are
+enqueued on torch's current stream and never synchronise.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..ir import Graph, fuse_elementwise, parse_program
+from ..lower import lower_graph
+from ..runtime import capi
+
+TORCH_DTYPE = {'float64': torch.float64, 'float32': torch.float32, 'float16': torch.float16,
+               'int64': torch.int64, 'int32': torch.int32, 'int16': torch.int16, 'int8': torch.int8,
+               'uint8': torch.uint8}
+_COMPATIBLE = {('int8', torch.uint8), ('uint8', torch.int8)}     # same bits, reinterpreted
+
+_CACHE_DIR = os.environ.get('AUTORT_CACHE_DIR') or os.path.join(
+    os.path.dirname(os.path.dirname(os.path.abspath(__file__))), '_cache')
+
+
+def current_stream_handle() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def compile_cached(source: str) -> bytes:
+    """HIP source -> code object.  Code objects are cached on disk by the hash
+    of their source, so a process only compiles what no earlier process has
+    compiled.  Needs no GPU."""
+    key = hashlib.sha256(source.encode()).hexdigest()[:24]
+    path = os.path.join(_CACHE_DIR, key + '.hsaco')
+    if os.path.exists(path):
+        with open(path, 'rb') as f:
+            image = f.read()
+    else:
+        image = capi.compile_hip(source)
+        try:
+            os.makedirs(_CACHE_DIR, exist_ok=True)
+            tmp = f'{path}.tmp{os.getpid()}'
+            with open(tmp, 'wb') as f:
+                f.write(image)
+            os.replace(tmp, path)
+        except OSError:
+            pass                     # a read-only tree only costs the recompilation next time
+    return image
+
+
+class ExportedOp:
+    """One einstein_v2 program bound to gfx950 kernels."""
+
+    def __init__(self, ir: str, inputs, config: Optional[str] = None, name: Optional[str] = None,
+                 extra_outputs: Sequence[str] = ()):
+        self.ir = ir
+        self.config = parse_config(config)
+        self.graph: Graph = parse_program(ir, inputs, extra_outputs)
+        self.fused: Graph = fuse_elementwise(self.graph)
+        self.name = name or self.graph.outputs[-1]
+        self.declared = list(self.graph.declared)
+        self.inout = list(self.graph.inout)
+        # outputs the caller does not pass among the declared tensors
+        self.fresh_outputs = [o for o in self.graph.outputs if o not in self.declared]
+        self.source, self.plans = lower_graph(self.fused, prefix='autort_' + _ident(self.name))
+        self._module: Optional[capi.Module] = None
+        self._image: Optional[bytes] = None
+        from . import patterns
+        self.fast_path = patterns.match(self.fused)
+
+    # -- compilation ---------------------------------------------------------
+    def compile(self) -> 'ExportedOp':
+        """Builds the generic kernels (or finds them in the cache).  Needs no GPU."""
+        if self._image is None:
+            self._image = compile_cached(self.source)
+        return self
+
+    def _load(self) -> capi.Module:
+        if self._module is None:
+            self.compile()
+            self._module = capi.Module(self._image)
+        return self._module
+
+    # -- calling -------------------------------------------------------------
+    def __call__(self, *tensors, extra=None, out=None):
+        g = self.fused
+        nd = len(self.declared)
+        if len(tensors) < nd:
+            raise TypeError(f'{self.name}() takes {nd} tensor(s) {self.declared}, got {len(tensors)}')
+        bound: Dict[str, torch.Tensor] = dict(zip(self.declared, tensors[:nd]))
+        trailing = list(tensors[nd:])
+        if len(trailing) > len(self.fresh_outputs):
+            raise TypeError(f'{self.name}() got {len(tensors)} tensors but declares {nd} inputs and '
+                            f'{len(self.fresh_outputs)} output(s)')
+        for n, t in zip(self.fresh_outputs, trailing):
+            bound[n] = t
+        if out is not None:
+            if not self.fresh_outputs:
+                raise TypeError(f'{self.name}() has no separate output tensor to pass as out=')
+            bound[self.fresh_outputs[-1]] = out
+        dev = None
+        for n, t in bound.items():
+            self._check_tensor(n, t)
+            dev = dev or t.device
+        if dev is None:
+            dev = torch.device('cuda', torch.cuda.current_device())
+        if dev.type != 'cuda':
+            raise RuntimeError(f'{self.name}(): tensors must live on the GPU (got {dev}); there is no CPU fallback')
+        env = g.bind_dims({n: tuple(bound[n].shape) for n in self.declared if n in g.tensors})
+        for n in self.fresh_outputs:
+            want = g.shape_of(n, env)
+            if n in bound:
+                if bound[n].numel() != _numel(want):
+                    raise ValueError(f'output `{n}` expects {want} ({_numel(want)} elements), got {list(bound[n].shape)}')
+            else:
+                bound[n] = torch.empty(want, dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)
+        capi.init(dev.index or 0)
+        stream = current_stream_handle()
+        if self.fast_path is None or not self.fast_path(self, bound, env, stream):
+            self._run_generic(bound, env, dev, stream)
+        outs = [bound[o] for o in self.graph.outputs]
+        return outs[0] if len(outs) == 1 else tuple(outs)
+
+    def _check_tensor(self, name: str, t: torch.Tensor):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f'argument `{name}` must be a torch.Tensor, got {type(t).__name__}')
+        info = self.fused.tensors.get(name) or self.graph.tensors[name]
+        want = TORCH_DTYPE[info.dtype]
+        if t.dtype != want and (info.dtype, t.dtype) not in _COMPATIBLE:
+            raise TypeError(f'tensor `{name}` must be {info.dtype}, got {t.dtype}')
+        if not t.is_contiguous():
+            raise ValueError(f'tensor `{name}` must be contiguous (views are fine if they are dense)')
+
+    def _run_generic(self, bound: Dict[str, torch.Tensor], env: Dict[str, int], dev, stream: int):
+        module = self._load()
+        g = self.fused
+        dims = [env[d] for d in g.dim_names]
+        for plan in self.plans:
+            for n in plan.args:
+                if n not in bound:         # intermediate (reduce result) of a multi-kernel program
+                    bound[n] = torch.empty(g.shape_of(n, env), dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)
+            ptrs = {n: bound[n].data_ptr() for n in plan.args}
+            sym, grid, block = plan.choose(env, ptrs)
+            if grid == 0:
+                continue
+            capi.launch(module.function(sym), (grid, 1, 1), (block, 1, 1), stream,
+                        [ptrs[n] for n in plan.args] + dims)
+
+    def __repr__(self):
+        return f'<autort op {self.name}: {" ".join(self.ir.split())[:80]}>'
+
+
+def parse_config(config: Optional[str]) -> Dict[str, object]:
+    """Tuning hints such as ``"tune:5"`` or ``"~N~:[256,8,32],~S~:[64,8]"``
+    (README.md:66, samples/05_llama2_7b_int4.py:139).  The grammar is not
+    documented; unknown keys are kept verbatim and never rejected."""
+    out: Dict[str, object] = {}
+    if not config:
+        return out
+    depth, cur, parts = 0, '', []
+    for ch in config:
+        if ch in '[(':
+            depth += 1
+        elif ch in '])':
+            depth -= 1
+        if ch == ',' and depth == 0:
+            parts.append(cur)
+            cur = ''
+        else:
+            cur += ch
+    if cur.strip():
+        parts.append(cur)
+    for p in parts:
+        k, _, v = p.partition(':')
+        k, v = k.strip(), v.strip()
+        if not k:
+            continue
+        try:
+            import json
+            out[k] = json.loads(v)
+        except Exception:
+            out[k] = v
+    return out
+
+
+def _ident(name: str) -> str:
+    return ''.join(c if c.isalnum() else '_' for c in name)
+
+
+def _numel(shape) -> int:
+    n = 1
+    for s in shape:
+        n *= s
+    return n

@@ -1,0 +1,93 @@
+"""Recognition of operator patterns that have a hand-written gfx950 kernel.
+
+A program is recognised by the canonical text of its fused statements (tensor
+and axis names replaced by order of appearance), so the user's spelling of
+names does not matter.  A handler returns True when it ran the operator, or
+False to leave it to the generic lowering (shapes it does not cover).
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, Optional
+
+from ctypes import c_void_p
+
+from ..ir import Graph, fuse_elementwise, parse_program
+from ..runtime import capi
+
+_TABLE: Dict[str, Callable] = {}
+
+
+def register(ir: str, inputs, handler: Callable):
+    key = fuse_elementwise(parse_program(ir, inputs)).canonical_key()
+    _TABLE[key] = handler
+    return key
+
+
+def match(fused: Graph) -> Optional[Callable]:
+    return _TABLE.get(fused.canonical_key())
+
+
+# ---------------------------------------------------------------------------
+# int4 GEMV in the reference's weight format (samples/05_llama2_7b_int4.py:135-139)
+# ---------------------------------------------------------------------------
+GPTQ_GEMV_IR = """
+  input1[S, N] = (qweight[S / 8, N] >> (S % 8 * 4)).call(strs.bitwise_and, 15) * input0[S].like(1)
+  w[S, N] = scales[S / 128, N] * (input1[S, N] - 8)
+  my_result[N] +=! input0[S] * w[S, N].to(input0.dtype())
+"""
+
+
+def _gptq_inputs(xdt: str, sdt: str):
+    return [f'input0={xdt}[S:4096]', 'qweight=int32[L:512, N:12288]', f'scales={sdt}[K:32, N:12288]']
+
+
+def _gptq_handler(op, bound, env, stream) -> bool:
+    g = op.fused
+    x_name, q_name, s_name = g.abi_inputs[0], g.abi_inputs[1], g.abi_inputs[2]
+    # abi order is sorted by name; find roles by dtype / rank instead
+    names = {n: g.tensors[n] for n in g.abi_inputs}
+    q_name = next(n for n, t in names.items() if t.dtype == 'int32')
+    x_name = next(n for n, t in names.items() if len(t.shape) == 1)
+    s_name = next(n for n in names if n not in (q_name, x_name))
+    out = bound[g.abi_outputs[0]]
+    x, q, s = bound[x_name], bound[q_name], bound[s_name]
+    K, N = x.shape[0], q.shape[1]
+    if K % 128 or N % 4 or q.shape[0] * 8 != K or s.shape[0] * 128 != K or q.data_ptr() % 16:
+        return False
+    capi.check(capi.lib().art_gemv_gptq(c_void_p(x.data_ptr()), c_void_p(q.data_ptr()), c_void_p(s.data_ptr()),
+                                       c_void_p(out.data_ptr()), K, N, int(names[x_name].dtype == 'float16'),
+                                       int(names[s_name].dtype == 'float16'), c_void_p(stream)))
+    return True
+
+
+for _x in ('float32', 'float16'):
+    for _s in ('float32', 'float16'):
+        register(GPTQ_GEMV_IR, _gptq_inputs(_x, _s), _gptq_handler)
+
+
+# ---------------------------------------------------------------------------
+# int4 g128 GEMV / skinny GEMM with per-group zero points:
+#   y[m,n] = sum_k x[m,k] * fp16( s[k/128,n] * (q[k,n] - z[k/128,n]) )     fp32 accumulate, fp16 out
+# qweight uint8 [K/2,N] (low nibble = even k), qzeros uint8 [K/128,N/2] (low nibble = even n).
+# ---------------------------------------------------------------------------
+W4A16_IR = """
+  acc[M, N] +=! x[M, K].to(`float32`) * (scales[K / 128, N] * (((qweight[K / 2, N] >> (K % 2 * 4)).call(strs.bitwise_and, 15) - (qzeros[K / 128, N / 2] >> (N % 2 * 4)).call(strs.bitwise_and, 15)) * scales[K / 128, N].like(1))).to(`float32`)
+  y[M, N] = acc[M, N].to(`float16`)
+"""
+W4A16_INPUTS = ['x=float16[M:1, K:4096]', 'qweight=int8[KH:2048, N:11008]', 'scales=float16[G:32, N:11008]',
+                'qzeros=int8[G:32, NH:5504]']
+
+
+def _w4a16_handler(op, bound, env, stream) -> bool:
+    x, q, s, z, y = bound['x'], bound['qweight'], bound['scales'], bound['qzeros'], bound['y']
+    M, K = x.shape
+    N = q.shape[1]
+    if M > 8 or K % 128 or N % 16 or q.shape[0] * 2 != K or s.shape[0] * 128 != K or z.shape[1] * 2 != N \
+            or q.data_ptr() % 16 or x.data_ptr() % 4:
+        return False
+    capi.check(capi.lib().art_gemv_w4a16(c_void_p(x.data_ptr()), c_void_p(q.data_ptr()), c_void_p(s.data_ptr()),
+                                        c_void_p(z.data_ptr()), c_void_p(y.data_ptr()), M, K, N, c_void_p(stream)))
+    return True
+
+
+register(W4A16_IR, W4A16_INPUTS, _w4a16_handler)

@@ -1,0 +1,48 @@
+// Shared helpers of libantares_amd.so: error reporting and launch checks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string>
+
+#include "../../include/antares_amd.h"
+
+namespace art {
+
+std::string& last_error();
+int fail(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+struct Workspace {
+  void* base = nullptr;      // device memory
+  size_t bytes = 0;
+};
+// Workspace of the current device (allocated by art_init).
+Workspace& workspace();
+
+// Workspace layout.  Ticket words must read zero whenever no kernel is running,
+// so they never share bytes with scratch data.
+constexpr size_t kGemvTicketOffset = 0;                 // 16384 ticket words of the split-K kernels
+constexpr size_t kGemvTicketBytes = 64 * 1024;
+constexpr size_t kScanTicketOffset = 64 * 1024;          // ticket words of the scan / partition kernels
+constexpr size_t kScratchOffset = 128 * 1024;            // partial sums, tile counts (any content)
+
+}  // namespace art
+
+#define ART_HIP(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t _e = (expr);                                                             \
+    if (_e != hipSuccess)                                                               \
+      return art::fail("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+  } while (0)
+
+#define ART_REQUIRE(cond, ...)            \
+  do {                                    \
+    if (!(cond)) return art::fail(__VA_ARGS__); \
+  } while (0)
+
+#define ART_LAUNCH_CHECK()                                                                \
+  do {                                                                                    \
+    hipError_t _e = hipGetLastError();                                                    \
+    if (_e != hipSuccess)                                                                 \
+      return art::fail("kernel launch failed: %s (%s:%d)", hipGetErrorString(_e), __FILE__, __LINE__); \
+  } while (0)

@@ -1,0 +1,220 @@
+// Device runtime of libantares_amd.so: initialisation, in-process compilation
+// of generated HIP source, code-object loading, kernel launch and timing.
+// This is the counterpart of the reference's `namespace ab` for HIP
+// (backends/c-rocm/include/backend.hpp:46-253) behind a flat C ABI.
+#include <hip/hiprtc.h>
+#include <string.h>
+
+#include <mutex>
+#include <vector>
+
+#include "art_common.h"
+
+namespace art {
+
+std::string& last_error() {
+  static thread_local std::string e;
+  return e;
+}
+
+int fail(const char* fmt, ...) {
+  char buf[2048];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  last_error() = buf;
+  return 1;
+}
+
+static constexpr int kMaxDevices = 16;
+static Workspace g_ws[kMaxDevices];
+static std::mutex g_mu;
+
+Workspace& workspace() {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  return g_ws[dev < 0 || dev >= kMaxDevices ? 0 : dev];
+}
+
+static std::string& compile_log() {
+  static thread_local std::string s;
+  return s;
+}
+
+}  // namespace art
+
+struct art_module {
+  hipModule_t handle;
+};
+struct art_func {
+  hipFunction_t handle;
+};
+
+// 16 MiB: split-K partial sums and tile states of the scan kernels.
+static constexpr size_t kWorkspaceBytes = 16u << 20;
+
+extern "C" {
+
+const char* art_last_error(void) { return art::last_error().c_str(); }
+const char* art_compile_log(void) { return art::compile_log().c_str(); }
+size_t art_workspace_bytes(void) { return kWorkspaceBytes; }
+
+int art_init(int device) {
+  int count = 0;
+  ART_HIP(hipGetDeviceCount(&count));
+  ART_REQUIRE(device >= 0 && device < count && device < art::kMaxDevices, "art_init: no such device %d (have %d)", device, count);
+  ART_HIP(hipSetDevice(device));
+  std::lock_guard<std::mutex> lock(art::g_mu);
+  art::Workspace& ws = art::g_ws[device];
+  if (!ws.base) {
+    ART_HIP(hipMalloc(&ws.base, kWorkspaceBytes));
+    ART_HIP(hipMemset(ws.base, 0, kWorkspaceBytes));
+    ws.bytes = kWorkspaceBytes;
+  }
+  return 0;
+}
+
+int art_device_props(art_props* out) {
+  ART_REQUIRE(out != nullptr, "art_device_props: null output");
+  int dev = 0;
+  ART_HIP(hipGetDevice(&dev));
+  hipDeviceProp_t p;
+  ART_HIP(hipGetDeviceProperties(&p, dev));
+  memset(out, 0, sizeof(*out));
+  snprintf(out->name, sizeof(out->name), "%s", p.name);
+  snprintf(out->arch, sizeof(out->arch), "%s", p.gcnArchName);
+  if (char* colon = strchr(out->arch, ':')) *colon = 0;
+  out->compute_units = p.multiProcessorCount;
+  out->wavefront_size = p.warpSize;
+  out->max_threads_per_block = p.maxThreadsPerBlock;
+  out->lds_bytes_per_block = (int)p.sharedMemPerBlock;
+  out->clock_khz = p.clockRate;
+  out->memory_clock_khz = p.memoryClockRate;
+  out->memory_bus_width_bits = p.memoryBusWidth;
+  out->l2_bytes = p.l2CacheSize;
+  out->total_memory_bytes = p.totalGlobalMem;
+  return 0;
+}
+
+int art_module_compile(const char* hip_source, const char* arch, void** blob, size_t* size) {
+  ART_REQUIRE(hip_source && blob && size, "art_module_compile: null argument");
+  art::compile_log().clear();
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, hip_source, "autort_kernel.hip", 0, nullptr, nullptr);
+  ART_REQUIRE(r == HIPRTC_SUCCESS, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+  std::string arch_opt = std::string("--offload-arch=") + ((arch && *arch) ? arch : "gfx950");
+  // Packed-FP32 instruction selection is switched off for every kernel of this library.
+  const char* opts[] = {arch_opt.c_str(), "-O3", "-std=c++17", "-Wno-ignored-attributes",
+                        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  r = hiprtcCompileProgram(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+  size_t log_size = 0;
+  hiprtcGetProgramLogSize(prog, &log_size);
+  if (log_size > 1) {
+    art::compile_log().resize(log_size);
+    hiprtcGetProgramLog(prog, &art::compile_log()[0]);
+  }
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    return art::fail("compilation failed: %s\n%s", hiprtcGetErrorString(r), art::compile_log().c_str());
+  }
+  size_t n = 0;
+  hiprtcGetCodeSize(prog, &n);
+  void* mem = malloc(n);
+  if (!mem) {
+    hiprtcDestroyProgram(&prog);
+    return art::fail("art_module_compile: out of host memory");
+  }
+  hiprtcGetCode(prog, (char*)mem);
+  hiprtcDestroyProgram(&prog);
+  *blob = mem;
+  *size = n;
+  return 0;
+}
+
+void art_blob_free(void* blob) { free(blob); }
+
+int art_module_load(const void* image, size_t size, art_module** out) {
+  ART_REQUIRE(image && size > 0 && out, "art_module_load: null argument");
+  hipModule_t m;
+  ART_HIP(hipModuleLoadData(&m, image));
+  *out = new art_module{m};
+  return 0;
+}
+
+int art_module_unload(art_module* module) {
+  ART_REQUIRE(module != nullptr, "art_module_unload: null module");
+  ART_HIP(hipModuleUnload(module->handle));
+  delete module;
+  return 0;
+}
+
+int art_get_function(art_module* module, const char* name, art_func** out) {
+  ART_REQUIRE(module && name && out, "art_get_function: null argument");
+  hipFunction_t f;
+  hipError_t e = hipModuleGetFunction(&f, module->handle, name);
+  if (e != hipSuccess) return art::fail("kernel `%s` not found in module: %s", name, hipGetErrorString(e));
+  *out = new art_func{f};
+  return 0;
+}
+
+int art_launch(art_func* func, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
+               unsigned lds_bytes, void* stream, const uint64_t* args, int nargs) {
+  ART_REQUIRE(func != nullptr, "art_launch: null function");
+  ART_REQUIRE(nargs >= 0 && nargs <= 64, "art_launch: bad argument count %d", nargs);
+  ART_REQUIRE(bx * by * bz >= 1 && bx * by * bz <= 1024, "art_launch: bad block %ux%ux%u", bx, by, bz);
+  if (gx == 0 || gy == 0 || gz == 0) return 0;   // empty iteration space: nothing to run
+  void* params[64];
+  for (int i = 0; i < nargs; ++i) params[i] = (void*)&args[i];
+  ART_HIP(hipModuleLaunchKernel(func->handle, gx, gy, gz, bx, by, bz, lds_bytes, (hipStream_t)stream, params, nullptr));
+  return 0;
+}
+
+int art_event_create(void** event) {
+  ART_REQUIRE(event != nullptr, "art_event_create: null output");
+  hipEvent_t e;
+  ART_HIP(hipEventCreate(&e));
+  *event = e;
+  return 0;
+}
+int art_event_record(void* event, void* stream) {
+  ART_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+  return 0;
+}
+int art_event_elapsed_ms(void* start, void* stop, float* ms) {
+  ART_REQUIRE(ms != nullptr, "art_event_elapsed_ms: null output");
+  ART_HIP(hipEventSynchronize((hipEvent_t)stop));
+  ART_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return 0;
+}
+int art_event_destroy(void* event) {
+  ART_HIP(hipEventDestroy((hipEvent_t)event));
+  return 0;
+}
+int art_stream_synchronize(void* stream) {
+  ART_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return 0;
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------ copy kernel
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void art_copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, size_t nvec) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (; i < nvec; i += stride) dst[i] = __builtin_nontemporal_load(&src[i]);
+}
+
+extern "C" int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* stream) {
+  ART_REQUIRE(((uintptr_t)dst_dev % 16) == 0 && ((uintptr_t)src_dev % 16) == 0 && bytes % 16 == 0,
+              "art_copy_bytes: pointers and size must be multiples of 16");
+  size_t nvec = bytes / 16;
+  if (nvec == 0) return 0;
+  size_t blocks = (nvec + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  art_copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>((u32x4*)dst_dev, (const u32x4*)src_dev, nvec);
+  ART_LAUNCH_CHECK();
+  return 0;
+}

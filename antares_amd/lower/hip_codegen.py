@@ -1,0 +1,374 @@
+"""Generic lowering of einstein_v2 statements to HIP kernels for gfx950.
+
+Replaces the reference's TVM-driven code generation for the c-rocm backend
+(antares/default_codegen.py:13-358 with the three schedules under
+backends/c-rocm/schedule/standard/) by direct emission from hand-written
+templates:
+
+* elementwise / gather statements: one flat grid-stride loop; when every tensor
+  is read and written at the same flat position the kernel moves 16-byte
+  vectors per lane (the reference's untuned default is one scalar element per
+  block, antares/common.py:81-100);
+* reduce statements: three variants compiled together — one wavefront per
+  output (DPP / readlane reduction), one 256-thread block per output, one
+  thread per output — and the launcher picks by extents and by which axis is
+  contiguous in memory (the reference reduces through LDS because its TVM patch
+  disables wavefront shuffles off CUDA, engine/device-stub/tvm_v0.8.0.patch:186-191);
+* scatter statements: one thread per point of the iteration space, atomics for
+  ``+=.  <=.  >=.``.
+
+Kernel signatures follow the reference's HIP kernel ABI
+(backends/c-rocm/config.py:25-85): tensor pointers first, in the order given by
+the caller, then the named run-time dimensions as ``int`` arguments.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Tuple
+
+from ..ir.nodes import Expr, ITEMSIZE, walk
+from .hip_prelude import PRELUDE
+
+HIP_TYPE = {'float64': 'double', 'float32': 'float', 'float16': 'half_t', 'int64': 'long long', 'int32': 'int',
+            'int16': 'short', 'int8': 'signed char', 'uint8': 'unsigned char'}
+
+BLOCK = 256
+MAX_GRID = 256 * 32       # 256 CUs, enough resident blocks each to hide HBM latency
+
+_CALLS = {'max': 'art_max', 'min': 'art_min', 'abs': 'art_abs', 'rsqrt': 'art_rsqrt', 'normcdf': 'art_normcdf'}
+_REDUCE_OP = {'+': 'OpAdd', '*': 'OpMul', '>': 'OpMax', '<': 'OpMin', '|': 'OpAny', '&': 'OpAll'}
+
+
+def dim_c(d) -> str:
+    return str(d) if isinstance(d, int) else f'__dim_{d}'
+
+
+def reduce_identity(op: str, dtype: str) -> str:
+    """Start value of each reduce operator (antares/default_codegen.py:113-128)."""
+    ct = HIP_TYPE[dtype]
+    if op in ('+', '|'):
+        return f'({ct})0'
+    if op in ('*', '&'):
+        return f'({ct})1'
+    hi = {'float64': '1.7976931348623157e308', 'float32': '3.402823466e38f', 'float16': '65504.0f',
+          'int64': '9223372036854775807LL', 'int32': '2147483647', 'int16': '32767', 'int8': '127', 'uint8': '255'}[dtype]
+    lo = {'int64': '(-9223372036854775807LL-1)', 'int32': '(-2147483647-1)', 'int16': '-32768', 'int8': '-128',
+          'uint8': '0'}.get(dtype, '-' + hi)
+    return f'({ct})({lo if op == ">" else hi})'
+
+
+def const_c(value, dtype: str) -> str:
+    if dtype == 'float32':
+        return repr(float(value)) + 'f'
+    if dtype == 'float64':
+        return repr(float(value))
+    if dtype == 'float16':
+        return f'((half_t){float(value)!r}f)'
+    return f'(({HIP_TYPE[dtype]}){int(value)})'
+
+
+class ExprEmitter:
+    """IR expression -> HIP C++ text.  ``load_override`` lets the vector kernels
+    replace tensor loads by lanes of a register vector."""
+
+    def __init__(self, tensors, load_override: Optional[Callable[[Expr], Optional[str]]] = None):
+        self.tensors = tensors
+        self.load_override = load_override
+
+    def offset(self, name: str, idx: List[str]) -> str:
+        shape = self.tensors[name].shape
+        terms = []
+        for i, ix in enumerate(idx):
+            stride = ' * '.join(f'(long long){dim_c(d)}' for d in shape[i + 1:])
+            terms.append(f'({ix}) * {stride}' if stride else f'({ix})')
+        return ' + '.join(terms) if terms else '0'
+
+    def expr(self, n: Expr) -> str:
+        k, ct = n.kind, HIP_TYPE[n.dtype]
+        if k == 'const':
+            return const_c(n.value, n.dtype)
+        if k == 'axis':
+            return n.name
+        if k == 'axis_range':
+            return f'__ext_{n.name}'
+        if k == 'dim':
+            return dim_c(n.value)
+        if k == 'load':
+            if self.load_override is not None:
+                o = self.load_override(n)
+                if o is not None:
+                    return o
+            return f'{n.name}[{self.offset(n.name, [self.expr(a) for a in n.args])}]'
+        if k == 'cast':
+            return f'(({ct})({self.expr(n.args[0])}))'
+        if k == 'op':
+            if n.name == '~':
+                return f'(({ct})(!({self.expr(n.args[0])})))'
+            a, b = self.expr(n.args[0]), self.expr(n.args[1])
+            sym = {'//': '/', '&': '&&', '|': '||'}.get(n.name, n.name)
+            return f'(({ct})({a} {sym} {b}))'
+        if k == 'call':
+            args = ', '.join(self.expr(a) for a in n.args)
+            return f'(({ct}){_CALLS.get(n.name, n.name)}({args}))'
+        if k == 'when':
+            if len(n.args) == 1:
+                raise ValueError('one-armed when() is only valid at the root of a statement')
+            rel = ' && ' if n.merge == 'all' else ' || '
+            cond = rel.join(f'({self.expr(c)})' for c in n.conds) or '1'
+            return f'(({cond}) ? ({self.expr(n.args[0])}) : ({self.expr(n.args[1])}))'
+        raise ValueError(f'unhandled node kind {k}')
+
+
+@dataclass
+class KernelPlan:
+    """Everything the runtime needs to launch one statement."""
+    name: str                      # base kernel name
+    args: List[str]                # tensor argument order
+    dims: List[str]                # named dimensions passed after the tensors
+    variants: Dict[str, str]       # variant tag -> kernel symbol
+    kind: str                      # 'map' | 'reduce' | 'scatter'
+    output: str
+    data_axes: List[Tuple[str, object]]
+    reduce_axes: List[Tuple[str, object]]
+    vec: int = 1                   # elements per lane in the vector variant
+    vec_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for it
+    reduce_contiguous: Optional[bool] = None   # True: a reduce axis is fastest in the biggest operand
+
+    def choose(self, env: Dict[str, int], pointers: Dict[str, int]) -> Tuple[str, int, int]:
+        """-> (kernel symbol, grid.x, block.x) for these extents and addresses."""
+        total = 1
+        for _, e in self.data_axes:
+            total *= e if isinstance(e, int) else env[e]
+        red = 1
+        for _, e in self.reduce_axes:
+            red *= e if isinstance(e, int) else env[e]
+        if total == 0:
+            return next(iter(self.variants.values())), 0, BLOCK
+        if self.kind == 'map':
+            if 'vec' in self.variants and all(pointers[t] % 16 == 0 for t in self.vec_tensors) and total >= self.vec:
+                work = (total + self.vec - 1) // self.vec
+                return self.variants['vec'], min((work + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
+            return self.variants['scalar'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
+        if self.kind == 'scatter':
+            return self.variants['scalar'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
+        # reduce
+        lanes_ok = self.reduce_contiguous is not False
+        if red >= 2048 and total <= 1024 and lanes_ok:
+            return self.variants['block'], min(total, MAX_GRID), BLOCK
+        if red >= 64 and lanes_ok and (self.reduce_contiguous or total < 64 * 1024):
+            waves_per_block = BLOCK // 64
+            return self.variants['wave'], min((total + waves_per_block - 1) // waves_per_block, MAX_GRID), BLOCK
+        return self.variants['thread'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
+
+
+def _signature(name: str, args: List[str], tensors, dims: List[str], written: List[str]) -> str:
+    ps = []
+    for a in args:
+        ct = HIP_TYPE[tensors[a].dtype]
+        ps.append(f'{ct}* __restrict__ {a}' if a in written else f'const {ct}* __restrict__ {a}')
+    ps += [f'int {dim_c(d)}' for d in dims]
+    return f'extern "C" __global__ __launch_bounds__({BLOCK}) void {name}({", ".join(ps)})'
+
+
+def _extents(st) -> List[str]:
+    return [f'  const int __ext_{ax} = {dim_c(e)}; (void)__ext_{ax};' for ax, e in st.data_axes + st.reduce_axes]
+
+
+def _decompose(var: str, axes, indent: str) -> List[str]:
+    out = [f'{indent}long long __r = {var};']
+    for ax, _ in reversed(axes):
+        out.append(f'{indent}const int {ax} = (int)(__r % __ext_{ax}); __r /= __ext_{ax};')
+    return out
+
+
+def _root_and_cond(st, em: ExprEmitter):
+    root, cond = st.root, None
+    if root.kind == 'when' and len(root.args) == 1:
+        rel = ' && ' if root.merge == 'all' else ' || '
+        cond = rel.join(f'({em.expr(c)})' for c in root.conds)
+        root = root.args[0]
+    return root, cond
+
+
+def _is_flat_map(st, tensors) -> bool:
+    """True when every load (and the store) addresses element ``flat`` of a
+    tensor whose extents equal the statement's data extents."""
+    axes = [a for a, _ in st.data_axes]
+    exts = [e for _, e in st.data_axes]
+    if st.scatter or st.reduce_axes or [i.name for i in st.out_index if i.kind == 'axis'] != axes:
+        return False
+    if list(tensors[st.output].shape) != exts:
+        return False
+    for e in [st.root]:
+        for n in walk(e):
+            if n.kind == 'load':
+                if [a.name if a.kind == 'axis' else None for a in n.args] != axes:
+                    return False
+                if list(tensors[n.name].shape) != exts:
+                    return False
+    # bare axes outside of loads need the decomposed index; allow them only in 1-D
+    loads_axes = 0
+    all_axes = 0
+    for n in walk(st.root):
+        if n.kind == 'axis':
+            all_axes += 1
+        if n.kind == 'load':
+            loads_axes += sum(1 for a in n.args if a.kind == 'axis')
+    return all_axes == loads_axes or len(axes) == 1
+
+
+def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
+    tensors, dims = graph.tensors, graph.dim_names
+    reads = [r for r in st.reads]
+    args = sorted(set(reads) - {st.output}) + [st.output]
+    written = [st.output]
+    em = ExprEmitter(tensors)
+    total = ' * '.join(f'(long long)__ext_{ax}' for ax, _ in st.data_axes) or '1LL'
+    oct_ = HIP_TYPE[st.out_dtype]
+    src: List[str] = []
+    variants: Dict[str, str] = {}
+    plan = KernelPlan(name=name, args=args, dims=dims, variants=variants,
+                      kind='scatter' if st.scatter else ('reduce' if st.reduce_axes else 'map'),
+                      output=st.output, data_axes=list(st.data_axes), reduce_axes=list(st.reduce_axes))
+
+    def header(sym):
+        return [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st) + \
+               [f'  const long long __total = {total};',
+                f'  const long long __tid = (long long)blockIdx.x * {BLOCK} + threadIdx.x;',
+                f'  const long long __nthr = (long long)gridDim.x * {BLOCK};']
+
+    root, cond = _root_and_cond(st, em)
+    dst = f'{st.output}[{em.offset(st.output, [em.expr(i) for i in st.out_index])}]'
+
+    if plan.kind == 'map':
+        sym = name
+        body = header(sym)
+        body.append('  for (long long __i = __tid; __i < __total; __i += __nthr) {')
+        body += _decompose('__i', st.data_axes, '    ')
+        store = f'{dst} = ({oct_})({em.expr(root)});'
+        body.append(f'    if ({cond}) {{ {store} }}' if cond else f'    {store}')
+        body += ['  }', '}']
+        src.append('\n'.join(body))
+        variants['scalar'] = sym
+        if _is_flat_map(st, tensors) and cond is None:
+            names = sorted({n.name for n in walk(root) if n.kind == 'load'} | {st.output})
+            width = max(ITEMSIZE[tensors[n].dtype] for n in names)
+            V = max(1, 16 // width)
+            if V > 1:
+                sym = name + '_v'
+                body = header(sym)
+                for n in names:
+                    body.append(f'  typedef {HIP_TYPE[tensors[n].dtype]} __vec_{n} __attribute__((ext_vector_type({V})));')
+                body.append(f'  const long long __nvec = __total / {V};')
+                body.append('  for (long long __v = __tid; __v < __nvec; __v += __nthr) {')
+                for n in names:
+                    if n != st.output or n in reads:
+                        body.append(f'    const __vec_{n} __in_{n} = ((const __vec_{n}*){n})[__v];')
+                body.append(f'    __vec_{st.output} __out;')
+                vem = ExprEmitter(tensors, load_override=lambda n: f'__in_{n.name}[__e]')
+                body.append('    #pragma unroll')
+                body.append(f'    for (int __e = 0; __e < {V}; ++__e) {{')
+                if len(st.data_axes) == 1:
+                    body.append(f'      const int {st.data_axes[0][0]} = (int)(__v * {V} + __e); (void){st.data_axes[0][0]};')
+                body.append(f'      __out[__e] = ({oct_})({vem.expr(root)});')
+                body.append('    }')
+                body.append(f'    ((__vec_{st.output}*){st.output})[__v] = __out;')
+                body.append('  }')
+                body.append(f'  for (long long __i = __nvec * {V} + __tid; __i < __total; __i += __nthr) {{')
+                body += _decompose('__i', st.data_axes, '    ')
+                body.append(f'    {dst} = ({oct_})({em.expr(root)});')
+                body += ['  }', '}']
+                src.append('\n'.join(body))
+                variants['vec'] = sym
+                plan.vec, plan.vec_tensors = V, names
+
+    elif plan.kind == 'scatter':
+        sym = name
+        body = header(sym)
+        body.append('  for (long long __i = __tid; __i < __total; __i += __nthr) {')
+        body += _decompose('__i', st.data_axes, '    ')
+        val = f'({oct_})({em.expr(root)})'
+        store = {'set': f'{dst} = {val};', 'add': f'atomicAdd(&{dst}, {val});',
+                 'min': f'atomicMin(&{dst}, {val});', 'max': f'atomicMax(&{dst}, {val});'}[st.set_op]
+        body.append(f'    if ({cond}) {{ {store} }}' if cond else f'    {store}')
+        body += ['  }', '}']
+        src.append('\n'.join(body))
+        variants['scalar'] = sym
+
+    else:
+        act = HIP_TYPE[root.dtype]
+        ident = reduce_identity(st.reduce, root.dtype)
+        op = _REDUCE_OP[st.reduce] + '()'
+        red_total = ' * '.join(f'(long long)__ext_{ax}' for ax, _ in st.reduce_axes)
+        store = f'{dst} = ({oct_})__acc;'
+        store = f'if ({cond}) {{ {store} }}' if cond else store
+
+        def reduce_body(sym, out_var, out_step, lane, nlanes, finish):
+            b = header(sym)
+            b.append(f'  const long long __red = {red_total};')
+            if sym.endswith('_b'):
+                b.append(f'  __shared__ {act} __smem[4];')
+            b.append(f'  for (long long __o = {out_var}; __o < __total; __o += {out_step}) {{')
+            b += _decompose('__o', st.data_axes, '    ')
+            b.append(f'    {act} __acc = {ident};')
+            b.append(f'    for (long long __k = {lane}; __k < __red; __k += {nlanes}) {{')
+            b += [l.replace('__r', '__q') for l in _decompose('__k', st.reduce_axes, '      ')]
+            b.append(f'      __acc = {op}(__acc, ({act})({em.expr(root)}));')
+            b.append('    }')
+            b += finish
+            b += ['  }', '}']
+            return '\n'.join(b)
+
+        src.append(reduce_body(name + '_t', '__tid', '__nthr', '0', '1', [f'    {store}']))
+        src.append(reduce_body(name + '_w', '(__tid >> 6)', '(__nthr >> 6)', '(threadIdx.x & 63)', '64',
+                               [f'    __acc = art_wave_reduce(__acc, {op});', f'    if ((threadIdx.x & 63) == 0) {{ {store} }}']))
+        src.append(reduce_body(name + '_b', '(long long)blockIdx.x', '(long long)gridDim.x', 'threadIdx.x', str(BLOCK),
+                               [f'    __acc = art_block_reduce(__acc, {op}, __smem);', f'    if (threadIdx.x == 0) {{ {store} }}']))
+        variants.update({'thread': name + '_t', 'wave': name + '_w', 'block': name + '_b'})
+        plan.reduce_contiguous = _reduce_axis_contiguous(st, tensors)
+
+    return '\n\n'.join(src), plan
+
+
+def _reduce_axis_contiguous(st, tensors) -> Optional[bool]:
+    """Looks at the last index of every load: votes, weighted by rank, whether a
+    reduce axis or a data axis walks memory contiguously."""
+    raxes = {a for a, _ in st.reduce_axes}
+    daxes = {a for a, _ in st.data_axes}
+    score = 0
+    for n in walk(st.root):
+        if n.kind == 'load' and n.args:
+            last = n.args[-1]
+            w = len(n.args)
+            if last.kind == 'axis' and last.name in raxes:
+                score += w
+            elif last.kind == 'axis' and last.name in daxes:
+                score -= w
+    if score == 0:
+        return None
+    return score > 0
+
+
+def lower_graph(graph, prefix: str = 'autort') -> Tuple[str, List[KernelPlan]]:
+    """Fused graph -> (HIP source text with container-format headers, plans).
+
+    The text carries the same ``// GLOBALS`` / ``// LOCAL`` headers as the
+    reference's kernel files (antares/antares_compiler.py:183-232) so it can be
+    read with the same eyes; the runtime itself works from the plans.
+    """
+    def disp(n):
+        t = graph.tensors[n]
+        return f'{n}:{t.dtype}{list(t.shape)}'.replace("'", '')
+    head = '// GLOBALS: ' + ', '.join(disp(n) for n in graph.abi_inputs) + ' -> ' + \
+        ', '.join(disp(n) for n in graph.abi_outputs) + '\n// BACKEND: c-mi355x (gfx950)\n'
+    if graph.dims:
+        head += '// VAMAP: ' + ','.join(f'{d}:{v if v is not None else "?"}' for d, v in sorted(graph.dims.items())) + '\n'
+    head += '// COMPUTE_V1: - einstein_v2(' + repr(' '.join(graph.source.split())) + ')\n'
+    parts, plans = [head + PRELUDE], []
+    for i, st in enumerate(graph.statements):
+        code, plan = lower_statement(st, graph, f'{prefix}_k{i}')
+        ins = ', '.join(disp(n) for n in plan.args[:-1])
+        parts.append(f'// LOCAL: {plan.name} -- {ins} -> {disp(plan.output)}\n\n{code}\n')
+        plans.append(plan)
+    sep = '\n// ---------------------------------------------------------------------------\n'
+    return sep.join(parts), plans

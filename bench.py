@@ -1,0 +1,181 @@
+#!/usr/bin/env python
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+Headline workload (BASELINE.json: "int4-GEMV HBM GB/s"): the int4 group-128
+GEMV y[1,11008] = x[1,4096] @ dequant(W), through ``autort.export`` and the
+C-ABI library.  One step is one pass over LAYERS distinct weight sets
+(LAYERS * 22.5 MB is larger than every cache of the chip, so each launch
+streams its weights from HBM, as a decode step does); all inputs are resident
+in HBM before the timed region.  The pass is recorded once in a HIP graph so
+that the timed region contains kernels, not Python.
+
+Prints ONE JSON line.  ``roofline`` is for the GEMV kernel: algorithmic bytes
+per launch / mean time per launch inside the timed region (HIP events on the
+launch stream) against the 8 TB/s HBM peak.  ``cpu_baseline`` is the CPU
+oracle's loop-nest restatement of the reference's c-mcpu backend for the same
+program, timed on this host on a bounded sample.  ``extra`` carries the other
+configurations (sigmoid, partition, other GEMV shapes) measured the same way.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+LAYERS = 32
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--no-extra', action='store_true', help='headline workload only')
+    ap.add_argument('--seed', type=int, default=0)
+    return ap.parse_args()
+
+
+def time_graph(torch, capi, fn, steps, warmup):
+    """Records ``fn`` (which enqueues kernels on the current stream) in a HIP
+    graph, replays it warmup + steps times, returns mean seconds per replay of
+    the timed ones, measured with events on the replay stream."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        fn()                                   # first call: compiles / loads modules, outside capture
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            fn()
+        for _ in range(warmup):
+            graph.replay()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        start, stop = capi.Event(), capi.Event()
+        start.record(stream.cuda_stream)
+        for _ in range(steps):
+            graph.replay()
+        stop.record(stream.cuda_stream)
+        ms = start.elapsed_ms(stop)
+        torch.cuda.synchronize()
+    return ms * 1e-3 / steps
+
+
+def bench_gemv(torch, autort, capi, workloads, K, N, M, steps, warmup, seed, layers=LAYERS):
+    from antares_amd.autort import patterns
+    dev = autort.device()
+    op = autort.export(ir=patterns.W4A16_IR, inputs=patterns.W4A16_INPUTS, name='gemv_w4a16')
+    p = workloads.w4_problem(seed, M, K, N)
+    # distinct weight sets: same distribution, different bits (rolled copies), so no launch finds its data cached
+    sets = []
+    for l in range(layers):
+        sets.append((torch.roll(p['qweight'], l, 0).to(dev), torch.roll(p['scales'], l, 0).to(dev), torch.roll(p['qzeros'], l, 0).to(dev)))
+    x = p['x'].to(dev)
+    ys = [torch.empty(M, N, dtype=torch.float16, device=dev) for _ in range(layers)]
+
+    def one_pass():
+        for (qw, sc, qz), y in zip(sets, ys):
+            op(x, qw, sc, qz, out=y)
+    sec = time_graph(torch, capi, one_pass, steps, warmup)
+    per_launch = sec / layers
+    by = workloads.w4_bytes(M, K, N)
+    return {'workload': f'int4 g128 GEMV M={M} K={K} N={N}', 'bytes_per_launch': by, 'launches_per_step': layers,
+            'sec_per_step': sec, 'us_per_launch': per_launch * 1e6, 'gbps': by / per_launch / 1e9}
+
+
+def bench_sigmoid(torch, autort, capi, workloads, steps, warmup, seed, n=4_096_000, copies=16):
+    dev = autort.device()
+    op = autort.export(ir='sigmoid_f32[N] = 1 - 1 / (1 + data[N].call(strs.exp))', inputs=['data=float32[N:4096000]'], config='tune:5')
+    base = workloads.sigmoid_input(seed, n)
+    xs = [torch.roll(base, i).to(dev) for i in range(copies)]
+    outs = [torch.empty_like(x) for x in xs]
+
+    def one_pass():
+        for x, o in zip(xs, outs):
+            op(x, out=o)
+    sec = time_graph(torch, capi, one_pass, steps, warmup) / copies
+    return {'workload': f'sigmoid f32 N={n}', 'bytes_per_launch': 8 * n, 'us_per_launch': sec * 1e6, 'gbps': 8 * n / sec / 1e9,
+            'roofline_frac': 8 * n / sec / 1e9 / HBM_PEAK_GBPS}
+
+
+def bench_partition(torch, autort, capi, workloads, steps, warmup, seed, n=16_777_216, copies=4):
+    dev = autort.device()
+    base = workloads.partition_input(seed, n)
+    xs = [torch.roll(base, i).to(dev) for i in range(copies)]
+    outs = [torch.empty_like(x) for x in xs]
+
+    def one_pass():
+        for x, o in zip(xs, outs):
+            autort.ops.partition_even_first_i32(x, o)
+    sec = time_graph(torch, capi, one_pass, max(5, steps // 5), warmup) / copies
+    return {'workload': f'stable even-first partition int32 N={n}', 'bytes_per_launch': 8 * n, 'us_per_call': sec * 1e6,
+            'gbps': 8 * n / sec / 1e9, 'roofline_frac': 8 * n / sec / 1e9 / HBM_PEAK_GBPS, 'melem_per_s': n / sec / 1e6}
+
+
+def cpu_baseline_gemv(workloads, K, N, M, seed, budget_s=15.0):
+    """The CPU oracle (loop nests of the reference's CPU backend, same compiler
+    flags, rank-striding thread pool) on the headline program."""
+    from antares_amd.autort import patterns
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    p = workloads.w4_problem(seed, M, K, N)
+    mod = CpuModule(parse_program(patterns.W4A16_IR, patterns.W4A16_INPUTS), nranks=256)
+    t = mod.time(budget_s=budget_s, x=p['x'].numpy(), qweight=p['qweight'].numpy().view('int8'),
+                 scales=p['scales'].numpy(), qzeros=p['qzeros'].numpy().view('int8'))
+    by = workloads.w4_bytes(M, K, N)
+    return {'value': by / t['seconds'] / 1e9, 'unit': 'GB/s', 'cores': t['threads'], 'kind': 'port',
+            'sample': f'{t["runs"]} timed run(s) of the same GEMV (M={M} K={K} N={N}) after 1 warm-up + 1 probe, '
+                      f'{t["seconds"] * 1e3:.1f} ms per run'}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1', file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import autort
+    from antares_amd import workloads
+    from antares_amd.runtime import capi
+    capi.init(0)
+    K, N, M = 4096, 11008, 1
+    head = bench_gemv(torch, autort, capi, workloads, K, N, M, args.steps, args.warmup, args.seed)
+    result = {
+        'metric': 'int4_gemv_hbm_gbps', 'value': round(head['gbps'], 2), 'unit': 'GB/s', 'n_gpus': 1,
+        'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(head['sec_per_step'] * 1e3, 5),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'u4*f16->f32', 'data': 'synthetic',
+        'config': {'workload': head['workload'], 'launches_per_step': head['launches_per_step'], 'group': 128,
+                   'weights': 'uint8 [K/2,N] two nibbles along K; fp16 scale + 4-bit zero per group',
+                   'distinct_weight_sets': head['launches_per_step'], 'timed_through': 'HIP graph replay'},
+        'roofline': {'bound': 'hbm', 'achieved': round(head['gbps'], 2), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+                     'frac': round(head['gbps'] / HBM_PEAK_GBPS, 4), 'traffic': None,
+                     'kernel': 'gemv_w4a16_kernel', 'bytes_per_launch': head['bytes_per_launch'],
+                     'us_per_launch': round(head['us_per_launch'], 3)},
+    }
+    if not args.no_extra:
+        extra = []
+        for (k, n) in [(4096, 4096), (11008, 4096), (4096, 32000)]:
+            r = bench_gemv(torch, autort, capi, workloads, k, n, 1, max(10, args.steps // 2), args.warmup, args.seed,
+                           layers=32 if n < 32000 else 8)
+            extra.append({'workload': r['workload'], 'us_per_launch': round(r['us_per_launch'], 3), 'gbps': round(r['gbps'], 1),
+                          'roofline_frac': round(r['gbps'] / HBM_PEAK_GBPS, 4)})
+        for fn in (bench_sigmoid, bench_partition):
+            r = fn(torch, autort, capi, workloads, args.steps, args.warmup, args.seed)
+            extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
+        result['extra'] = extra
+    if not args.no_cpu:
+        result['cpu_baseline'] = cpu_baseline_gemv(workloads, K, N, M, args.seed)
+        result['cpu_baseline']['value'] = round(result['cpu_baseline']['value'], 4)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == '__main__':
+    main()

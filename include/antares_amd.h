@@ -1,0 +1,123 @@
+/*
+ * antares_amd.h — flat C ABI of libantares_amd.so, the MI355X (gfx950) runtime
+ * and kernel library behind the AutoRT / Antares operator surface.
+ *
+ * Every function returns 0 on success and non-zero on failure; the message of
+ * the last failure on the calling thread is available from art_last_error().
+ * Nothing here calls exit().  All pointers named *_dev are raw device
+ * addresses (e.g. torch `tensor.data_ptr()`); `stream` is a hipStream_t passed
+ * as void* (NULL = the default stream).  The caller owns all tensor memory;
+ * the library owns loaded modules for the life of the process and one internal
+ * workspace per device that is allocated by art_init().
+ *
+ * The first group replaces the reference's header-only `namespace ab` device
+ * runtime and its ExecutionModule; the second group are typed entry points for
+ * the hand-written kernels that replace generated code on the hot path.
+ */
+#ifndef ANTARES_AMD_H_
+#define ANTARES_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---------------------------------------------------------------- runtime */
+
+typedef struct art_module art_module;   /* a loaded code object            */
+typedef struct art_func art_func;       /* one kernel inside a module      */
+
+typedef struct art_props {
+  char name[256];
+  char arch[64];              /* e.g. "gfx950" */
+  int compute_units;
+  int wavefront_size;
+  int max_threads_per_block;
+  int lds_bytes_per_block;
+  int clock_khz;
+  int memory_clock_khz;
+  int memory_bus_width_bits;
+  int l2_bytes;
+  size_t total_memory_bytes;
+} art_props;
+
+/* Bind the calling process to `device` and allocate the library workspace.
+ * Idempotent.  Replaces ab::init (backends/c-rocm/include/backend.hpp:51). */
+int art_init(int device);
+
+/* Message of the last error on this thread ("" if none). */
+const char* art_last_error(void);
+
+/* Device properties; replaces the device-property probe used to fill
+ * hardware configs (engine/cuda_properties.cc:35-52). */
+int art_device_props(art_props* out);
+
+/* Compile HIP source text for `arch` (NULL = "gfx950") into a code object.
+ * Works without a GPU.  `*blob` is owned by the library until art_blob_free.
+ * Replaces ab::moduleCompile (backends/c-rocm/include/backend.hpp:116-158),
+ * which forks `hipcc --genco`; this one compiles in-process. */
+int art_module_compile(const char* hip_source, const char* arch, void** blob, size_t* size);
+void art_blob_free(void* blob);
+/* Text of the compiler log of the last art_module_compile on this thread. */
+const char* art_compile_log(void);
+
+/* Load a code object; replaces ab::moduleLoad (backend.hpp:161-170). */
+int art_module_load(const void* image, size_t size, art_module** out);
+int art_module_unload(art_module* module);
+
+/* Look a kernel up by name; replaces ab::moduleGetFunction (backend.hpp:172-197). */
+int art_get_function(art_module* module, const char* name, art_func** out);
+
+/* Launch with `nargs` kernel arguments, each held in one 64-bit slot of
+ * `args` (device pointers as they are, integers widened) — the slot convention
+ * of the reference's launch path (graph_evaluator/execute_module.hpp:340-352).
+ * Replaces ab::launchKernel (backend.hpp:199-219). */
+int art_launch(art_func* func, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
+               unsigned lds_bytes, void* stream, const uint64_t* args, int nargs);
+
+/* Timing and synchronisation; replace ab::recordTime / convertToElapsedTime /
+ * synchronize (backend.hpp:233-252). */
+int art_event_create(void** event);
+int art_event_record(void* event, void* stream);
+int art_event_elapsed_ms(void* start, void* stop, float* ms);   /* synchronises on `stop` */
+int art_event_destroy(void* event);
+int art_stream_synchronize(void* stream);
+
+/* Plain device copy kernel (dst, src: 16-byte aligned, bytes % 16 == 0); used
+ * as the calibration workload for memory-traffic counters. */
+int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+
+/* ---------------------------------------------------- hand-written kernels */
+
+/* Weight-only int4 GEMV / skinny GEMM, group size 128 along K:
+ *     y[m,n] = sum_k x[m,k] * (q[k,n] - z[k/128,n]) * s[k/128,n]
+ * x: fp16 [M,K]; qweight: uint8 [K/2,N], low nibble = even k; scales: fp16
+ * [K/128,N]; qzeros: uint8 [K/128,N/2], low nibble = even n; y: fp16 [M,N].
+ * fp32 accumulation.  M <= 8 here (decode); K % 128 == 0, N % 16 == 0.
+ * Replaces the kernel the reference generates from the dequant+GEMV program
+ * of samples/05_llama2_7b_int4.py:135-144 (antares/default_codegen.py:13). */
+int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                   void* y_dev, int M, int K, int N, void* stream);
+
+/* The reference's own weight format (samples/05_llama2_7b_int4.py:135-139):
+ * qweight int32 [K/8,N], eight nibbles per word along K (least significant
+ * first), zero point fixed at 8, scales fp32 or fp16 [K/128,N], x and y fp32
+ * or fp16 (x_f16 / scales_f16 select).  M = 1. */
+int art_gemv_gptq(const void* x_dev, const void* qweight_dev, const void* scales_dev, void* y_dev,
+                  int K, int N, int x_f16, int scales_f16, void* stream);
+
+/* Stable even-first partition of int32 values: all even values in input order,
+ * then all odd values in input order.  One pass (decoupled look-back scan).
+ * Replaces the classify -> cumsum -> bucket pipeline of
+ * samples/01_sort_even_first.py:9-27. */
+int art_partition_even_first_i32(const void* in_dev, void* out_dev, long long n, void* stream);
+
+/* Bytes of library workspace art_partition_even_first_i32 / split-K kernels may use. */
+size_t art_workspace_bytes(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* ANTARES_AMD_H_ */

@@ -39,9 +39,9 @@ PRELUDE = r'''
 #include <algorithm>
 ''' + _HALF_H + r'''
 #define rsqrt(x)  (1.0f / sqrt(x))
-template <class T> static inline T bitwise_and(T a, T b) { return (T)(a & b); }
-template <class T> static inline T bitwise_or(T a, T b) { return (T)(a | b); }
-template <class T> static inline T bitwise_xor(T a, T b) { return (T)(a ^ b); }
+template <class T, class U> static inline T bitwise_and(T a, U b) { return (T)(a & (T)b); }
+template <class T, class U> static inline T bitwise_or(T a, U b) { return (T)(a | (T)b); }
+template <class T, class U> static inline T bitwise_xor(T a, U b) { return (T)(a ^ (T)b); }
 static inline float normcdf(float x) { return 0.5f * erfcf(-x * 0.70710678118654752440f); }
 static inline double normcdf(double x) { return 0.5 * erfc(-x * 0.70710678118654752440); }
 static inline half fp16_exp(half x) { return half(expf((float)x)); }

@@ -1,0 +1,84 @@
+/* TEST INFRASTRUCTURE ONLY — CPU oracle.  Only tests/, __graft_entry__.smoke()
+ * and the cpu_baseline leg of bench.py load this library; the GPU path never
+ * does.
+ *
+ * Plain-C restatements of the hot operators, written directly from the
+ * reference's sample programs as the loop nests AntaresIR.md:6-67 prescribes.
+ * They are independent of this repository's IR parser, so they also check the
+ * generic loop-nest emitter (cpu_emit.py) on the same programs.
+ *
+ * Pinned by (see tests/test_oracle.py): README known answers for sigmoid and
+ * the even-first sort; one-hot / all-equal special cases and a float64 numpy
+ * recomputation for the int4 products; the closed forms stated at each
+ * function for rmsnorm / rotary / attention.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "ref_half.h"
+
+/* sigmoid_f32[N] = 1 - 1 / (1 + exp(data[N]))          (README.md:66) */
+void ref_sigmoid_f32(const float* data, float* out, long long n) {
+  for (long long i = 0; i < n; ++i) out[i] = 1.0f - 1.0f / (1.0f + expf(data[i]));
+}
+
+/* samples/01_sort_even_first.py:9-27, step by step:
+ *   space[data[n] % 2, n] = 1                                  (classify, space zeroed)
+ *   ids = cumsum(space.flat, int32) * space.flat               (host glue at :24)
+ *   output[ids[n] - 1] = val[n % M]   when ids[n] > 0          (bucket, n over 2M) */
+int ref_sort_even_first_i32(const int32_t* data, int32_t* output, long long m) {
+  int32_t* space = (int32_t*)calloc((size_t)(2 * m), sizeof(int32_t));
+  int32_t* ids = (int32_t*)malloc((size_t)(2 * m) * sizeof(int32_t));
+  if (!space || !ids) { free(space); free(ids); return 1; }
+  for (long long n = 0; n < m; ++n) space[(long long)(data[n] % 2) * m + n] = 1;
+  int32_t run = 0;
+  for (long long n = 0; n < 2 * m; ++n) { run += space[n]; ids[n] = run * space[n]; }
+  for (long long n = 0; n < m; ++n) output[n] = 0;
+  for (long long n = 0; n < 2 * m; ++n)
+    if (ids[n] > 0) output[ids[n] - 1] = data[n % m];
+  free(space); free(ids);
+  return 0;
+}
+
+/* int4 g128 GEMV / GEMM with per-group zero points (the packed format of the
+ * benchmark configuration):
+ *   q[k,n]  = (qweight[k/2, n] >> (k%2*4)) & 15          uint8 [K/2,N], low nibble = even k
+ *   z[g,n]  = (qzeros[g, n/2] >> (n%2*4)) & 15           uint8 [K/128,N/2], low nibble = even n
+ *   w[k,n]  = fp16( scales[k/128,n] * fp16(q - z) )      the dequantised weight is a half, as in
+ *                                                        samples/05_llama2_7b_int4.py:138 (.to(x.dtype))
+ *   y[m,n]  = fp16( sum_k float(x[m,k]) * float(w[k,n]) )   fp32 accumulate in k order */
+void ref_gemm_w4a16(const uint16_t* x, const uint8_t* qweight, const uint16_t* scales, const uint8_t* qzeros,
+                    uint16_t* y, int M, int K, int N) {
+  for (int m = 0; m < M; ++m)
+    for (int n = 0; n < N; ++n) {
+      float acc = 0.0f;
+      for (int k = 0; k < K; ++k) {
+        const int q = (qweight[(size_t)(k / 2) * N + n] >> (k % 2 * 4)) & 15;
+        const int z = (qzeros[(size_t)(k / 128) * (N / 2) + n / 2] >> (n % 2 * 4)) & 15;
+        const float s = ref_h2f(scales[(size_t)(k / 128) * N + n]);
+        const float w = ref_h2f(ref_f2h(s * ref_h2f(ref_f2h((float)(q - z)))));
+        acc += ref_h2f(x[(size_t)m * K + k]) * w;
+      }
+      y[(size_t)m * N + n] = ref_f2h(acc);
+    }
+}
+
+/* The sample's own program (samples/05_llama2_7b_int4.py:135-139), fp32 x:
+ *   input1[s,n] = float((qweight[s/8, n] >> (s%8*4)) & 15)
+ *   w[s,n]      = float(scales[s/128, n]) * (input1[s,n] - 8)
+ *   y[n]       += x[s] * w[s,n]
+ * scales_f16 selects half scales (promoted to float before the multiply). */
+void ref_gemv_gptq_f32(const float* x, const int32_t* qweight, const void* scales, int scales_f16, float* y, int K, int N) {
+  for (int n = 0; n < N; ++n) {
+    float acc = 0.0f;
+    for (int s = 0; s < K; ++s) {
+      const float q = (float)((qweight[(size_t)(s / 8) * N + n] >> (s % 8 * 4)) & 15);
+      const float sc = scales_f16 ? ref_h2f(((const uint16_t*)scales)[(size_t)(s / 128) * N + n])
+                                  : ((const float*)scales)[(size_t)(s / 128) * N + n];
+      acc += x[s] * (sc * (q - 8.0f));
+    }
+    y[n] = acc;
+  }
+}

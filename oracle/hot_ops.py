@@ -1,0 +1,68 @@
+"""TEST INFRASTRUCTURE ONLY — numpy-facing wrappers of libref_hotops.so (the
+plain-C restatements in hot_ops.c).  Only tests/, __graft_entry__.smoke() and
+bench.py's cpu_baseline leg may import this."""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        path = os.path.join(_HERE, 'libref_hotops.so')
+        if not os.path.exists(path):
+            subprocess.check_call(['make', '-s', '-C', _HERE, 'libref_hotops.so'])
+        _lib = ctypes.CDLL(path)
+    return _lib
+
+
+def _p(a: np.ndarray):
+    assert a.flags['C_CONTIGUOUS']
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def sigmoid_f32(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().ref_sigmoid_f32(_p(x), _p(out), ctypes.c_longlong(x.size))
+    return out
+
+
+def sort_even_first_i32(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.int32)
+    out = np.empty_like(x)
+    rc = lib().ref_sort_even_first_i32(_p(x), _p(out), ctypes.c_longlong(x.size))
+    assert rc == 0
+    return out
+
+
+def gemm_w4a16(x, qweight, scales, qzeros) -> np.ndarray:
+    """x fp16 [M,K], qweight uint8 [K/2,N], scales fp16 [K/128,N], qzeros uint8 [K/128,N/2] -> fp16 [M,N]."""
+    x = np.ascontiguousarray(x, dtype=np.float16)
+    qweight = np.ascontiguousarray(qweight).view(np.uint8)
+    scales = np.ascontiguousarray(scales, dtype=np.float16)
+    qzeros = np.ascontiguousarray(qzeros).view(np.uint8)
+    M, K = x.shape
+    N = qweight.shape[1]
+    assert qweight.shape[0] * 2 == K and scales.shape == (K // 128, N) and qzeros.shape == (K // 128, N // 2)
+    y = np.empty((M, N), dtype=np.float16)
+    lib().ref_gemm_w4a16(_p(x), _p(qweight), _p(scales), _p(qzeros), _p(y), M, K, N)
+    return y
+
+
+def gemv_gptq_f32(x, qweight, scales) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    qweight = np.ascontiguousarray(qweight, dtype=np.int32)
+    scales = np.ascontiguousarray(scales)
+    assert scales.dtype in (np.float32, np.float16)
+    K, N = x.shape[0], qweight.shape[1]
+    y = np.empty(N, dtype=np.float32)
+    lib().ref_gemv_gptq_f32(_p(x), _p(qweight), _p(scales), int(scales.dtype == np.float16), _p(y), K, N)
+    return y

@@ -1,0 +1,214 @@
+"""GPU parity tests: every operator is called through the autort surface (which
+goes through the C-ABI library) and compared with the CPU oracle on the same
+seeded inputs.  Integer results must be bit-exact; fp32 within 1e-5, fp16
+within rtol 1e-2 / atol 1e-2."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from antares_amd import workloads
+
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures('oracle_built')]
+
+FP32_TOL = dict(rtol=1e-5, atol=1e-5)
+FP16_TOL = dict(rtol=1e-2, atol=1e-2)
+
+
+@pytest.fixture(scope='module')
+def autort():
+    import autort as mod
+    assert torch.cuda.is_available(), 'these tests need the GPU'
+    return mod
+
+
+def note(msg):
+    print(f'[case] {msg}', flush=True)
+    sys.stdout.flush()
+
+
+SIGMOID_IR = 'sigmoid_f32[N] = 1 - 1 / (1 + data[N].call(strs.exp))'
+
+
+def test_sigmoid_readme_example(autort):
+    note('sigmoid N=10')
+    f = autort.export(ir=SIGMOID_IR, inputs=['data=float32[N:4096000]'], config='tune:5')
+    data = torch.arange(0, 10, dtype=torch.float32, device=autort.device())
+    want = [0.5000, 0.7311, 0.8808, 0.9526, 0.9820, 0.9933, 0.9975, 0.9991, 0.9997, 0.9999]
+    assert np.allclose(f(data).cpu().numpy(), want, atol=5e-5)
+    assert np.allclose(autort.ops.sigmoid_f32(data).cpu().numpy(), want, atol=5e-5)
+
+
+@pytest.mark.parametrize('n', [0, 1, 3, 4, 5, 1023, 4_096_000, 4_096_003])
+def test_sigmoid_matches_oracle(autort, n):
+    from oracle import hot_ops
+    note(f'sigmoid N={n}')
+    f = autort.export(ir=SIGMOID_IR, inputs=['data=float32[N:4096000]'])
+    x = workloads.sigmoid_input(7, n)
+    got = f(x.to(autort.device())).cpu().numpy()
+    assert got.shape == (n,)
+    assert np.allclose(got, hot_ops.sigmoid_f32(x.numpy()), **FP32_TOL)
+
+
+def test_sigmoid_unaligned_view(autort):
+    from oracle import hot_ops
+    note('sigmoid on a view that is not 16-byte aligned')
+    f = autort.export(ir=SIGMOID_IR, inputs=['data=float32[N:4096000]'])
+    x = workloads.sigmoid_input(8, 10_001)
+    xd = x.to(autort.device())
+    out = torch.zeros(10_001, dtype=torch.float32, device=autort.device())
+    f(xd[1:], out=out[1:])
+    assert np.allclose(out[1:].cpu().numpy(), hot_ops.sigmoid_f32(x.numpy()[1:]), **FP32_TOL)
+    assert float(out[0]) == 0.0
+
+
+def run_sort_sample(autort, x: torch.Tensor) -> torch.Tensor:
+    """samples/01_sort_even_first.py:16-27 verbatim in structure."""
+    autort.export(ir='space[data[N] % 2, N] = 1', inputs=['data=int32[N]', 'space=int32[2, N]'],
+                  config='~N~:[1,256,1]', name='my_classify_i32')
+    autort.export(ir='output[ids[N] - 1] = (val[N % val.size(0)]).when(ids[N] > 0)',
+                  inputs=['ids=int32[N]', 'val=int32[M]', 'output=int32[M]'], config='~N~:[1,256,1]', name='my_bucket_i32')
+    y = torch.zeros([2, x.size(0)], dtype=torch.int32, device=x.device)
+    autort.ops.my_classify_i32(x, y)
+    ids = torch.cumsum(y.view(-1), 0, dtype=y.dtype) * y.view(-1)
+    output = torch.zeros_like(x)
+    autort.ops.my_bucket_i32(ids, x, output)
+    return output
+
+
+def test_sort_sample_known_answer(autort):
+    note('sort sample, README input')
+    x = torch.tensor([101, 102, 208, 99, 1, 127, 62, 8, 336, 336], dtype=torch.int32, device=autort.device())
+    assert run_sort_sample(autort, x).cpu().tolist() == [102, 208, 62, 8, 336, 336, 101, 99, 1, 127]
+    assert autort.ops.partition_even_first_i32(x).cpu().tolist() == [102, 208, 62, 8, 336, 336, 101, 99, 1, 127]
+
+
+@pytest.mark.parametrize('n', [1, 2, 63, 64, 65, 4095, 4096, 4097, 8191, 8192, 100_003, 1_048_576])
+def test_partition_bit_exact(autort, n):
+    from oracle import hot_ops
+    note(f'partition N={n}')
+    x = workloads.partition_input(100 + n, n)
+    want = hot_ops.sort_even_first_i32(x.numpy())
+    xd = x.to(autort.device())
+    assert np.array_equal(autort.ops.partition_even_first_i32(xd).cpu().numpy(), want)
+    assert np.array_equal(run_sort_sample(autort, xd).cpu().numpy(), want)
+
+
+def test_partition_empty_and_degenerate(autort):
+    note('partition edge cases')
+    dev = autort.device()
+    assert autort.ops.partition_even_first_i32(torch.empty(0, dtype=torch.int32, device=dev)).numel() == 0
+    ev = torch.arange(0, 20000, 2, dtype=torch.int32, device=dev)
+    assert torch.equal(autort.ops.partition_even_first_i32(ev), ev)
+    assert torch.equal(autort.ops.partition_even_first_i32(ev + 1), ev + 1)
+
+
+def test_partition_full_size_properties(autort):
+    note('partition N=16777216 (size-independent properties)')
+    x = workloads.partition_input(2, 16_777_216).to(autort.device())
+    out = autort.ops.partition_even_first_i32(x)
+    want = torch.cat([x[x % 2 == 0], x[x % 2 == 1]])
+    assert torch.equal(out, want)
+    # idempotent
+    assert torch.equal(autort.ops.partition_even_first_i32(out), out)
+    # two calls in a row give the same bits (ticket words are restored)
+    assert torch.equal(autort.ops.partition_even_first_i32(x), out)
+
+
+# ------------------------------------------------------------------ int4 GEMV
+def w4_op(autort):
+    from antares_amd.autort import patterns
+    return autort.export(ir=patterns.W4A16_IR, inputs=patterns.W4A16_INPUTS, name='gemv_w4a16')
+
+
+@pytest.mark.parametrize('M,K,N', [(1, 128, 16), (1, 256, 64), (2, 384, 144), (3, 1024, 1040), (4, 4096, 512), (8, 512, 256),
+                                   (1, 4096, 4096), (1, 4096, 11008), (1, 11008, 4096), (1, 4096, 32000)])
+def test_w4a16_gemv_matches_oracle(autort, M, K, N):
+    from oracle import hot_ops
+    note(f'w4a16 M={M} K={K} N={N}')
+    p = workloads.w4_problem(K + N + M, M, K, N)
+    f = w4_op(autort)
+    assert f.fast_path is not None
+    dev = autort.device()
+    y = f(p['x'].to(dev), p['qweight'].to(dev), p['scales'].to(dev), p['qzeros'].to(dev))
+    torch.cuda.synchronize()
+    want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy())
+    assert np.allclose(y.cpu().numpy().astype(np.float32), want.astype(np.float32), **FP16_TOL)
+    # second call must see clean ticket words
+    y2 = f(p['x'].to(dev), p['qweight'].to(dev), p['scales'].to(dev), p['qzeros'].to(dev))
+    assert torch.equal(y, y2)
+
+
+def test_w4a16_generic_lowering_agrees(autort):
+    """The same program through the generic reduce lowering (no hand kernel)."""
+    from oracle import hot_ops
+    note('w4a16 through the generic lowering')
+    p = workloads.w4_problem(9, 2, 256, 64)
+    f = w4_op(autort)
+    dev = autort.device()
+    bound = {'x': p['x'].to(dev), 'qweight': p['qweight'].to(dev), 'scales': p['scales'].to(dev), 'qzeros': p['qzeros'].to(dev)}
+    saved, f.fast_path = f.fast_path, None
+    try:
+        y = f(bound['x'], bound['qweight'], bound['scales'], bound['qzeros'])
+    finally:
+        f.fast_path = saved
+    want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy())
+    assert np.allclose(y.cpu().numpy().astype(np.float32), want.astype(np.float32), **FP16_TOL)
+
+
+@pytest.mark.parametrize('K,N,sdt', [(4096, 12288, 'float32'), (4096, 4096, 'float16'), (11008, 4096, 'float32'), (256, 36, 'float32')])
+def test_gptq_gemv_sample_program(autort, K, N, sdt):
+    from antares_amd.autort import patterns
+    from oracle import hot_ops
+    note(f'gptq gemv K={K} N={N} scales={sdt}')
+    g = torch.Generator().manual_seed(K + N)
+    q = torch.randint(0, 16, (K, N), generator=g)
+    s = (torch.rand(K // 128, N, generator=g) * 0.019 + 0.001).to(torch.float32 if sdt == 'float32' else torch.float16)
+    x = torch.randn(K, generator=g)
+    qw = workloads.pack_gptq(q)
+    f = autort.export(ir=patterns.GPTQ_GEMV_IR, inputs=patterns._gptq_inputs('float32', sdt), config='~N~:[256,8,32],~S~:[64,8]')
+    dev = autort.device()
+    out = torch.empty(N, dtype=torch.float32, device=dev)
+    y = f(x.to(dev), qw.to(dev), s.to(dev), out=out)
+    assert y.data_ptr() == out.data_ptr()
+    want = hot_ops.gemv_gptq_f32(x.numpy(), qw.numpy(), s.numpy())
+    exact = x.numpy().astype(np.float64) @ ((q.numpy().astype(np.float64) - 8) * np.repeat(s.numpy().astype(np.float64), 128, axis=0))
+    got = y.cpu().numpy()
+    # fp32 sums of K terms: the oracle's own distance from the exact value sets the scale of the tolerance
+    tol = max(1e-5, 4 * float(np.abs(want - exact).max()))
+    assert np.abs(got - exact).max() <= tol, (np.abs(got - exact).max(), tol)
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+# ------------------------------------------------------------------ generic lowering
+def test_generic_reduce_variants(autort):
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note('generic reduce: softmax program')
+    ir = ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
+          'output0[N, C] = (input0[N, C] - temp0[N]).call(`exp`) / temp1[N]')
+    dev = autort.device()
+    for shape in [(32, 1024), (3, 5000), (300, 7)]:
+        inp = {'input0': {'dtype': 'float32', 'shape': list(shape)}}
+        x = torch.randn(*shape, generator=torch.Generator().manual_seed(1))
+        f = autort.export(ir=ir, inputs=['input0=float32[%d, %d]' % shape])
+        got = f(x.to(dev)).cpu().numpy()
+        want = CpuModule(parse_program(ir, inp))(input0=x.numpy())['output0']
+        assert np.allclose(got, want, **FP32_TOL)
+
+
+def test_generic_matmul_and_scatter(autort):
+    note('generic matmul + scatter-add')
+    dev = autort.device()
+    g = torch.Generator().manual_seed(3)
+    a, b = torch.randn(70, 50, generator=g), torch.randn(50, 33, generator=g)
+    f = autort.export(ir='output0[N, M] +=! input0[N, K] * input1[K, M]', inputs=['input0=float32[N:70, K:50]', 'input1=float32[K:50, M:33]'])
+    assert np.allclose(f(a.to(dev), b.to(dev)).cpu().numpy(), (a.double() @ b.double()).numpy(), rtol=1e-4, atol=1e-4)
+    idx = torch.randint(0, 16, (1000,), generator=g, dtype=torch.int64).to(torch.int32)
+    upd = torch.randint(0, 100, (1000,), generator=g, dtype=torch.int64).to(torch.int32)
+    hist = torch.zeros(16, dtype=torch.int32, device=dev)
+    h = autort.export(ir='hist[idx[B]] +=. upd[B]', inputs=['hist=int32[H]', 'idx=int32[B]', 'upd=int32[B]'], name='scatter_add_i32')
+    h(hist, idx.to(dev), upd.to(dev))
+    want = torch.zeros(16, dtype=torch.int64).index_add_(0, idx.long(), upd.long())
+    assert hist.cpu().long().tolist() == want.tolist()

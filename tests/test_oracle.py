@@ -1,0 +1,189 @@
+"""Pins the CPU oracle: README known answers, closed forms, special cases that
+a dropped term / wrong nibble order / transposed operand would break, and the
+agreement of its two independent halves (plain-C hot_ops vs the loop nests
+emitted from the IR)."""
+import numpy as np
+import pytest
+import torch
+
+from antares_amd import workloads
+from antares_amd.autort import patterns
+from antares_amd.ir import parse_program
+
+pytestmark = pytest.mark.usefixtures('oracle_built')
+
+README_SIGMOID = [0.5000, 0.7311, 0.8808, 0.9526, 0.9820, 0.9933, 0.9975, 0.9991, 0.9997, 0.9999]   # README.md:68
+README_SORT_IN = [101, 102, 208, 99, 1, 127, 62, 8, 336, 336]                                       # samples/01_sort_even_first.py:36
+README_SORT_OUT = [102, 208, 62, 8, 336, 336, 101, 99, 1, 127]                                      # README.md:95-99
+
+
+def cpu_module(ir, inputs, **kw):
+    from oracle.cpu_backend import CpuModule
+    return CpuModule(parse_program(ir, inputs), **kw)
+
+
+def test_sigmoid_known_answer():
+    from oracle import hot_ops
+    x = np.arange(10, dtype=np.float32)
+    assert np.allclose(hot_ops.sigmoid_f32(x), README_SIGMOID, atol=5e-5)
+    m = cpu_module('sigmoid_f32[N] = 1 - 1 / (1 + data[N].call(strs.exp))', ['data=float32[N:4096000]'])
+    assert np.allclose(m(data=x)['sigmoid_f32'], README_SIGMOID, atol=5e-5)
+
+
+def test_sigmoid_matches_float64_closed_form():
+    from oracle import hot_ops
+    x = workloads.sigmoid_input(1, 100_000).numpy()
+    want = 1.0 / (1.0 + np.exp(-x.astype(np.float64)))
+    assert np.allclose(hot_ops.sigmoid_f32(x), want, rtol=1e-5, atol=1e-6)
+    m = cpu_module('sigmoid_f32[N] = 1 - 1 / (1 + data[N].call(strs.exp))', ['data=float32[N:4096000]'])
+    assert np.allclose(m(data=x)['sigmoid_f32'], want, rtol=1e-5, atol=1e-6)
+
+
+def sort_pipeline_via_ir(x: np.ndarray) -> np.ndarray:
+    """The sample's three steps with the two exported programs run by the IR oracle."""
+    m1 = cpu_module('space[data[N] % 2, N] = 1', ['data=int32[N]', 'space=int32[2, N]'])
+    m2 = cpu_module('output[ids[N] - 1] = (val[N % val.size(0)]).when(ids[N] > 0)',
+                    ['ids=int32[N]', 'val=int32[M]', 'output=int32[M]'])
+    space = np.zeros((2, x.size), np.int32)
+    m1(data=x, space=space)
+    ids = (np.cumsum(space.reshape(-1), dtype=np.int32) * space.reshape(-1)).astype(np.int32)
+    out = np.zeros_like(x)
+    m2(ids=ids, val=x, output=out)
+    return out
+
+
+def test_sort_known_answer():
+    from oracle import hot_ops
+    x = np.array(README_SORT_IN, dtype=np.int32)
+    assert hot_ops.sort_even_first_i32(x).tolist() == README_SORT_OUT
+    assert sort_pipeline_via_ir(x).tolist() == README_SORT_OUT
+
+
+@pytest.mark.parametrize('n', [1, 2, 63, 64, 65, 4095, 4096, 4097, 100_003])
+def test_sort_is_stable_partition(n):
+    from oracle import hot_ops
+    x = workloads.partition_input(n, n).numpy()
+    want = np.concatenate([x[x % 2 == 0], x[x % 2 == 1]])
+    assert np.array_equal(hot_ops.sort_even_first_i32(x), want)
+    if n <= 4097:
+        assert np.array_equal(sort_pipeline_via_ir(x), want)
+
+
+def test_sort_all_even_all_odd():
+    from oracle import hot_ops
+    ev = np.arange(0, 2000, 2, dtype=np.int32)
+    od = ev + 1
+    assert np.array_equal(hot_ops.sort_even_first_i32(ev), ev)
+    assert np.array_equal(hot_ops.sort_even_first_i32(od), od)
+
+
+# ---------------------------------------------------------------- int4 products
+def dequant_f64(p):
+    q, z, s = p['q'].numpy().astype(np.float64), p['z'].numpy().astype(np.float64), p['scales'].numpy().astype(np.float64)
+    return (q - np.repeat(z, 128, axis=0)) * np.repeat(s, 128, axis=0)
+
+
+def test_w4a16_against_float64():
+    from oracle import hot_ops
+    p = workloads.w4_problem(3, 2, 256, 64)
+    got = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy())
+    want = p['x'].numpy().astype(np.float64) @ dequant_f64(p)
+    assert np.allclose(got.astype(np.float64), want, rtol=4e-3, atol=4e-3)
+
+
+def test_w4a16_special_cases_pin_layout():
+    from oracle import hot_ops
+    K, N = 256, 32
+    ones = np.ones((K // 128, N), np.float16)
+    # q == z everywhere -> y == 0
+    q = torch.full((K, N), 7, dtype=torch.uint8)
+    z = torch.full((K // 128, N), 7, dtype=torch.uint8)
+    x = np.random.default_rng(0).standard_normal((1, K)).astype(np.float16)
+    y = hot_ops.gemm_w4a16(x, workloads.pack_w4(q).numpy(), ones, workloads.pack_z4(z).numpy())
+    assert np.all(y == 0)
+    # scales 1, z 0, q 1 -> y = sum(x)
+    q = torch.ones((K, N), dtype=torch.uint8)
+    z = torch.zeros((K // 128, N), dtype=torch.uint8)
+    y = hot_ops.gemm_w4a16(x, workloads.pack_w4(q).numpy(), ones, workloads.pack_z4(z).numpy())
+    assert np.allclose(y.astype(np.float32), x.astype(np.float32).sum(), atol=2e-2)
+    # a single nibble q[k0, n0] = 9 and x one-hot at k0: y[n0] = 9, zero elsewhere (pins nibble order along K)
+    for k0, n0 in [(0, 0), (1, 5), (130, 17), (255, 31)]:
+        q = torch.zeros((K, N), dtype=torch.uint8)
+        q[k0, n0] = 9
+        xx = np.zeros((1, K), np.float16)
+        xx[0, k0] = 1
+        y = hot_ops.gemm_w4a16(xx, workloads.pack_w4(q).numpy(), ones, workloads.pack_z4(z).numpy())
+        want = np.zeros(N)
+        want[n0] = 9
+        assert np.array_equal(y[0].astype(np.float64), want)
+    # a single zero point z[g0, n0] = 5 with q = 5 at one k of that group and x all ones (pins nibble order along N)
+    for g0, n0 in [(0, 0), (1, 1), (1, 30)]:
+        z = torch.zeros((K // 128, N), dtype=torch.uint8)
+        z[g0, n0] = 5
+        q = torch.zeros((K, N), dtype=torch.uint8)
+        xx = np.ones((1, K), np.float16)
+        y = hot_ops.gemm_w4a16(xx, workloads.pack_w4(q).numpy(), ones, workloads.pack_z4(z).numpy())
+        want = np.zeros(N)
+        want[n0] = -5 * 128
+        assert np.array_equal(y[0].astype(np.float64), want)
+
+
+def test_w4a16_ir_program_agrees_with_plain_c():
+    from oracle import hot_ops
+    p = workloads.w4_problem(5, 3, 256, 64)
+    m = cpu_module(patterns.W4A16_IR, patterns.W4A16_INPUTS, fast_math=False)
+    got = m(x=p['x'].numpy(), qweight=p['qweight'].numpy(), scales=p['scales'].numpy(), qzeros=p['qzeros'].numpy())['y']
+    want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy())
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize('scales_dtype', [np.float32, np.float16])
+def test_gptq_program(scales_dtype):
+    from oracle import hot_ops
+    K, N = 512, 96
+    g = torch.Generator().manual_seed(11)
+    q = torch.randint(0, 16, (K, N), generator=g)
+    s = (torch.rand(K // 128, N, generator=g) * 0.019 + 0.001).numpy().astype(scales_dtype)
+    x = torch.randn(K, generator=g).numpy()
+    qw = workloads.pack_gptq(q).numpy()
+    got = hot_ops.gemv_gptq_f32(x, qw, s)
+    want = x.astype(np.float64) @ ((q.numpy().astype(np.float64) - 8) * np.repeat(s.astype(np.float64), 128, axis=0))
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
+    sd = 'float32' if scales_dtype == np.float32 else 'float16'
+    m = cpu_module(patterns.GPTQ_GEMV_IR, patterns._gptq_inputs('float32', sd), fast_math=False)
+    got_ir = m(input0=x, qweight=qw, scales=s)['my_result']
+    assert np.allclose(got_ir, got, rtol=1e-6, atol=1e-6)
+    # nibble j of a word is k % 8 == j: one-hot check
+    q1 = torch.full((K, N), 8)
+    q1[13, 7] = 15
+    x1 = np.zeros(K, np.float32)
+    x1[13] = 1
+    y = hot_ops.gemv_gptq_f32(x1, workloads.pack_gptq(q1).numpy(), np.ones((K // 128, N), scales_dtype))
+    want1 = np.zeros(N)
+    want1[7] = 7
+    assert np.array_equal(y, want1)
+
+
+# ---------------------------------------------------------------- harness
+def test_fill_and_digest_closed_form():
+    from oracle.cpu_backend import digest, fill
+    a = fill(np.zeros(1000, np.float32), 'float32', 2)
+    assert np.array_equal(a, (np.arange(1000) + 3) % 71)
+    assert np.array_equal(fill(np.ones(10, np.int32), 'int32', 0), np.zeros(10))
+    h = fill(np.zeros(100, np.float16), 'float16', 0)
+    assert np.array_equal(h.astype(np.float32), (np.arange(100) + 1) % 71)
+    out = np.linspace(-1, 1, 500).astype(np.float32)
+    want = float(np.sum(((np.arange(500) + 1) % 83) * out.astype(np.float64)))
+    assert digest(out, 'float32') == pytest.approx(want, rel=1e-12)
+
+
+def test_reduce_identities_and_ops():
+    x = np.random.default_rng(1).standard_normal((8, 33)).astype(np.float32)
+    inp = {'input0': {'dtype': 'float32', 'shape': [8, 33]}}
+    assert np.allclose(cpu_module('output0[N] +=! input0[N, C]', dict(inp))(input0=x)['output0'], x.sum(1), rtol=1e-5, atol=1e-5)
+    assert np.array_equal(cpu_module('output0[N] >=! input0[N, C]', dict(inp))(input0=x)['output0'], x.max(1))
+    assert np.array_equal(cpu_module('output0[N] <=! input0[N, C]', dict(inp))(input0=x)['output0'], x.min(1))
+    b = (np.random.default_rng(2).random((8, 33)) > 0.9).astype(np.int8)
+    inp8 = {'input0': {'dtype': 'int8', 'shape': [8, 33]}}
+    assert np.array_equal(cpu_module('output0[N] |=! input0[N, C]', dict(inp8))(input0=b)['output0'], b.any(1))
+    assert np.array_equal(cpu_module('output0[N] &=! input0[N, C]', dict(inp8))(input0=b)['output0'], b.all(1))
