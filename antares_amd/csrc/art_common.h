@@ -23,8 +23,8 @@ Workspace& workspace();
 // so they never share bytes with scratch data.
 constexpr size_t kGemvTicketOffset = 0;                 // 16384 ticket words of the split-K kernels
 constexpr size_t kGemvTicketBytes = 64 * 1024;
-constexpr size_t kScanTicketOffset = 64 * 1024;          // ticket words of the scan / partition kernels
-constexpr size_t kScratchOffset = 128 * 1024;            // partial sums, tile counts (any content)
+constexpr size_t kSlotOffset = 64 * 1024;                // 64-bit split-K accumulators (zero between launches)
+constexpr size_t kScratchOffset = 4 * 1024 * 1024;       // partial sums, tile counts (any content)
 
 }  // namespace art
 

@@ -94,12 +94,16 @@ __global__ __launch_bounds__(kThreads) void gemv_gptq_kernel(const XT* __restric
     return;
   }
   if (owner) __hip_atomic_store(&partial[(size_t)split * N + col], res, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __threadfence();
+  // The partial sums were written through to device-coherent memory; wait until
+  // they have landed (vmcnt(0)) before this block's ticket can be seen.  A device-scope
+  // release fence would do the same but writes back the whole L2 of the XCD.
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
-  if (tid == 0) s_ticket = atomicAdd(&tickets[tile], 1u);
+  if (tid == 0) s_ticket = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   if (s_ticket != (unsigned int)(splits - 1)) return;
-  __threadfence();
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
   if (owner) {
     float r = 0.f;
     for (int s = 0; s < splits; ++s)

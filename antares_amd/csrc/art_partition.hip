@@ -3,17 +3,19 @@
 // Replaces the reference's three-step pipeline of samples/01_sort_even_first.py:9-27
 // (classify scatter into a [2,N] flag plane, torch cumsum over 2N flags, bucket
 // scatter; about 64 bytes of traffic per element) by two launches that move
-// 12 bytes per element:
+// 12 bytes per element and need no atomics, fences or zeroed state:
 //
-//   count    reads the input once, leaves the number of even values of every
-//            4096-element tile in the workspace; the block that draws the last
-//            ticket turns the counts into exclusive prefixes and the total.
-//   scatter  reads the input again, ranks the even values of a tile with
-//            wavefront ballots + popcounts and a 4-wave prefix through LDS,
-//            compacts evens and odds of the tile into LDS and writes each run
-//            with fully coalesced stores:
-//              even -> out[prefix[t] + rank]
-//              odd  -> out[total_even + (t*4096 - prefix[t]) + rank]
+//   count    block b reads its span of the input (a whole number of
+//            4096-element tiles) and stores the number of even values in
+//            counts[b].
+//   scatter  block b adds up counts[0..b) and counts[b..B) (B <= 8192 words,
+//            served by L2) to get the number of evens before its span and the
+//            total; then, tile by tile, it ranks the even values with a
+//            wavefront prefix + a 4-wave prefix through LDS, compacts evens
+//            and odds of the tile in LDS and writes both runs with fully
+//            coalesced stores:
+//              even -> out[evens_before + rank]
+//              odd  -> out[total_even + odds_before + rank]
 //
 // The order inside both halves is the input order, and the result is
 // bit-identical to the reference pipeline for non-negative inputs (for negative
@@ -44,119 +46,113 @@ __device__ __forceinline__ i32x4 load_vec(const int* __restrict__ in, long long 
   return v;
 }
 
-__global__ __launch_bounds__(kThreads) void partition_count_kernel(const int* __restrict__ in, long long n, int tiles,
-                                                                    unsigned int* __restrict__ counts,   // [tiles + 1]
-                                                                    unsigned int* __restrict__ ticket) {
+__global__ __launch_bounds__(kThreads) void partition_count_kernel(const int* __restrict__ in, long long n, int tiles_per_block,
+                                                                    unsigned int* __restrict__ counts) {
   __shared__ unsigned int s_wave[4];
-  __shared__ unsigned int s_last;
   const int tid = threadIdx.x;
-  for (int t = blockIdx.x; t < tiles; t += gridDim.x) {
-    const long long base = (long long)t * kTile;
-    unsigned int c = 0;
+  unsigned int c = 0;
+  for (int s = 0; s < tiles_per_block; ++s) {
+    const long long base = ((long long)blockIdx.x * tiles_per_block + s) * kTile;
+    if (base >= n) break;
 #pragma unroll
     for (int j = 0; j < kVecPerThread; ++j) c += even_count4(load_vec(in, base, j, n));
-    // wavefront sum: xor butterfly
+  }
 #pragma unroll
-    for (int m = 1; m < 64; m <<= 1) c += __shfl_xor(c, m, 64);
-    if ((tid & 63) == 0) s_wave[tid >> 6] = c;
-    __syncthreads();
-    if (tid == 0)
-      __hip_atomic_store(&counts[t], s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-  }
-  __threadfence();
-  if (tid == 0) s_last = (atomicAdd(ticket, 1u) == gridDim.x - 1) ? 1u : 0u;
+  for (int m = 1; m < 64; m <<= 1) c += __shfl_xor(c, m, 64);
+  if ((tid & 63) == 0) s_wave[tid >> 6] = c;
   __syncthreads();
-  if (!s_last) return;
-  __threadfence();
-  // exclusive scan of counts[0..tiles) in place; counts[tiles] = total.  One block, chunks of 256.
-  __shared__ unsigned int s_scan[kThreads];
-  unsigned int carry = 0;
-  for (int c0 = 0; c0 < tiles; c0 += kThreads) {
-    const int i = c0 + tid;
-    const unsigned int v = (i < tiles) ? __hip_atomic_load(&counts[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    s_scan[tid] = v;
-    __syncthreads();
-    // Hillis-Steele inclusive scan over 256 entries
-    for (int off = 1; off < kThreads; off <<= 1) {
-      const unsigned int add = (tid >= off) ? s_scan[tid - off] : 0u;
-      __syncthreads();
-      s_scan[tid] += add;
-      __syncthreads();
-    }
-    if (i < tiles) counts[i] = carry + s_scan[tid] - v;
-    carry += s_scan[kThreads - 1];
-    __syncthreads();
-  }
-  if (tid == 0) {
-    counts[tiles] = carry;
-    *ticket = 0u;
-  }
+  if (tid == 0) counts[blockIdx.x] = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
 }
 
 __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* __restrict__ in, int* __restrict__ out,
-                                                                      long long n, const unsigned int* __restrict__ prefix,
-                                                                      int tiles) {
+                                                                      long long n, const unsigned int* __restrict__ counts,
+                                                                      int tiles_per_block) {
   __shared__ int s_items[kTile];
   __shared__ unsigned int s_wave[4][kVecPerThread];
+  __shared__ unsigned long long s_sum[4][2];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int t = blockIdx.x;
-  const long long base = (long long)t * kTile;
-  const long long valid = (n - base < kTile) ? (n - base) : kTile;      // elements of this tile that exist
-  const unsigned int tile_prefix = prefix[t];
-  const unsigned int total_even = prefix[tiles];
+  const int b = blockIdx.x, nblocks = gridDim.x;
 
+  // first tile's loads go out before the prefix work
+  const long long span_base = (long long)b * tiles_per_block * kTile;
   i32x4 v[kVecPerThread];
-  unsigned int cnt[kVecPerThread], incl[kVecPerThread];
 #pragma unroll
-  for (int j = 0; j < kVecPerThread; ++j) {
-    v[j] = load_vec(in, base, j, n);
-    cnt[j] = even_count4(v[j]);
+  for (int j = 0; j < kVecPerThread; ++j) v[j] = load_vec(in, span_base, j, n);
+
+  // evens before this block and in total (64-bit: n may exceed 2^31 / 2)
+  unsigned long long before_sum = 0, total_sum = 0;
+  for (int i = tid; i < nblocks; i += kThreads) {
+    const unsigned int c = counts[i];
+    total_sum += c;
+    if (i < b) before_sum += c;
   }
-  // inclusive prefix of cnt[j] over the lanes of the wavefront
 #pragma unroll
-  for (int j = 0; j < kVecPerThread; ++j) {
-    unsigned int s = cnt[j];
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const unsigned int up = __shfl_up(s, off, 64);
-      if (lane >= off) s += up;
-    }
-    incl[j] = s;
-    if (lane == 63) s_wave[wave][j] = s;
+  for (int m = 1; m < 64; m <<= 1) {
+    before_sum += __shfl_xor(before_sum, m, 64);
+    total_sum += __shfl_xor(total_sum, m, 64);
   }
+  if (lane == 0) { s_sum[wave][0] = before_sum; s_sum[wave][1] = total_sum; }
   __syncthreads();
-  // evens before (j, wave, lane) in tile order (j outermost, then thread id)
-  unsigned int tile_even = 0, before[kVecPerThread];
+  long long even_before = (long long)(s_sum[0][0] + s_sum[1][0] + s_sum[2][0] + s_sum[3][0]);
+  const long long total_even = (long long)(s_sum[0][1] + s_sum[1][1] + s_sum[2][1] + s_sum[3][1]);
+
+  for (int s = 0; s < tiles_per_block; ++s) {
+    const long long base = span_base + (long long)s * kTile;
+    if (base >= n) break;
+    if (s > 0) {
 #pragma unroll
-  for (int j = 0; j < kVecPerThread; ++j) {
-    unsigned int b = tile_even;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      if (w < wave) b += s_wave[w][j];
-      tile_even += s_wave[w][j];
+      for (int j = 0; j < kVecPerThread; ++j) v[j] = load_vec(in, base, j, n);
     }
-    before[j] = b + incl[j] - cnt[j];
-  }
-  // compact into LDS: evens to [0, tile_even), odds to [tile_even, kTile)
+    const long long valid = (n - base < kTile) ? (n - base) : kTile;      // elements of this tile that exist
+    unsigned int cnt[kVecPerThread], incl[kVecPerThread];
+    // inclusive prefix of the per-vector even counts over the lanes of the wavefront
 #pragma unroll
-  for (int j = 0; j < kVecPerThread; ++j) {
-    const unsigned int p0 = 4u * (j * kThreads + tid);      // tile-order index of v[j].x
-    unsigned int ev = before[j];
-    const int items[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+    for (int j = 0; j < kVecPerThread; ++j) {
+      cnt[j] = even_count4(v[j]);
+      unsigned int p = cnt[j];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const bool is_even = (items[e] & 1) == 0;
-      const unsigned int dst = is_even ? ev : (tile_even + (p0 + e - ev));
-      s_items[dst] = items[e];
-      ev += is_even ? 1u : 0u;
+      for (int off = 1; off < 64; off <<= 1) {
+        const unsigned int up = __shfl_up(p, off, 64);
+        if (lane >= off) p += up;
+      }
+      incl[j] = p;
+      if (lane == 63) s_wave[wave][j] = p;
     }
+    __syncthreads();
+    // evens before (j, wave, lane) in tile order (j outermost, then thread id)
+    unsigned int tile_even = 0, before[kVecPerThread];
+#pragma unroll
+    for (int j = 0; j < kVecPerThread; ++j) {
+      unsigned int acc = tile_even;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        if (w < wave) acc += s_wave[w][j];
+        tile_even += s_wave[w][j];
+      }
+      before[j] = acc + incl[j] - cnt[j];
+    }
+    // compact into LDS: evens to [0, tile_even), odds to [tile_even, kTile)
+#pragma unroll
+    for (int j = 0; j < kVecPerThread; ++j) {
+      const unsigned int p0 = 4u * (j * kThreads + tid);      // tile-order index of v[j].x
+      unsigned int ev = before[j];
+      const int items[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool is_even = (items[e] & 1) == 0;
+        const unsigned int dst = is_even ? ev : (tile_even + (p0 + e - ev));
+        s_items[dst] = items[e];
+        ev += is_even ? 1u : 0u;
+      }
+    }
+    __syncthreads();
+    const long long odd_base = total_even + (base - even_before);
+    const unsigned int tile_odd = (unsigned int)valid - tile_even;     // padding was counted as odd and sits last
+    for (unsigned int i = tid; i < tile_even; i += kThreads) out[even_before + i] = s_items[i];
+    for (unsigned int i = tid; i < tile_odd; i += kThreads) out[odd_base + i] = s_items[tile_even + i];
+    even_before += tile_even;
+    __syncthreads();                                            // s_items / s_wave are reused by the next tile
   }
-  __syncthreads();
-  const long long odd_base = (long long)total_even + (base - tile_prefix);
-  const unsigned int tile_odd = (unsigned int)valid - tile_even;     // padded elements were counted as odd and sit last
-  for (unsigned int i = tid; i < tile_even; i += kThreads) out[tile_prefix + i] = s_items[i];
-  for (unsigned int i = tid; i < tile_odd; i += kThreads) out[odd_base + i] = s_items[tile_even + i];
 }
 
 }  // namespace
@@ -168,16 +164,15 @@ extern "C" int art_partition_even_first_i32(const void* in_dev, void* out_dev, l
   ART_REQUIRE(((uintptr_t)in_dev % 16) == 0, "art_partition_even_first_i32: input must be 16-byte aligned");
   art::Workspace& ws = art::workspace();
   ART_REQUIRE(ws.base != nullptr, "art_partition_even_first_i32: call art_init first");
-  const long long tiles_ll = (n + kTile - 1) / kTile;
-  ART_REQUIRE(art::kScratchOffset + (size_t)(tiles_ll + 1) * 4 <= ws.bytes, "art_partition_even_first_i32: n too large (%lld)", n);
-  const int tiles = (int)tiles_ll;
-  unsigned int* ticket = reinterpret_cast<unsigned int*>(reinterpret_cast<char*>(ws.base) + art::kScanTicketOffset);
+  const long long tiles = (n + kTile - 1) / kTile;
+  constexpr long long kMaxBlocks = 8192;                        // bounds the counts every block adds up
+  const int tiles_per_block = (int)((tiles + kMaxBlocks - 1) / kMaxBlocks);
+  const int blocks = (int)((tiles + tiles_per_block - 1) / tiles_per_block);
   unsigned int* counts = reinterpret_cast<unsigned int*>(reinterpret_cast<char*>(ws.base) + art::kScratchOffset);
   hipStream_t st = (hipStream_t)stream;
-  const int count_blocks = tiles < 2048 ? tiles : 2048;
-  partition_count_kernel<<<dim3(count_blocks), dim3(kThreads), 0, st>>>((const int*)in_dev, n, tiles, counts, ticket);
+  partition_count_kernel<<<dim3(blocks), dim3(kThreads), 0, st>>>((const int*)in_dev, n, tiles_per_block, counts);
   ART_LAUNCH_CHECK();
-  partition_scatter_kernel<<<dim3(tiles), dim3(kThreads), 0, st>>>((const int*)in_dev, (int*)out_dev, n, counts, tiles);
+  partition_scatter_kernel<<<dim3(blocks), dim3(kThreads), 0, st>>>((const int*)in_dev, (int*)out_dev, n, counts, tiles_per_block);
   ART_LAUNCH_CHECK();
   return 0;
 }
