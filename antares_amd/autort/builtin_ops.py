@@ -44,3 +44,137 @@ class PartitionEvenFirst:
 @builtin('partition_even_first_i32')
 def _partition():
     return PartitionEvenFirst()
+
+
+# ---------------------------------------------------------------------------
+# Llama decode operators (call sites: samples/05_llama2_7b_int4.py:128-131,157-158,165)
+# ---------------------------------------------------------------------------
+_DT = {torch.float32: 0, torch.float16: 1}
+RMS_EPS = 1e-5
+
+
+def _dt(t: torch.Tensor, what: str) -> int:
+    if t.dtype not in _DT:
+        raise TypeError(f'{what} must be float32 or float16, got {t.dtype}')
+    return _DT[t.dtype]
+
+
+def _pos_args(extra, what: str):
+    """``extra=[pos]``: a Python int, or a 1-element int32 GPU tensor (read on the
+    device, so a recorded HIP graph can be replayed for every position)."""
+    if not extra:
+        raise TypeError(f'{what} needs extra=[pos]')
+    pos = extra[0]
+    if isinstance(pos, torch.Tensor):
+        if pos.dtype != torch.int32 or pos.numel() != 1 or not pos.is_cuda:
+            raise TypeError(f'{what}: a tensor position must be a 1-element int32 GPU tensor')
+        return c_void_p(pos.data_ptr()), 0
+    return c_void_p(0), int(pos)
+
+
+class RmsNorm:
+    """``rmsnorm_f32(x[N], vsum[1], w[N], extra=[1/N]) -> out[N]``:
+    ``out = x * rsqrt(vsum * extra[0] + eps) * w`` with eps = 1e-5 (``extra[1]``
+    overrides it).  ``vsum`` is the caller's fp32 sum of squares; passing ``None``
+    lets the kernel compute it.  ``x`` may also be [rows, N] with one vsum per row."""
+
+    def __init__(self, out_dtype: torch.dtype):
+        self.out_dtype = out_dtype
+        self.name = 'rmsnorm_f32' if out_dtype == torch.float32 else 'rmsnorm_f16'
+
+    def __call__(self, x, vsum, w, out=None, extra=None):
+        n = w.numel()
+        rows = x.numel() // n
+        if rows * n != x.numel() or n == 0:
+            raise ValueError(f'{self.name}: x has {x.numel()} elements, weight {n}')
+        inv_n = float(extra[0]) if extra else 1.0 / n
+        eps = float(extra[1]) if extra and len(extra) > 1 else RMS_EPS
+        if out is None:
+            out = torch.empty(x.shape, dtype=self.out_dtype, device=x.device)
+        if out.numel() != x.numel():
+            raise ValueError(f'{self.name}: out has the wrong size')
+        tensors = [x, w, out]
+        vptr = c_void_p(0)
+        if vsum is not None:
+            vsum = vsum.view(-1)
+            if vsum.dtype != torch.float32 or vsum.numel() != rows:
+                raise TypeError(f'{self.name}: vsum must be float32 with one value per row')
+            tensors.append(vsum)
+            vptr = c_void_p(vsum.data_ptr())
+        _require_cuda(*tensors)
+        capi.check(capi.lib().art_rmsnorm(c_void_p(x.data_ptr()), vptr, c_void_p(w.data_ptr()), c_void_p(out.data_ptr()),
+                                         rows, n, inv_n, eps, _dt(x, 'x'), _dt(w, 'weight'), _dt(out, 'out'),
+                                         c_void_p(current_stream_handle())))
+        return out
+
+
+class Rotary:
+    """``rotary_f32(x[H,2,D/2], inv_freq[D], out[H,D], extra=[pos])`` (rotate-half
+    form) and ``rotate_f32(coef[1,dim/2], data[dim], out[dim], extra=[pos])``
+    (interleaved pairs, samples/03_llama_tiny.py:68-70)."""
+
+    def __init__(self, name: str, interleaved: bool):
+        self.name, self.interleaved = name, interleaved
+
+    def __call__(self, a, b, out=None, extra=None):
+        x, freq = (b, a) if self.interleaved else (a, b)
+        if out is None:
+            out = torch.empty_like(x)
+        if self.interleaved:
+            heads, head_dim = 1, x.numel()
+            if freq.numel() * 2 != x.numel():
+                raise ValueError(f'{self.name}: coefficient tensor must have one entry per pair')
+        else:
+            if x.dim() != 3 or x.shape[1] != 2:
+                raise ValueError(f'{self.name}: x must be viewed as [heads, 2, head_dim/2]')
+            heads, head_dim = x.shape[0], 2 * x.shape[2]
+            if freq.numel() < head_dim // 2:
+                raise ValueError(f'{self.name}: inv_freq is too short')
+        if out.numel() != x.numel() or out.dtype != x.dtype:
+            raise ValueError(f'{self.name}: out must match x in size and dtype')
+        _require_cuda(x, freq, out)
+        pos_dev, pos = _pos_args(extra, self.name)
+        capi.check(capi.lib().art_rotary(c_void_p(x.data_ptr()), c_void_p(freq.data_ptr()), c_void_p(out.data_ptr()), heads,
+                                        head_dim, int(self.interleaved), pos_dev, pos, _dt(x, 'x'), _dt(freq, 'inv_freq'),
+                                        _dt(out, 'out'), c_void_p(current_stream_handle())))
+        return out
+
+
+class DecodeAttention:
+    """``attention_f32(q[H,D], k[S,H,D], v[S,H,D], att_f[1]) -> out[H,D]``: scores
+    ``att_f * q.k``, softmax over S, weighted sum of v (the torch spelling is at
+    samples/03_llama_tiny.py:94-99).  ``extra=[pos]`` with a 1-element int32 GPU
+    tensor makes the kernel use S = pos + 1 read on the device (k, v are then the
+    whole cache)."""
+
+    def __init__(self, name: str):
+        self.name = name
+
+    def __call__(self, q, k, v, att_f, out=None, extra=None):
+        if q.dim() != 2 or k.dim() != 3 or k.shape != v.shape or k.shape[1:] != q.shape:
+            raise ValueError(f'{self.name}: expected q[H,D], k[S,H,D], v[S,H,D]; got {list(q.shape)}, {list(k.shape)}, {list(v.shape)}')
+        if att_f.dtype != torch.float32 or att_f.numel() != 1:
+            raise TypeError(f'{self.name}: att_f must be a 1-element float32 tensor')
+        if k.dtype != v.dtype:
+            raise TypeError(f'{self.name}: k and v must have the same dtype')
+        if out is None:
+            out = torch.empty_like(q)
+        _require_cuda(q, k, v, att_f, out)
+        pos_dev = c_void_p(0)
+        if extra and isinstance(extra[0], torch.Tensor):
+            pos_dev, _ = _pos_args(extra, self.name)
+        capi.check(capi.lib().art_decode_attention(c_void_p(q.data_ptr()), c_void_p(k.data_ptr()), c_void_p(v.data_ptr()),
+                                                  c_void_p(att_f.data_ptr()), c_void_p(out.data_ptr()), k.shape[0], q.shape[0],
+                                                  q.shape[1], pos_dev, _dt(q, 'q'), _dt(k, 'k'), _dt(out, 'out'),
+                                                  c_void_p(current_stream_handle())))
+        return out
+
+
+builtin('rmsnorm_f32')(lambda: RmsNorm(torch.float32))
+builtin('rmsnorm_f16')(lambda: RmsNorm(torch.float16))
+builtin('rotary_f32')(lambda: Rotary('rotary_f32', False))
+builtin('rotary_f16')(lambda: Rotary('rotary_f16', False))
+builtin('rotate_f32')(lambda: Rotary('rotate_f32', True))
+builtin('rotate_f16')(lambda: Rotary('rotate_f16', True))
+builtin('attention_f32')(lambda: DecodeAttention('attention_f32'))
+builtin('attention_f16')(lambda: DecodeAttention('attention_f16'))

@@ -1,0 +1,259 @@
+// Llama decode operators for gfx950: RMSNorm, rotary position embedding
+// (rotate-half and interleaved), single-query attention with softmax.
+//
+// These are the built-in operators the reference's samples call as
+// autort.ops.rmsnorm_f32/_f16, rotary_f32/_f16, rotate_f32, attention_f32/_f16
+// (samples/05_llama2_7b_int4.py:128-131,157-158,165;
+//  samples/04_llama2_7b_fp16.py:83,96-97,103; samples/03_llama_tiny.py:66-70).
+// Their source is not part of the reference tree; the semantics implemented
+// here are stated at each entry point and are the ones the call sites imply
+// (samples/03_llama_tiny.py:94-99 spells the attention in torch).
+//
+// All three are bound by memory latency / bandwidth, not arithmetic: one pass
+// over the data, 128-bit loads, fp32 math, wavefront reductions through DPP.
+#include <hip/hip_fp16.h>
+
+#include "art_common.h"
+
+namespace {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <class T> __device__ __forceinline__ float ld(const T* p, size_t i) { return (float)p[i]; }
+template <class T> __device__ __forceinline__ void st(T* p, size_t i, float v) { p[i] = (T)v; }
+
+// sum over the 64 lanes of a wavefront; every lane gets the result (fixed order)
+__device__ __forceinline__ float wave_sum(float v) {
+#define ART_DPP_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false))
+  ART_DPP_ADD(0xB1);    // quad_perm [1,0,3,2]
+  ART_DPP_ADD(0x4E);    // quad_perm [2,3,0,1]
+  ART_DPP_ADD(0x141);   // row_half_mirror
+  ART_DPP_ADD(0x140);   // row_mirror
+#undef ART_DPP_ADD
+  const int b = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// out[i] = x[i] * rsqrt(vsum * inv_n + eps) * w[i];  vsum = sum x^2 (given by the caller or computed here)
+template <class XT, class WT, class OT>
+__global__ __launch_bounds__(1024) void rmsnorm_kernel(const XT* __restrict__ x, const float* __restrict__ vsum,
+                                                        const WT* __restrict__ w, OT* __restrict__ out, int n, float inv_n,
+                                                        float eps) {
+  __shared__ float s_part[16];
+  const int tid = threadIdx.x;
+  const XT* xr = x + (size_t)blockIdx.x * n;
+  OT* orow = out + (size_t)blockIdx.x * n;
+  float ss;
+  if (vsum != nullptr) {
+    ss = vsum[blockIdx.x];
+  } else {
+    float a = 0.f;
+    for (int i = tid; i < n; i += 1024) {
+      const float v = ld(xr, i);
+      a = fmaf(v, v, a);
+    }
+    a = wave_sum(a);
+    if ((tid & 63) == 0) s_part[tid >> 6] = a;
+    __syncthreads();
+    ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) ss += s_part[k];
+  }
+  const float r = 1.0f / sqrtf(ss * inv_n + eps);
+  for (int i = tid; i < n; i += 1024) st(orow, i, ld(xr, i) * r * ld(w, i));
+}
+
+// ------------------------------------------------------------------ rotary
+// rotate-half (HF Llama): x viewed as [H, 2, D/2]; theta_j = pos * inv_freq[j]
+//   out[h,0,j] = x[h,0,j] cos - x[h,1,j] sin ;  out[h,1,j] = x[h,1,j] cos + x[h,0,j] sin
+// interleaved (llama2.c): pairs (2j, 2j+1) of a flat vector, theta_j = pos * coef[j]
+template <class XT, class FT, class OT, bool INTERLEAVED>
+__global__ __launch_bounds__(256) void rotary_kernel(const XT* __restrict__ x, const FT* __restrict__ freq, OT* __restrict__ out,
+                                                      int heads, int half, const int* __restrict__ pos_dev, int pos_host) {
+  const int pos = pos_dev ? *pos_dev : pos_host;
+  const int i = blockIdx.x * 256 + threadIdx.x;       // pair index over heads * half
+  if (i >= heads * half) return;
+  const int h = i / half, j = i % half;
+  float s, c;
+  if (INTERLEAVED) {
+    sincosf((float)pos * ld(freq, i), &s, &c);        // coef has one entry per pair of the whole vector
+    const size_t a = 2 * (size_t)i, b = a + 1;
+    const float xa = ld(x, a), xb = ld(x, b);
+    st(out, a, xa * c - xb * s);
+    st(out, b, xa * s + xb * c);
+  } else {
+    sincosf((float)pos * ld(freq, j), &s, &c);
+    const size_t a = (size_t)h * 2 * half + j, b = a + half;
+    const float xa = ld(x, a), xb = ld(x, b);
+    st(out, a, xa * c - xb * s);
+    st(out, b, xb * c + xa * s);
+  }
+}
+
+// ------------------------------------------------------------------ attention (one query)
+// att[h,s] = (sum_m q[h,m] k[s,h,m]) * att_f ; p = softmax_s(att) ; out[h,m] = sum_s p[h,s] v[s,h,m]
+// One block per head.  Eight lanes share a position (16 dims = 32 bytes of fp16 each), so a wavefront
+// reads eight 256-byte rows per step; every 8-lane group keeps an online-softmax state (max, sum, 16
+// partial outputs) for the positions it visits; the 32 groups of the block are merged through LDS.
+template <class T> struct Row16;   // 16 consecutive elements as floats
+template <> struct Row16<_Float16> {
+  static __device__ __forceinline__ void load(const _Float16* p, float (&f)[16]) {
+    const u32x4 a = *reinterpret_cast<const u32x4*>(p), b = *reinterpret_cast<const u32x4*>(p + 8);
+    const unsigned int wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+      const h2 v = __builtin_bit_cast(h2, wds[i]);
+      f[2 * i] = (float)v.x;
+      f[2 * i + 1] = (float)v.y;
+    }
+  }
+};
+template <> struct Row16<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&f)[16]) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(p + 4 * i);
+      f[4 * i] = a[0];
+      f[4 * i + 1] = a[1];
+      f[4 * i + 2] = a[2];
+      f[4 * i + 3] = a[3];
+    }
+  }
+};
+
+constexpr int kAttThreads = 256;
+constexpr int kAttGroups = kAttThreads / 8;   // 32 position groups per block
+
+template <class QT, class KT, class OT>
+__global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __restrict__ q, const KT* __restrict__ k,
+                                                                 const KT* __restrict__ v, const float* __restrict__ att_f,
+                                                                 OT* __restrict__ out, int heads, const int* __restrict__ len_dev,
+                                                                 int len_host) {
+  constexpr int D = 128;
+  __shared__ float s_m[kAttGroups], s_l[kAttGroups];
+  __shared__ float s_acc[kAttGroups][D];
+  const int S = len_dev ? (*len_dev + 1) : len_host;     // device form carries the position, length = pos + 1
+  const int h = blockIdx.x, tid = threadIdx.x;
+  const int sub = tid & 7, group = tid >> 3;
+  const float scale = att_f[0];
+  float qf[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) qf[i] = ld(q, (size_t)h * D + sub * 16 + i) * scale;
+
+  float m = -INFINITY, l = 0.f, acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  const size_t row = (size_t)heads * D;
+  for (int s = group; s < S; s += kAttGroups) {
+    float kf[16], vf[16];
+    Row16<KT>::load(k + (size_t)s * row + (size_t)h * D + sub * 16, kf);
+    Row16<KT>::load(v + (size_t)s * row + (size_t)h * D + sub * 16, vf);
+    float d = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kf[i], d);
+    // sum over the 8 lanes of the group (xor 1, xor 2 inside a quad, then the neighbouring quad)
+    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xf, 0xf, false));
+    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xf, 0xf, false));
+    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xf, 0xf, false));
+    const float mn = fmaxf(m, d);
+    const float corr = __expf(m - mn), p = __expf(d - mn);
+    l = l * corr + p;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * vf[i]);
+    m = mn;
+  }
+  if (sub == 0) { s_m[group] = m; s_l[group] = l; }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s_acc[group][sub * 16 + i] = acc[i];
+  __syncthreads();
+  if (tid < D) {
+    float mm = -INFINITY;
+#pragma unroll
+    for (int g = 0; g < kAttGroups; ++g) mm = fmaxf(mm, s_m[g]);
+    float ll = 0.f, o = 0.f;
+#pragma unroll
+    for (int g = 0; g < kAttGroups; ++g) {
+      const float wgt = (s_m[g] == -INFINITY) ? 0.f : __expf(s_m[g] - mm);
+      ll = fmaf(s_l[g], wgt, ll);
+      o = fmaf(s_acc[g][tid], wgt, o);
+    }
+    st(out, (size_t)h * D + tid, o / ll);
+  }
+}
+
+}  // namespace
+
+// dtype codes: 0 = float32, 1 = float16
+#define ART_DT_OK(d) ((d) == 0 || (d) == 1)
+
+extern "C" int art_rmsnorm(const void* x_dev, const void* vsum_dev, const void* w_dev, void* out_dev, int rows, int n,
+                           float inv_n, float eps, int x_dtype, int w_dtype, int out_dtype, void* stream) {
+  ART_REQUIRE(x_dev && w_dev && out_dev && rows >= 1 && n >= 1, "art_rmsnorm: bad arguments");
+  ART_REQUIRE(ART_DT_OK(x_dtype) && ART_DT_OK(w_dtype) && ART_DT_OK(out_dtype), "art_rmsnorm: dtype codes are 0 (f32) / 1 (f16)");
+  hipStream_t st = (hipStream_t)stream;
+  const float* vs = (const float*)vsum_dev;
+#define ART_RMS(XT, WT, OT) rmsnorm_kernel<XT, WT, OT><<<dim3(rows), dim3(1024), 0, st>>>((const XT*)x_dev, vs, (const WT*)w_dev, (OT*)out_dev, n, inv_n, eps)
+  const int key = x_dtype * 4 + w_dtype * 2 + out_dtype;
+  switch (key) {
+    case 0: ART_RMS(float, float, float); break;
+    case 1: ART_RMS(float, float, _Float16); break;
+    case 2: ART_RMS(float, _Float16, float); break;
+    case 3: ART_RMS(float, _Float16, _Float16); break;
+    case 4: ART_RMS(_Float16, float, float); break;
+    case 5: ART_RMS(_Float16, float, _Float16); break;
+    case 6: ART_RMS(_Float16, _Float16, float); break;
+    default: ART_RMS(_Float16, _Float16, _Float16); break;
+  }
+#undef ART_RMS
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int art_rotary(const void* x_dev, const void* freq_dev, void* out_dev, int heads, int head_dim, int interleaved,
+                          const void* pos_dev, int pos, int x_dtype, int freq_dtype, int out_dtype, void* stream) {
+  ART_REQUIRE(x_dev && freq_dev && out_dev && heads >= 1 && head_dim >= 2 && head_dim % 2 == 0, "art_rotary: bad arguments");
+  ART_REQUIRE(ART_DT_OK(x_dtype) && ART_DT_OK(freq_dtype) && ART_DT_OK(out_dtype), "art_rotary: dtype codes are 0 (f32) / 1 (f16)");
+  ART_REQUIRE(x_dtype == out_dtype, "art_rotary: input and output must have the same dtype");
+  hipStream_t st = (hipStream_t)stream;
+  const int half = head_dim / 2, pairs = heads * half;
+  const dim3 grid((pairs + 255) / 256), block(256);
+  const int* pd = (const int*)pos_dev;
+#define ART_ROT(XT, FT, IL) rotary_kernel<XT, FT, XT, IL><<<grid, block, 0, st>>>((const XT*)x_dev, (const FT*)freq_dev, (XT*)out_dev, heads, half, pd, pos)
+  if (interleaved) {
+    if (x_dtype == 0) { if (freq_dtype == 0) ART_ROT(float, float, true); else ART_ROT(float, _Float16, true); }
+    else { if (freq_dtype == 0) ART_ROT(_Float16, float, true); else ART_ROT(_Float16, _Float16, true); }
+  } else {
+    if (x_dtype == 0) { if (freq_dtype == 0) ART_ROT(float, float, false); else ART_ROT(float, _Float16, false); }
+    else { if (freq_dtype == 0) ART_ROT(_Float16, float, false); else ART_ROT(_Float16, _Float16, false); }
+  }
+#undef ART_ROT
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev, const void* att_f_dev, void* out_dev,
+                                    int seq_len, int heads, int head_dim, const void* pos_dev, int q_dtype, int kv_dtype,
+                                    int out_dtype, void* stream) {
+  ART_REQUIRE(q_dev && k_dev && v_dev && att_f_dev && out_dev, "art_decode_attention: null pointer");
+  ART_REQUIRE(head_dim == 128, "art_decode_attention: head_dim must be 128 (got %d)", head_dim);
+  ART_REQUIRE(heads >= 1 && (pos_dev || seq_len >= 1), "art_decode_attention: bad shape");
+  ART_REQUIRE(ART_DT_OK(q_dtype) && ART_DT_OK(kv_dtype) && ART_DT_OK(out_dtype), "art_decode_attention: dtype codes are 0 (f32) / 1 (f16)");
+  ART_REQUIRE(q_dtype == out_dtype, "art_decode_attention: q and out must have the same dtype");
+  ART_REQUIRE(((uintptr_t)k_dev % 16) == 0 && ((uintptr_t)v_dev % 16) == 0, "art_decode_attention: k and v must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const int* pd = (const int*)pos_dev;
+  const float* af = (const float*)att_f_dev;
+#define ART_ATT(QT, KT) attention_kernel<QT, KT, QT><<<dim3(heads), dim3(kAttThreads), 0, st>>>((const QT*)q_dev, (const KT*)k_dev, (const KT*)v_dev, af, (QT*)out_dev, heads, pd, seq_len)
+  if (q_dtype == 0) { if (kv_dtype == 0) ART_ATT(float, float); else ART_ATT(float, _Float16); }
+  else { if (kv_dtype == 0) ART_ATT(_Float16, float); else ART_ATT(_Float16, _Float16); }
+#undef ART_ATT
+  ART_LAUNCH_CHECK();
+  return 0;
+}

@@ -109,10 +109,37 @@ int art_gemv_gptq(const void* x_dev, const void* qweight_dev, const void* scales
                   int K, int N, int x_f16, int scales_f16, void* stream);
 
 /* Stable even-first partition of int32 values: all even values in input order,
- * then all odd values in input order.  One pass (decoupled look-back scan).
+ * then all odd values in input order.  Two launches (count, then rank + scatter),
+ * 12 bytes of traffic per element, no atomics.
  * Replaces the classify -> cumsum -> bucket pipeline of
  * samples/01_sort_even_first.py:9-27. */
 int art_partition_even_first_i32(const void* in_dev, void* out_dev, long long n, void* stream);
+
+/* Llama decode operators.  dtype codes: 0 = float32, 1 = float16.  They replace
+ * the built-in operators the reference's samples call by name and whose source
+ * is not in the reference tree (call sites: samples/05_llama2_7b_int4.py:128-131,
+ * 157-158,165; samples/04_llama2_7b_fp16.py:83,96-97,103; samples/03_llama_tiny.py:66-70).
+ *
+ * art_rmsnorm: out[r,i] = x[r,i] * rsqrt(vsum[r] * inv_n + eps) * w[i], r < rows, i < n.
+ *   vsum (fp32, one per row) is the caller's sum of squares as in the samples, or
+ *   NULL to have the kernel compute it.
+ * art_rotary: rotate-half form, x viewed as [heads, 2, head_dim/2]:
+ *     out[h,0,j] = x[h,0,j] cos(t) - x[h,1,j] sin(t);  out[h,1,j] = x[h,1,j] cos(t) + x[h,0,j] sin(t)
+ *   with t = pos * freq[j]; or, with interleaved != 0, the pairwise form over a
+ *   flat vector: (x[2j], x[2j+1]) rotated by pos * freq[j], freq having one entry
+ *   per pair of the whole vector.  pos is read from pos_dev (int32 on the device)
+ *   when pos_dev != NULL, else taken from `pos`.
+ * art_decode_attention: one query per head against a cache of seq_len positions:
+ *     a[h,s] = att_f[0] * sum_m q[h,m] k[s,h,m];  p = softmax_s(a);  out[h,m] = sum_s p[h,s] v[s,h,m]
+ *   q, out: [heads, 128]; k, v: [seq_len, heads, 128] (dense).  When pos_dev != NULL
+ *   the length is *pos_dev + 1 and seq_len is ignored. */
+int art_rmsnorm(const void* x_dev, const void* vsum_dev, const void* w_dev, void* out_dev, int rows, int n, float inv_n,
+                float eps, int x_dtype, int w_dtype, int out_dtype, void* stream);
+int art_rotary(const void* x_dev, const void* freq_dev, void* out_dev, int heads, int head_dim, int interleaved,
+               const void* pos_dev, int pos, int x_dtype, int freq_dtype, int out_dtype, void* stream);
+int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev, const void* att_f_dev, void* out_dev,
+                         int seq_len, int heads, int head_dim, const void* pos_dev, int q_dtype, int kv_dtype, int out_dtype,
+                         void* stream);
 
 /* Bytes of library workspace art_partition_even_first_i32 / split-K kernels may use. */
 size_t art_workspace_bytes(void);

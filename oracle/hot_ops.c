@@ -82,3 +82,64 @@ void ref_gemv_gptq_f32(const float* x, const int32_t* qweight, const void* scale
     y[n] = acc;
   }
 }
+
+/* RMSNorm as the samples call it (samples/05_llama2_7b_int4.py:128-131): the caller passes
+ * vsum = sum x^2 and 1/N; out[i] = x[i] * rsqrt(vsum/N + eps) * w[i].  vsum == NULL: computed here.
+ * Closed form used to pin it: sum_i (out[i]/w[i])^2 = N / (1 + eps*N/sum x^2). */
+void ref_rmsnorm_f32(const float* x, const float* vsum, const float* w, float* out, int n, float inv_n, float eps) {
+  float ss = 0.0f;
+  if (vsum) ss = vsum[0];
+  else for (int i = 0; i < n; ++i) ss += x[i] * x[i];
+  const float r = 1.0f / sqrtf(ss * inv_n + eps);
+  for (int i = 0; i < n; ++i) out[i] = x[i] * r * w[i];
+}
+
+/* Rotate-half RoPE on x viewed as [heads, 2, half] (the view the sample passes,
+ * samples/05_llama2_7b_int4.py:157): theta_j = pos * inv_freq[j];
+ * out[h,0,j] = x[h,0,j] cos - x[h,1,j] sin ; out[h,1,j] = x[h,1,j] cos + x[h,0,j] sin.
+ * Pinned by: pos = 0 is the identity; every (j, j+half) pair keeps its norm; equals
+ * x*cos + rotate_half(x)*sin of the HF Llama formulation. */
+void ref_rotary_f32(const float* x, const float* inv_freq, float* out, int heads, int head_dim, int pos) {
+  const int half = head_dim / 2;
+  for (int h = 0; h < heads; ++h)
+    for (int j = 0; j < half; ++j) {
+      const float t = (float)pos * inv_freq[j], c = cosf(t), s = sinf(t);
+      const float a = x[(size_t)h * head_dim + j], b = x[(size_t)h * head_dim + half + j];
+      out[(size_t)h * head_dim + j] = a * c - b * s;
+      out[(size_t)h * head_dim + half + j] = b * c + a * s;
+    }
+}
+
+/* Interleaved-pair rotation (samples/03_llama_tiny.py:60,68-70): pair (2j, 2j+1) of a flat
+ * vector is rotated by pos * coef[j]; coef has dim/2 entries. */
+void ref_rotate_f32(const float* coef, const float* data, float* out, int dim, int pos) {
+  for (int j = 0; j < dim / 2; ++j) {
+    const float t = (float)pos * coef[j], c = cosf(t), s = sinf(t);
+    const float a = data[2 * j], b = data[2 * j + 1];
+    out[2 * j] = a * c - b * s;
+    out[2 * j + 1] = a * s + b * c;
+  }
+}
+
+/* Single-query attention, the torch spelling of samples/03_llama_tiny.py:94-99:
+ * att[h,s] = (sum_m q[h,m] k[s,h,m]) * att_f ; softmax over s ; out[h,m] = sum_s att[h,s] v[s,h,m]. */
+void ref_attention_f32(const float* q, const float* k, const float* v, float att_f, float* out, int S, int H, int D) {
+  float* att = (float*)malloc((size_t)S * sizeof(float));
+  for (int h = 0; h < H; ++h) {
+    float mx = -INFINITY;
+    for (int s = 0; s < S; ++s) {
+      float d = 0.0f;
+      for (int m = 0; m < D; ++m) d += q[(size_t)h * D + m] * k[((size_t)s * H + h) * D + m];
+      att[s] = d * att_f;
+      if (att[s] > mx) mx = att[s];
+    }
+    float sum = 0.0f;
+    for (int s = 0; s < S; ++s) { att[s] = expf(att[s] - mx); sum += att[s]; }
+    for (int m = 0; m < D; ++m) {
+      float o = 0.0f;
+      for (int s = 0; s < S; ++s) o += (att[s] / sum) * v[((size_t)s * H + h) * D + m];
+      out[(size_t)h * D + m] = o;
+    }
+  }
+  free(att);
+}

@@ -66,3 +66,45 @@ def gemv_gptq_f32(x, qweight, scales) -> np.ndarray:
     y = np.empty(N, dtype=np.float32)
     lib().ref_gemv_gptq_f32(_p(x), _p(qweight), _p(scales), int(scales.dtype == np.float16), _p(y), K, N)
     return y
+
+
+def _f32(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float32))
+
+
+def rmsnorm(x, vsum, w, inv_n=None, eps=1e-5, out_dtype=np.float32) -> np.ndarray:
+    """Inputs of any float dtype are widened exactly to fp32, the result is rounded to out_dtype."""
+    x, w = _f32(x).reshape(-1), _f32(w).reshape(-1)
+    out = np.empty_like(x)
+    vs = None if vsum is None else _f32(vsum).reshape(-1)
+    lib().ref_rmsnorm_f32(_p(x), _p(vs) if vs is not None else None, _p(w), _p(out), x.size,
+                          ctypes.c_float(1.0 / x.size if inv_n is None else inv_n), ctypes.c_float(eps))
+    return out.astype(out_dtype)
+
+
+def rotary(x, inv_freq, pos: int) -> np.ndarray:
+    """x: [heads, 2, half] (any float dtype); result has x's dtype and shape [heads, 2*half]."""
+    dt = np.asarray(x).dtype
+    xf, f = _f32(x), _f32(inv_freq).reshape(-1)
+    heads, _, half = xf.shape
+    out = np.empty((heads, 2 * half), np.float32)
+    lib().ref_rotary_f32(_p(xf), _p(f), _p(out), heads, 2 * half, int(pos))
+    return out.astype(dt)
+
+
+def rotate(coef, data, pos: int) -> np.ndarray:
+    dt = np.asarray(data).dtype
+    c, d = _f32(coef).reshape(-1), _f32(data).reshape(-1)
+    out = np.empty_like(d)
+    lib().ref_rotate_f32(_p(c), _p(d), _p(out), d.size, int(pos))
+    return out.astype(dt)
+
+
+def attention(q, k, v, att_f: float) -> np.ndarray:
+    """q [H,D], k/v [S,H,D] (any float dtype) -> [H,D] in q's dtype."""
+    dt = np.asarray(q).dtype
+    qf, kf, vf = _f32(q), _f32(k), _f32(v)
+    S, H, D = kf.shape
+    out = np.empty((H, D), np.float32)
+    lib().ref_attention_f32(_p(qf), _p(kf), _p(vf), ctypes.c_float(att_f), _p(out), S, H, D)
+    return out.astype(dt)

@@ -1,0 +1,126 @@
+"""GPU parity tests of the Llama decode operators (autort.ops.rmsnorm_*, rotary_*,
+rotate_*, attention_*) against the CPU oracle.  fp32: 1e-5, fp16: rtol/atol 1e-2."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures('oracle_built')]
+
+FP32_TOL = dict(rtol=1e-5, atol=1e-5)
+FP16_TOL = dict(rtol=1e-2, atol=1e-2)
+
+
+@pytest.fixture(scope='module')
+def autort():
+    import autort as mod
+    return mod
+
+
+def note(msg):
+    print(f'[case] {msg}', flush=True)
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.mark.parametrize('n', [64, 4096, 11008, 1000])
+def test_rmsnorm_f32_like_the_sample(autort, n):
+    """samples/05_llama2_7b_int4.py:128-131: torch computes vsum, the op normalises."""
+    from oracle import hot_ops
+    note(f'rmsnorm_f32 n={n}')
+    dev = autort.device()
+    x = torch.randn(1, n, generator=gen(n))
+    w = 1 + 0.1 * torch.randn(n, generator=gen(n + 1))
+    xd = x.to(dev).float()
+    vsum = (xd * xd).sum().view(1)
+    out = autort.ops.rmsnorm_f32(xd.view(-1), vsum, w.to(dev).float(), extra=[1.0 / int(xd.numel())])
+    want = hot_ops.rmsnorm(x.numpy(), vsum.cpu().numpy(), w.numpy(), 1.0 / n)
+    assert out.dtype == torch.float32 and out.shape == (n,)
+    assert np.allclose(out.cpu().numpy(), want, **FP32_TOL)
+    # fused sum of squares (vsum=None) agrees
+    out2 = autort.ops.rmsnorm_f32(xd.view(-1), None, w.to(dev).float(), extra=[1.0 / n])
+    assert np.allclose(out2.cpu().numpy(), hot_ops.rmsnorm(x.numpy(), None, w.numpy()), **FP32_TOL)
+
+
+def test_rmsnorm_f16_variants(autort):
+    from oracle import hot_ops
+    note('rmsnorm_f16: fp32 x + fp16 w (sample 04), fp16 x + fp16 w')
+    dev = autort.device()
+    n = 4096
+    x = torch.randn(n, generator=gen(1))
+    w = (1 + 0.1 * torch.randn(n, generator=gen(2))).half()
+    xd = x.to(dev)
+    vsum = (xd * xd).sum().view(1)
+    out = autort.ops.rmsnorm_f16(xd, vsum, w.to(dev), extra=[1.0 / n])
+    assert out.dtype == torch.float16
+    want = hot_ops.rmsnorm(x.numpy(), vsum.cpu().numpy(), w.numpy(), 1.0 / n, out_dtype=np.float16)
+    assert np.allclose(out.cpu().numpy().astype(np.float32), want.astype(np.float32), **FP16_TOL)
+    xh = x.half()
+    out = autort.ops.rmsnorm_f16(xh.to(dev), None, w.to(dev))
+    want = hot_ops.rmsnorm(xh.numpy(), None, w.numpy(), out_dtype=np.float16)
+    assert np.allclose(out.cpu().numpy().astype(np.float32), want.astype(np.float32), **FP16_TOL)
+
+
+@pytest.mark.parametrize('dtype,pos', [(torch.float32, 0), (torch.float32, 5), (torch.float32, 383), (torch.float16, 77)])
+def test_rotary_rotate_half(autort, dtype, pos):
+    from oracle import hot_ops
+    note(f'rotary {dtype} pos={pos}')
+    dev = autort.device()
+    H, D = 32, 128
+    x = torch.randn(H * D, generator=gen(pos)).to(dtype)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D)).to(dtype))
+    inv_freq = torch.cat([inv_freq, inv_freq]).view(D)
+    op = autort.ops.rotary_f32 if dtype == torch.float32 else autort.ops.rotary_f16
+    out = torch.empty(H, D, dtype=dtype, device=dev)
+    r = op(x.to(dev).view(H, 2, -1), inv_freq.to(dev), out, extra=[pos])
+    assert r.data_ptr() == out.data_ptr()
+    want = hot_ops.rotary(x.numpy().reshape(H, 2, D // 2), inv_freq.numpy(), pos)
+    tol = FP32_TOL if dtype == torch.float32 else FP16_TOL
+    # fp32 sin/cos of angles up to 383 rad differ by a few ulp of the angle between libraries
+    tol = dict(rtol=tol['rtol'], atol=max(tol['atol'], 1e-4 if pos > 100 else tol['atol']))
+    assert np.allclose(out.cpu().numpy().astype(np.float32), want.astype(np.float32), **tol)
+    # position read on the device gives the same bits
+    pos_t = torch.tensor([pos], dtype=torch.int32, device=dev)
+    out2 = op(x.to(dev).view(H, 2, -1), inv_freq.to(dev), torch.empty_like(out), extra=[pos_t])
+    assert torch.equal(out, out2)
+
+
+def test_rotate_interleaved(autort):
+    from oracle import hot_ops
+    note('rotate_f32 (interleaved pairs)')
+    dev = autort.device()
+    dim, head = 768, 64
+    coef = (1 / torch.pow(1e4, torch.arange(0, dim, 2, dtype=torch.int64) % head / head)).view(1, -1).float()
+    data = torch.randn(dim, generator=gen(3))
+    out = torch.empty(dim, device=dev)
+    autort.ops.rotate_f32(coef.to(dev), data.to(dev).view(-1), out.view(-1), extra=[9])
+    assert np.allclose(out.cpu().numpy(), hot_ops.rotate(coef.numpy(), data.numpy(), 9), **FP32_TOL)
+
+
+@pytest.mark.parametrize('dtype,S', [(torch.float32, 1), (torch.float32, 31), (torch.float32, 130), (torch.float16, 7), (torch.float16, 384)])
+def test_attention_on_cache_views(autort, dtype, S):
+    """k, v are narrow() views of a larger cache, as in samples/05_llama2_7b_int4.py:161-165."""
+    from oracle import hot_ops
+    note(f'attention {dtype} S={S}')
+    dev = autort.device()
+    H, D, seq_len = 32, 128, 400
+    g = gen(S)
+    key_cache = torch.randn(seq_len, H * D, generator=g).to(dtype).to(dev)
+    val_cache = torch.randn(seq_len, H * D, generator=g).to(dtype).to(dev)
+    q = torch.randn(H, D, generator=g).to(dtype).to(dev)
+    att_f = torch.tensor([1 / math.sqrt(D)], dtype=torch.float32, device=dev)
+    b_sk = key_cache.view(seq_len, H, D).narrow(0, 0, S)
+    b_sv = val_cache.view(seq_len, H, D).narrow(0, 0, S)
+    op = autort.ops.attention_f32 if dtype == torch.float32 else autort.ops.attention_f16
+    out = op(q, b_sk, b_sv, att_f)
+    want = hot_ops.attention(q.cpu().numpy(), b_sk.cpu().numpy(), b_sv.cpu().numpy(), float(att_f[0]))
+    tol = FP32_TOL if dtype == torch.float32 else FP16_TOL
+    assert out.shape == (H, D) and out.dtype == dtype
+    assert np.allclose(out.cpu().numpy().astype(np.float32), want.astype(np.float32), **tol)
+    # length taken from a device-side position
+    pos_t = torch.tensor([S - 1], dtype=torch.int32, device=dev)
+    out2 = op(q, key_cache.view(seq_len, H, D), val_cache.view(seq_len, H, D), att_f, extra=[pos_t])
+    assert torch.equal(out, out2)

@@ -187,3 +187,74 @@ def test_reduce_identities_and_ops():
     inp8 = {'input0': {'dtype': 'int8', 'shape': [8, 33]}}
     assert np.array_equal(cpu_module('output0[N] |=! input0[N, C]', dict(inp8))(input0=b)['output0'], b.any(1))
     assert np.array_equal(cpu_module('output0[N] &=! input0[N, C]', dict(inp8))(input0=b)['output0'], b.all(1))
+
+
+# ---------------------------------------------------------------- llama operators
+def test_rmsnorm_closed_forms():
+    from oracle import hot_ops
+    rng = np.random.default_rng(5)
+    n = 4096
+    x, w = rng.standard_normal(n).astype(np.float32), (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    vsum = np.array([(x.astype(np.float64) ** 2).sum()], np.float32)
+    out = hot_ops.rmsnorm(x, vsum, w, 1.0 / n)
+    want = x.astype(np.float64) / np.sqrt((x.astype(np.float64) ** 2).mean() + 1e-5) * w
+    assert np.allclose(out, want, rtol=1e-5, atol=1e-6)
+    # invariant: sum (out/w)^2 = N / (1 + eps N / sum x^2)
+    lhs = ((out.astype(np.float64) / w) ** 2).sum()
+    assert lhs == pytest.approx(n / (1 + 1e-5 * n / float(vsum[0])), rel=1e-5)
+    # computing the sum of squares inside gives the same thing
+    assert np.allclose(hot_ops.rmsnorm(x, None, w), out, rtol=1e-5, atol=1e-6)
+    # eps matters: a tiny input is damped, not blown up
+    tiny = hot_ops.rmsnorm(x * 1e-4, None, w)
+    assert np.abs(tiny).max() < np.abs(out).max()
+
+
+def test_rotary_closed_forms():
+    from oracle import hot_ops
+    rng = np.random.default_rng(6)
+    H, D = 4, 128
+    x = rng.standard_normal((H, 2, D // 2)).astype(np.float32)
+    f = (1.0 / (10000.0 ** (np.arange(0, D, 2, dtype=np.float64) / D))).astype(np.float32)
+    inv_freq = np.concatenate([f, f])
+    assert np.array_equal(hot_ops.rotary(x, inv_freq, 0), x.reshape(H, D))          # pos 0 = identity
+    for pos in (1, 7, 383):
+        out = hot_ops.rotary(x, inv_freq, pos).astype(np.float64)
+        # HF Llama: x*cos + rotate_half(x)*sin, rotate_half(x) = cat(-x2, x1)
+        xf = x.reshape(H, D).astype(np.float64)
+        ang = pos * inv_freq.astype(np.float32).astype(np.float64)
+        rot = np.concatenate([-xf[:, D // 2:], xf[:, :D // 2]], axis=1)
+        assert np.allclose(out, xf * np.cos(ang) + rot * np.sin(ang), atol=2e-4)   # fp32 sin/cos of angles up to 383 rad
+        # each (j, j + D/2) pair keeps its norm
+        n_in = xf[:, :D // 2] ** 2 + xf[:, D // 2:] ** 2
+        n_out = out[:, :D // 2] ** 2 + out[:, D // 2:] ** 2
+        assert np.allclose(n_in, n_out, rtol=1e-5, atol=1e-6)
+
+
+def test_rotate_interleaved():
+    from oracle import hot_ops
+    rng = np.random.default_rng(7)
+    dim = 64
+    data = rng.standard_normal(dim).astype(np.float32)
+    coef = rng.random(dim // 2).astype(np.float32)
+    assert np.array_equal(hot_ops.rotate(coef, data, 0), data)
+    out = hot_ops.rotate(coef, data, 5).astype(np.float64)
+    z = (data[0::2] + 1j * data[1::2]) * np.exp(1j * 5 * coef.astype(np.float64))       # complex multiplication form
+    assert np.allclose(out[0::2], z.real, atol=1e-5) and np.allclose(out[1::2], z.imag, atol=1e-5)
+
+
+def test_attention_closed_forms():
+    from oracle import hot_ops
+    rng = np.random.default_rng(8)
+    S, H, D = 37, 4, 128
+    q = rng.standard_normal((H, D)).astype(np.float32)
+    k = rng.standard_normal((S, H, D)).astype(np.float32)
+    v = rng.standard_normal((S, H, D)).astype(np.float32)
+    f = 1.0 / np.sqrt(D)
+    out = hot_ops.attention(q, k, v, f)
+    att = np.einsum('hm,shm->hs', q.astype(np.float64), k.astype(np.float64)) * f
+    att = np.exp(att - att.max(1, keepdims=True))
+    att /= att.sum(1, keepdims=True)
+    assert np.allclose(out, np.einsum('hs,shm->hm', att, v.astype(np.float64)), rtol=1e-5, atol=1e-5)
+    # q = 0 -> uniform weights -> mean of v ; S = 1 -> v[0]
+    assert np.allclose(hot_ops.attention(np.zeros_like(q), k, v, f), v.mean(0), rtol=1e-5, atol=1e-5)
+    assert np.allclose(hot_ops.attention(q, k[:1], v[:1], f), v[0], rtol=1e-6, atol=1e-6)
