@@ -130,12 +130,18 @@ class Rotary:
             heads, head_dim = x.shape[0], 2 * x.shape[2]
             if freq.numel() < head_dim // 2:
                 raise ValueError(f'{self.name}: inv_freq is too short')
-        if out.numel() != x.numel() or out.dtype != x.dtype:
-            raise ValueError(f'{self.name}: out must match x in size and dtype')
         _require_cuda(x, freq, out)
         pos_dev, pos = _pos_args(extra, self.name)
+        stride = 0
+        if out.numel() != x.numel():
+            # a whole [positions, heads*head_dim] cache: the row is chosen by the device-side position
+            if not pos_dev.value or out.numel() % x.numel() != 0:
+                raise ValueError(f'{self.name}: out must match x in size (or be a cache with extra=[position tensor])')
+            stride = x.numel()
+        if out.dtype != x.dtype:
+            raise ValueError(f'{self.name}: out must have the dtype of x')
         capi.check(capi.lib().art_rotary(c_void_p(x.data_ptr()), c_void_p(freq.data_ptr()), c_void_p(out.data_ptr()), heads,
-                                        head_dim, int(self.interleaved), pos_dev, pos, _dt(x, 'x'), _dt(freq, 'inv_freq'),
+                                        head_dim, int(self.interleaved), pos_dev, pos, stride, _dt(x, 'x'), _dt(freq, 'inv_freq'),
                                         _dt(out, 'out'), c_void_p(current_stream_handle())))
         return out
 

@@ -74,8 +74,10 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const XT* __restrict__ x,
 // interleaved (llama2.c): pairs (2j, 2j+1) of a flat vector, theta_j = pos * coef[j]
 template <class XT, class FT, class OT, bool INTERLEAVED>
 __global__ __launch_bounds__(256) void rotary_kernel(const XT* __restrict__ x, const FT* __restrict__ freq, OT* __restrict__ out,
-                                                      int heads, int half, const int* __restrict__ pos_dev, int pos_host) {
+                                                      int heads, int half, const int* __restrict__ pos_dev, int pos_host,
+                                                      long long out_row_stride) {
   const int pos = pos_dev ? *pos_dev : pos_host;
+  out += (size_t)pos * out_row_stride;                // out is a [positions, heads*head_dim] cache when the stride is set
   const int i = blockIdx.x * 256 + threadIdx.x;       // pair index over heads * half
   if (i >= heads * half) return;
   const int h = i / half, j = i % half;
@@ -217,15 +219,17 @@ extern "C" int art_rmsnorm(const void* x_dev, const void* vsum_dev, const void* 
 }
 
 extern "C" int art_rotary(const void* x_dev, const void* freq_dev, void* out_dev, int heads, int head_dim, int interleaved,
-                          const void* pos_dev, int pos, int x_dtype, int freq_dtype, int out_dtype, void* stream) {
+                          const void* pos_dev, int pos, long long out_row_stride, int x_dtype, int freq_dtype, int out_dtype,
+                          void* stream) {
   ART_REQUIRE(x_dev && freq_dev && out_dev && heads >= 1 && head_dim >= 2 && head_dim % 2 == 0, "art_rotary: bad arguments");
   ART_REQUIRE(ART_DT_OK(x_dtype) && ART_DT_OK(freq_dtype) && ART_DT_OK(out_dtype), "art_rotary: dtype codes are 0 (f32) / 1 (f16)");
   ART_REQUIRE(x_dtype == out_dtype, "art_rotary: input and output must have the same dtype");
+  ART_REQUIRE(out_row_stride >= 0, "art_rotary: negative row stride");
   hipStream_t st = (hipStream_t)stream;
   const int half = head_dim / 2, pairs = heads * half;
   const dim3 grid((pairs + 255) / 256), block(256);
   const int* pd = (const int*)pos_dev;
-#define ART_ROT(XT, FT, IL) rotary_kernel<XT, FT, XT, IL><<<grid, block, 0, st>>>((const XT*)x_dev, (const FT*)freq_dev, (XT*)out_dev, heads, half, pd, pos)
+#define ART_ROT(XT, FT, IL) rotary_kernel<XT, FT, XT, IL><<<grid, block, 0, st>>>((const XT*)x_dev, (const FT*)freq_dev, (XT*)out_dev, heads, half, pd, pos, out_row_stride)
   if (interleaved) {
     if (x_dtype == 0) { if (freq_dtype == 0) ART_ROT(float, float, true); else ART_ROT(float, _Float16, true); }
     else { if (freq_dtype == 0) ART_ROT(_Float16, float, true); else ART_ROT(_Float16, _Float16, true); }

@@ -1,0 +1,194 @@
+"""Llama-2-shaped int4 decode driven through ``autort.ops`` — the host-side glue of
+the reference's samples/05_llama2_7b_int4.py:109-200 for the benchmark
+configuration: every linear layer in the packed int4 group-128 format with
+per-group zero points, fp16 embeddings / norm weights / activations / KV cache,
+batch 1, one token per step.
+
+Differences from the sample's ``forward`` that do not change results:
+* the sum of squares of RMSNorm is computed inside the operator (``vsum=None``);
+* q, k, v are projected into a scratch vector; k is rotated straight into its
+  cache row and v copied into its row by kernels that read the position from a
+  1-element device tensor, so one recorded HIP graph serves every position;
+* residual add, SiLU*up and the embedding row select are einstein_v2 programs
+  exported through ``autort.export`` (the sample uses torch ops for them).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+from . import workloads
+from .autort import patterns
+
+
+@dataclass
+class LlamaConfig:
+    n_layers: int = 32
+    dim: int = 4096
+    n_heads: int = 32
+    ffn: int = 11008
+    vocab: int = 32000
+    max_seq: int = 384
+    rms_eps: float = 1e-5
+    rope_base: float = 10000.0
+
+    @property
+    def head_dim(self) -> int:
+        return self.dim // self.n_heads
+
+    def weight_bytes_per_token(self) -> int:
+        """Bytes of packed weights, scales and zero points one decode step streams."""
+        per_layer = sum(workloads.w4_bytes(0, k, n) for k, n in self.layer_shapes())
+        return self.n_layers * per_layer + workloads.w4_bytes(0, self.dim, self.vocab)
+
+    def layer_shapes(self):
+        return [(self.dim, 3 * self.dim), (self.dim, self.dim), (self.dim, 2 * self.ffn), (self.ffn, self.dim)]
+
+
+def random_int4_linear(gen: torch.Generator, K: int, N: int) -> Dict[str, torch.Tensor]:
+    """Packed weights drawn directly as bytes: a uniform byte is two independent uniform nibbles."""
+    qweight = torch.empty(K // 2, N, dtype=torch.uint8).random_(0, 256, generator=gen)
+    qzeros = torch.empty(K // 128, N // 2, dtype=torch.uint8).random_(0, 256, generator=gen)
+    scales = (torch.rand(K // 128, N, generator=gen, dtype=torch.float32) * 0.019 + 0.001).to(torch.float16)
+    return {'qweight': qweight, 'qzeros': qzeros, 'scales': scales}
+
+
+def random_weights(cfg: LlamaConfig, seed: int = 0) -> Dict[str, object]:
+    """Random-init weights of the architecture on the CPU (one generator per matrix,
+    seeded from ``seed``), so the GPU path and the CPU oracle share bits."""
+    def g(i):
+        return torch.Generator().manual_seed(seed * 100003 + i)
+    w: Dict[str, object] = {
+        'embed': (torch.randn(cfg.vocab, cfg.dim, generator=g(1)) * 0.02).to(torch.float16),
+        'final_norm': (1 + 0.1 * torch.randn(cfg.dim, generator=g(2))).to(torch.float16),
+        'lm_head': random_int4_linear(g(3), cfg.dim, cfg.vocab),
+        'layers': [],
+    }
+    for l in range(cfg.n_layers):
+        base = 1000 + 10 * l
+        w['layers'].append({
+            'att_norm': (1 + 0.1 * torch.randn(cfg.dim, generator=g(base))).to(torch.float16),
+            'ffn_norm': (1 + 0.1 * torch.randn(cfg.dim, generator=g(base + 1))).to(torch.float16),
+            'qkv': random_int4_linear(g(base + 2), cfg.dim, 3 * cfg.dim),          # columns: q | k | v
+            'o': random_int4_linear(g(base + 3), cfg.dim, cfg.dim),
+            'gate_up': random_int4_linear(g(base + 4), cfg.dim, 2 * cfg.ffn),      # columns: gate | up
+            'down': random_int4_linear(g(base + 5), cfg.ffn, cfg.dim),
+        })
+    return w
+
+
+def _to_device(obj, dev):
+    if isinstance(obj, torch.Tensor):
+        return obj.to(dev)
+    if isinstance(obj, dict):
+        return {k: _to_device(v, dev) for k, v in obj.items()}
+    if isinstance(obj, list):
+        return [_to_device(v, dev) for v in obj]
+    return obj
+
+
+class LlamaInt4Decoder:
+    """One-token-per-step decoder.  ``step()`` enqueues a whole forward pass on the
+    current stream; ``capture()`` records it once in a HIP graph."""
+
+    def __init__(self, cfg: LlamaConfig, weights: Dict[str, object], device=None):
+        import autort
+        self.autort = autort
+        self.cfg = cfg
+        self.dev = device or autort.device()
+        self.w = _to_device(weights, self.dev)
+        d, H, D = cfg.dim, cfg.n_heads, cfg.head_dim
+        f16 = dict(dtype=torch.float16, device=self.dev)
+        self.key_cache = torch.zeros(cfg.n_layers, cfg.max_seq, d, **f16)
+        self.val_cache = torch.zeros(cfg.n_layers, cfg.max_seq, d, **f16)
+        inv = (1.0 / (cfg.rope_base ** (torch.arange(0, D, 2).float() / D))).to(torch.float16)
+        self.inv_freq = torch.cat([inv, inv]).view(D).to(self.dev)
+        self.att_f = torch.tensor([1 / math.sqrt(D)], dtype=torch.float32, device=self.dev)
+        # device-side step state
+        self.token = torch.zeros(1, dtype=torch.int32, device=self.dev)
+        self.pos = torch.zeros(1, dtype=torch.int32, device=self.dev)
+        # activations (fixed addresses: the step can be recorded in a graph)
+        self.x = torch.empty(d, **f16)
+        self.xb = torch.empty(d, **f16)
+        self.qkv = torch.empty(3 * d, **f16)
+        self.q_rot = torch.empty(H, D, **f16)
+        self.att = torch.empty(H, D, **f16)
+        self.proj = torch.empty(d, **f16)
+        self.gu = torch.empty(2 * cfg.ffn, **f16)
+        self.hb = torch.empty(cfg.ffn, **f16)
+        self.logits = torch.empty(cfg.vocab, **f16)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self._ops()
+
+    def _ops(self):
+        a = self.autort
+        self.gemv = a.export(ir=patterns.W4A16_IR, inputs=patterns.W4A16_INPUTS, name='gemv_w4a16')
+        self.embed = a.export(ir='emb[D] = table[tok[0], D]', inputs=['table=float16[V, D]', 'tok=int32[1]'], name='embed_row_f16')
+        self.add = a.export(ir='acc[N] = acc[N] + delta[N]', inputs=['acc=float16[N]', 'delta=float16[N]'], name='residual_add_f16')
+        self.silu_mul = a.export(
+            ir='hidden[N] = (gu[0, N].to(`float32`) / (1.0 + (0.0 - gu[0, N].to(`float32`)).call(strs.exp)) * gu[1, N].to(`float32`)).to(`float16`)',
+            inputs=['gu=float16[2, N]'], name='silu_mul_f16')
+        self.store_row = a.export(ir='cache[pos[0], D] = row[D]', inputs=['cache=float16[S, D]', 'pos=int32[1]', 'row=float16[D]'],
+                                  name='store_row_f16')
+
+    def _linear(self, x: torch.Tensor, lin: Dict[str, torch.Tensor], out: torch.Tensor):
+        self.gemv(x.view(1, -1), lin['qweight'], lin['scales'], lin['qzeros'], out=out.view(1, -1))
+
+    def step(self) -> torch.Tensor:
+        """Forward pass for (self.token, self.pos); leaves fp16 logits in self.logits."""
+        cfg, ops = self.cfg, self.autort.ops
+        d, H, D = cfg.dim, cfg.n_heads, cfg.head_dim
+        self.embed(self.w['embed'], self.token, out=self.x)
+        for l, lw in enumerate(self.w['layers']):
+            ops.rmsnorm_f16(self.x, None, lw['att_norm'], self.xb, extra=[1.0 / d, cfg.rms_eps])
+            self._linear(self.xb, lw['qkv'], self.qkv)
+            q, k, v = self.qkv[:d], self.qkv[d:2 * d], self.qkv[2 * d:]
+            ops.rotary_f16(q.view(H, 2, -1), self.inv_freq, self.q_rot, extra=[self.pos])
+            ops.rotary_f16(k.view(H, 2, -1), self.inv_freq, self.key_cache[l], extra=[self.pos])
+            self.store_row(self.val_cache[l], self.pos, v)
+            ops.attention_f16(self.q_rot, self.key_cache[l].view(cfg.max_seq, H, D), self.val_cache[l].view(cfg.max_seq, H, D),
+                              self.att_f, self.att, extra=[self.pos])
+            self._linear(self.att.view(-1), lw['o'], self.proj)
+            self.add(self.x, self.proj)
+            ops.rmsnorm_f16(self.x, None, lw['ffn_norm'], self.xb, extra=[1.0 / d, cfg.rms_eps])
+            self._linear(self.xb, lw['gate_up'], self.gu)
+            self.silu_mul(self.gu.view(2, -1), out=self.hb)
+            self._linear(self.hb, lw['down'], self.proj)
+            self.add(self.x, self.proj)
+        ops.rmsnorm_f16(self.x, None, self.w['final_norm'], self.xb, extra=[1.0 / d, cfg.rms_eps])
+        self._linear(self.xb, self.w['lm_head'], self.logits)
+        return self.logits
+
+    def advance(self, prompt: Optional[torch.Tensor] = None):
+        """pos <- pos + 1; token <- prompt[pos] while the prompt lasts, else argmax(logits).
+        All on the device, so it can be part of the recorded graph."""
+        nxt = torch.argmax(self.logits).to(torch.int32).view(1)
+        self.pos.add_(1)
+        if prompt is not None and prompt.numel() > 0:
+            L = prompt.numel()
+            idx = torch.clamp(self.pos, max=L - 1).long()
+            nxt = torch.where(self.pos < L, prompt[idx], nxt)
+        self.token.copy_(nxt)
+
+    def capture(self, greedy: bool = True, prompt: Optional[torch.Tensor] = None):
+        """Record one step (+ advance) in a HIP graph.  ``prompt`` (int32 on the device)
+        is fed token by token before greedy decoding takes over."""
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            self.step()                       # loads every module outside the capture
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                self.step()
+                if greedy:
+                    self.advance(prompt)
+        torch.cuda.synchronize()
+        self.graph = g
+        return g
+
+    def reset(self, token: int = 0, pos: int = 0):
+        self.token.fill_(token)
+        self.pos.fill_(pos)

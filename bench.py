@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-extra', action='store_true', help='headline workload only')
+    ap.add_argument('--no-decode', action='store_true', help='skip the 32-layer decode leg')
+    ap.add_argument('--decode-cpu-steps', type=int, default=2, help='decode steps timed on the CPU oracle (0 = skip)')
     ap.add_argument('--seed', type=int, default=0)
     return ap.parse_args()
 
@@ -120,6 +122,76 @@ def bench_partition(torch, autort, capi, workloads, steps, warmup, seed, n=16_77
             'gbps': 8 * n / sec / 1e9, 'roofline_frac': 8 * n / sec / 1e9 / HBM_PEAK_GBPS, 'melem_per_s': n / sec / 1e6}
 
 
+def bench_decode(torch, autort, capi, seed, prompt_len=128, decode_steps=256, cpu_steps=0):
+    """BASELINE configuration 5: 32-layer Llama-2-7B-shaped int4 decode through autort.ops,
+    batch 1, random-init weights, a 128-token random prompt fed token by token, then
+    256 greedy steps; every step is one replay of the same recorded HIP graph.  The
+    timed region is the 256 greedy steps."""
+    from antares_amd.llama import LlamaConfig, LlamaInt4Decoder, random_weights
+    cfg = LlamaConfig(max_seq=prompt_len + decode_steps)
+    t0 = time.time()
+    weights = random_weights(cfg, seed)
+    gen_s = time.time() - t0
+    dec = LlamaInt4Decoder(cfg, weights)
+    g = torch.Generator().manual_seed(seed + 7)
+    prompt = torch.randint(0, cfg.vocab, (prompt_len,), generator=g, dtype=torch.int64).to(torch.int32)
+    prompt_dev = prompt.to(dec.dev)
+    dec.capture(greedy=True, prompt=prompt_dev)
+    dec.key_cache.zero_()
+    dec.val_cache.zero_()
+    dec.reset(int(prompt[0]), 0)
+    stream = torch.cuda.Stream()
+    tokens = []
+    with torch.cuda.stream(stream):
+        for _ in range(prompt_len - 1):          # positions 0 .. prompt_len-2 consume the prompt
+            dec.graph.replay()
+        stream.synchronize()
+        start, stop = capi.Event(), capi.Event()
+        start.record(stream.cuda_stream)
+        for _ in range(decode_steps):
+            dec.graph.replay()
+        stop.record(stream.cuda_stream)
+        ms = start.elapsed_ms(stop)
+        stream.synchronize()
+    sec_per_token = ms * 1e-3 / decode_steps
+    mean_s = prompt_len - 1 + (decode_steps + 1) / 2.0           # mean attended length over the timed steps
+    kv_bytes = cfg.n_layers * 2 * mean_s * cfg.dim * 2
+    bytes_per_token = cfg.weight_bytes_per_token() + kv_bytes
+    out = {'workload': f'Llama-2-7B-shaped int4 decode, {cfg.n_layers} layers, batch 1, prompt {prompt_len} + {decode_steps} greedy steps',
+           'tokens_per_s': round(1.0 / sec_per_token, 2), 'ms_per_token': round(sec_per_token * 1e3, 4),
+           'weight_bytes_per_token': cfg.weight_bytes_per_token(), 'mean_kv_bytes_per_token': int(kv_bytes),
+           'hbm_gbps': round(bytes_per_token / sec_per_token / 1e9, 1),
+           'roofline_frac': round(bytes_per_token / sec_per_token / 1e9 / HBM_PEAK_GBPS, 4),
+           'final_pos': int(dec.pos.item()), 'last_token': int(dec.token.item()),
+           'prompt': 'fed token by token through the same graph', 'weight_init_s': round(gen_s, 1)}
+    if cpu_steps > 0:
+        out['cpu_baseline'] = cpu_baseline_decode(cfg, weights, int(prompt[0]), cpu_steps)
+    return out
+
+
+def cpu_baseline_decode(cfg, weights, first_token, steps):
+    """The oracle's decode step with its GEMVs on the rank-striding thread pool; `steps`
+    positions from an empty cache (the weight stream, which dominates, does not depend on position)."""
+    import numpy as np
+    from antares_amd.autort import patterns
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule, threads
+    from oracle.llama_ref import LlamaRef
+    mod = CpuModule(parse_program(patterns.W4A16_IR, patterns.W4A16_INPUTS), nranks=256)
+
+    def linear(x, lin):
+        return mod(x=np.ascontiguousarray(x), qweight=lin['qweight'].numpy().view('int8'), scales=lin['scales'].numpy(),
+                   qzeros=lin['qzeros'].numpy().view('int8'))['y']
+    ref = LlamaRef(cfg, weights, linear=linear)
+    tok = first_token
+    t0 = time.perf_counter()
+    for pos in range(steps):
+        tok = int(np.argmax(ref.forward(tok, pos).astype(np.float32)))
+    sec = (time.perf_counter() - t0) / steps
+    return {'value': round(1.0 / sec, 4), 'unit': 'tokens/s', 'cores': threads(), 'kind': 'port',
+            'sample': f'{steps} decode steps of the same 32-layer model from an empty cache, {sec:.2f} s per token'}
+
+
 def cpu_baseline_gemv(workloads, K, N, M, seed, budget_s=15.0):
     """The CPU oracle (loop nests of the reference's CPU backend, same compiler
     flags, rank-striding thread pool) on the headline program."""
@@ -171,6 +243,8 @@ def main():
             r = fn(torch, autort, capi, workloads, args.steps, args.warmup, args.seed)
             extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
         result['extra'] = extra
+    if not args.no_decode:
+        result['decode'] = bench_decode(torch, autort, capi, args.seed, cpu_steps=0 if args.no_cpu else args.decode_cpu_steps)
     if not args.no_cpu:
         result['cpu_baseline'] = cpu_baseline_gemv(workloads, K, N, M, args.seed)
         result['cpu_baseline']['value'] = round(result['cpu_baseline']['value'], 4)

@@ -128,7 +128,8 @@ int art_partition_even_first_i32(const void* in_dev, void* out_dev, long long n,
  *   with t = pos * freq[j]; or, with interleaved != 0, the pairwise form over a
  *   flat vector: (x[2j], x[2j+1]) rotated by pos * freq[j], freq having one entry
  *   per pair of the whole vector.  pos is read from pos_dev (int32 on the device)
- *   when pos_dev != NULL, else taken from `pos`.
+ *   when pos_dev != NULL, else taken from `pos`.  With out_row_stride > 0 the result
+ *   is written at out + pos * out_row_stride elements (a row of a key cache).
  * art_decode_attention: one query per head against a cache of seq_len positions:
  *     a[h,s] = att_f[0] * sum_m q[h,m] k[s,h,m];  p = softmax_s(a);  out[h,m] = sum_s p[h,s] v[s,h,m]
  *   q, out: [heads, 128]; k, v: [seq_len, heads, 128] (dense).  When pos_dev != NULL
@@ -136,7 +137,8 @@ int art_partition_even_first_i32(const void* in_dev, void* out_dev, long long n,
 int art_rmsnorm(const void* x_dev, const void* vsum_dev, const void* w_dev, void* out_dev, int rows, int n, float inv_n,
                 float eps, int x_dtype, int w_dtype, int out_dtype, void* stream);
 int art_rotary(const void* x_dev, const void* freq_dev, void* out_dev, int heads, int head_dim, int interleaved,
-               const void* pos_dev, int pos, int x_dtype, int freq_dtype, int out_dtype, void* stream);
+               const void* pos_dev, int pos, long long out_row_stride, int x_dtype, int freq_dtype, int out_dtype,
+               void* stream);
 int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev, const void* att_f_dev, void* out_dev,
                          int seq_len, int heads, int head_dim, const void* pos_dev, int q_dtype, int kv_dtype, int out_dtype,
                          void* stream);
