@@ -338,11 +338,11 @@ def parse_statement(text: str, tensors: Dict[str, TensorInfo], dim_defaults: Dic
     for k, v in defaults.items():
         dim_defaults.setdefault(k, v)
 
-    ranges: Dict[str, Optional[Dim]] = {}
+    # axes of the where clause come first, in clause order, then the others in order of
+    # appearance (the reference keeps the where clause's dict order and adds the rest)
+    ranges: Dict[str, Optional[Dim]] = dict(ranges_in)
     for ax in find_axis_names(text):
-        ranges[ax] = ranges_in.get(ax)
-    for ax, r in ranges_in.items():
-        ranges.setdefault(ax, r)
+        ranges.setdefault(ax, None)
 
     # legacy scatter spelling  ``out[idx..] =. value``  (reference: lang/einstein_v2.py:309-329)
     set_op = None

@@ -31,6 +31,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 LAYERS = 32
+# HBM bytes per launch of the headline GEMV kernel, from FETCH_SIZE / WRITE_SIZE counters scaled by
+# the copy-kernel calibration (profiles/gemv_w4a16_4096x11008_traffic_pmc.md): 23.80 MB read + 0.81 MB written.
+GEMV_4096x11008_TRAFFIC_BYTES = 24_614_000
 
 
 def parse_args():
@@ -228,7 +231,7 @@ def main():
                    'weights': 'uint8 [K/2,N] two nibbles along K; fp16 scale + 4-bit zero per group',
                    'distinct_weight_sets': head['launches_per_step'], 'timed_through': 'HIP graph replay'},
         'roofline': {'bound': 'hbm', 'achieved': round(head['gbps'], 2), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-                     'frac': round(head['gbps'] / HBM_PEAK_GBPS, 4), 'traffic': None,
+                     'frac': round(head['gbps'] / HBM_PEAK_GBPS, 4), 'traffic': GEMV_4096x11008_TRAFFIC_BYTES,
                      'kernel': 'gemv_w4a16_kernel', 'bytes_per_launch': head['bytes_per_launch'],
                      'us_per_launch': round(head['us_per_launch'], 3)},
     }
