@@ -91,3 +91,28 @@ def _w4a16_handler(op, bound, env, stream) -> bool:
 
 
 register(W4A16_IR, W4A16_INPUTS, _w4a16_handler)
+
+
+# ---------------------------------------------------------------------------
+# fp16 GEMM with fp32 accumulation: C[M,N] = A[M,K] @ B[K,N] (AntaresIR.md:115 with the casts that
+# make the accumulator fp32)
+# ---------------------------------------------------------------------------
+GEMM_F16_IR = """
+  acc[M, N] +=! a[M, K].to(`float32`) * b[K, N].to(`float32`)
+  c[M, N] = acc[M, N].to(`float16`)
+"""
+GEMM_F16_INPUTS = ['a=float16[M:4096, K:4096]', 'b=float16[K:4096, N:4096]']
+
+
+def _gemm_f16_handler(op, bound, env, stream) -> bool:
+    a, b, c = bound['a'], bound['b'], bound['c']
+    M, K = a.shape
+    N = b.shape[1]
+    if M % 256 or N % 256 or K % 64 or a.data_ptr() % 16 or b.data_ptr() % 16 or c.data_ptr() % 16:
+        return False
+    capi.check(capi.lib().art_gemm_f16(c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()), M, N, K,
+                                      c_void_p(stream)))
+    return True
+
+
+register(GEMM_F16_IR, GEMM_F16_INPUTS, _gemm_f16_handler)

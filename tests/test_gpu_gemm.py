@@ -1,0 +1,67 @@
+"""fp16 GEMM on the matrix cores against the oracle (fp32 accumulate, fp16 out; rtol/atol 1e-2)."""
+import numpy as np
+import pytest
+import torch
+
+from antares_amd import workloads
+
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures('oracle_built')]
+FP16_TOL = dict(rtol=1e-2, atol=1e-2)
+
+
+@pytest.fixture(scope='module')
+def gemm():
+    import autort
+    from antares_amd.autort import patterns
+    return autort, autort.export(ir=patterns.GEMM_F16_IR, inputs=patterns.GEMM_F16_INPUTS, name='gemm_f16')
+
+
+def oracle_gemm(a, b):
+    """fp32-accumulated product of the fp16 operands, rounded to fp16 (float64 sums are exact enough to stand in
+    for the fp32 loop nest at these sizes; the oracle's own loop nest is used for the small case below)."""
+    return (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32).astype(np.float16)
+
+
+def test_small_against_loop_nest_oracle(gemm):
+    from antares_amd.autort import patterns
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    autort, op = gemm
+    print('[case] gemm 256x256x64 vs loop nest', flush=True)
+    g = torch.Generator().manual_seed(1)
+    a = (torch.randn(256, 64, generator=g) * 0.5).half()
+    b = (torch.randn(64, 256, generator=g) * 0.5).half()
+    want = CpuModule(parse_program(patterns.GEMM_F16_IR, patterns.GEMM_F16_INPUTS), fast_math=False)(a=a.numpy(), b=b.numpy())['c']
+    got = op(a.to(autort.device()), b.to(autort.device())).cpu().numpy()
+    assert np.allclose(got.astype(np.float32), want.astype(np.float32), **FP16_TOL)
+
+
+@pytest.mark.parametrize('M,N,K', [(256, 256, 64), (256, 512, 128), (512, 256, 192), (1024, 2048, 1024), (4096, 4096, 4096)])
+def test_against_float64_product(gemm, M, N, K):
+    autort, op = gemm
+    print(f'[case] gemm {M}x{N}x{K}', flush=True)
+    g = torch.Generator().manual_seed(M + N + K)
+    a = (torch.randn(M, K, generator=g) * 0.02).half()
+    b = (torch.randn(K, N, generator=g) * 0.02).half()
+    dev = autort.device()
+    got = op(a.to(dev), b.to(dev))
+    assert op.fast_path is not None and got.dtype == torch.float16 and got.shape == (M, N)
+    want = torch.from_numpy(oracle_gemm(a.numpy(), b.numpy()))
+    assert torch.allclose(got.cpu().float(), want.float(), **FP16_TOL)
+    # identity and one-hot structure: pins operand order / transposition
+    if M == N == 256:
+        eye = torch.eye(256, dtype=torch.float16)
+        bb = (torch.randn(256, 256, generator=g)).half()
+        f = autort.export(ir=op.ir, inputs=['a=float16[M:256, K:256]', 'b=float16[K:256, N:256]'], name='gemm_f16_sq')
+        assert torch.equal(f(eye.to(dev), bb.to(dev)).cpu(), bb)
+        assert torch.equal(f(bb.to(dev), eye.to(dev)).cpu(), bb)
+
+
+def test_shapes_outside_the_tile_grid_use_the_generic_lowering(gemm):
+    autort, op = gemm
+    print('[case] gemm 96x80x40 (generic lowering)', flush=True)
+    g = torch.Generator().manual_seed(5)
+    a = (torch.randn(96, 40, generator=g) * 0.1).half()
+    b = (torch.randn(40, 80, generator=g) * 0.1).half()
+    got = op(a.to(autort.device()), b.to(autort.device())).cpu().numpy()
+    assert np.allclose(got.astype(np.float32), oracle_gemm(a.numpy(), b.numpy()).astype(np.float32), **FP16_TOL)
