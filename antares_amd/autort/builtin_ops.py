@@ -184,3 +184,89 @@ builtin('rotate_f32')(lambda: Rotary('rotate_f32', True))
 builtin('rotate_f16')(lambda: Rotary('rotate_f16', True))
 builtin('attention_f32')(lambda: DecodeAttention('attention_f32'))
 builtin('attention_f16')(lambda: DecodeAttention('attention_f16'))
+
+
+class GemvW4Fused:
+    """``gemv_w4a16_fused(x[K], qweight, scales, qzeros, out[N], norm_weight=None, residual=None, eps=1e-5)``:
+    the packed int4 GEMV with an RMSNorm of its input and/or a residual add of its output folded in
+    (the operators around every projection of the decode step, samples/05_llama2_7b_int4.py:150-173)."""
+    name = 'gemv_w4a16_fused'
+
+    def __call__(self, x, qweight, scales, qzeros, out=None, norm_weight=None, residual=None, eps=RMS_EPS, swiglu=False,
+                 extra=None):
+        """``swiglu=True``: ``x`` holds gate | up (2*K values) and the product is taken with silu(gate) * up."""
+        K, N = qweight.shape[0] * 2, qweight.shape[1]
+        if x.numel() != (2 * K if swiglu else K):
+            raise ValueError('gemv_w4a16_fused: x has the wrong length')
+        if x.dtype != torch.float16 or scales.dtype != torch.float16:
+            raise TypeError('gemv_w4a16_fused: x and scales must be float16')
+        if qweight.shape[0] * 2 != K or scales.shape != (K // 128, N) or qzeros.shape != (K // 128, N // 2):
+            raise ValueError('gemv_w4a16_fused: operand shapes do not match K, N')
+        if out is None:
+            out = torch.empty(N, dtype=torch.float16, device=x.device)
+        tensors = [x, qweight, scales, qzeros, out]
+        for t, what in ((norm_weight, 'norm_weight'), (residual, 'residual')):
+            if t is not None:
+                if t.dtype != torch.float16 or t.numel() != (K if what == 'norm_weight' else N):
+                    raise TypeError(f'gemv_w4a16_fused: {what} must be float16 of matching length')
+                tensors.append(t)
+        _require_cuda(*tensors)
+        capi.check(capi.lib().art_gemv_w4a16_fused(
+            c_void_p(x.data_ptr()), c_void_p(qweight.data_ptr()), c_void_p(scales.data_ptr()), c_void_p(qzeros.data_ptr()),
+            c_void_p(out.data_ptr()), K, N, c_void_p(norm_weight.data_ptr() if norm_weight is not None else 0), float(eps),
+            c_void_p(residual.data_ptr() if residual is not None else 0), int(bool(swiglu)), c_void_p(current_stream_handle())))
+        return out
+
+
+class AttentionRope:
+    """``attention_rope_f16(qkv[3*H*D], inv_freq[D], key_cache[S,H*D], val_cache[S,H*D], att_f[1], out[H,D], extra=[pos_tensor])``:
+    rotary embedding of q and k, both cache writes and the attention over rows 0..pos, one launch per layer."""
+    name = 'attention_rope_f16'
+
+    def __call__(self, qkv, inv_freq, key_cache, val_cache, att_f, out, extra=None):
+        heads, head_dim = out.shape
+        if qkv.numel() != 3 * heads * head_dim or key_cache.shape[-1] != heads * head_dim or val_cache.shape != key_cache.shape:
+            raise ValueError('attention_rope_f16: shapes do not fit together')
+        for t in (qkv, inv_freq, key_cache, val_cache, out):
+            if t.dtype != torch.float16:
+                raise TypeError('attention_rope_f16: tensors must be float16')
+        if att_f.dtype != torch.float32 or att_f.numel() != 1:
+            raise TypeError('attention_rope_f16: att_f must be a 1-element float32 tensor')
+        _require_cuda(qkv, inv_freq, key_cache, val_cache, att_f, out)
+        pos_dev, _ = _pos_args(extra, self.name)
+        if not pos_dev.value:
+            raise TypeError('attention_rope_f16: extra=[pos] must be a 1-element int32 GPU tensor')
+        capi.check(capi.lib().art_decode_attention_rope(c_void_p(qkv.data_ptr()), c_void_p(inv_freq.data_ptr()),
+                                                       c_void_p(key_cache.data_ptr()), c_void_p(val_cache.data_ptr()),
+                                                       c_void_p(att_f.data_ptr()), c_void_p(out.data_ptr()), heads, head_dim, pos_dev,
+                                                       c_void_p(current_stream_handle())))
+        return out
+
+
+class RopeQkvStore:
+    """``rope_qkv_store_f16(qkv[3*H*D], inv_freq[D], q_out[H,D], key_cache[S,H*D], val_cache[S,H*D], extra=[pos_tensor])``:
+    rotary embedding of q and k (k straight into its cache row) and the copy of v into its cache row, one launch."""
+
+    def __init__(self, name):
+        self.name = name
+
+    def __call__(self, qkv, inv_freq, q_out, key_cache, val_cache, extra=None):
+        heads, head_dim = q_out.shape
+        if qkv.numel() != 3 * heads * head_dim or key_cache.shape[-1] != heads * head_dim or val_cache.shape != key_cache.shape:
+            raise ValueError(f'{self.name}: shapes do not fit together')
+        if not (qkv.dtype == q_out.dtype == key_cache.dtype == val_cache.dtype):
+            raise TypeError(f'{self.name}: qkv, q_out and the caches must share one dtype')
+        _require_cuda(qkv, inv_freq, q_out, key_cache, val_cache)
+        pos_dev, _ = _pos_args(extra, self.name)
+        if not pos_dev.value:
+            raise TypeError(f'{self.name}: extra=[pos] must be a 1-element int32 GPU tensor')
+        capi.check(capi.lib().art_rope_qkv_store(c_void_p(qkv.data_ptr()), c_void_p(inv_freq.data_ptr()), c_void_p(q_out.data_ptr()),
+                                                c_void_p(key_cache.data_ptr()), c_void_p(val_cache.data_ptr()), heads, head_dim,
+                                                pos_dev, _dt(qkv, 'qkv'), _dt(inv_freq, 'inv_freq'), c_void_p(current_stream_handle())))
+        return q_out
+
+
+builtin('gemv_w4a16_fused')(lambda: GemvW4Fused())
+builtin('attention_rope_f16')(lambda: AttentionRope())
+builtin('rope_qkv_store_f16')(lambda: RopeQkvStore('rope_qkv_store_f16'))
+builtin('rope_qkv_store_f32')(lambda: RopeQkvStore('rope_qkv_store_f32'))

@@ -101,33 +101,56 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
   const int b_k = (lane >> 5) * 8 + (s >> 2);               // + kk*16 + r*4
   const int b_n = wn * 128 + ((lane & 31) >> 4) * 16 + (s & 3) * 4;   // + j*32
 
+  auto load_frags = [&](h8 (&af)[4], h8 (&bf)[4], const _Float16* as, const _Float16* bs, int kk) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const h8*>(as + (a_row + i * 32) * A_LD + kk * 16 + a_k);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const _Float16* p = bs + (kk * 16 + b_k) * B_LD + b_n + j * 32;
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * B_LD));
+      const h4 l4 = __builtin_bit_cast(h4, lo), h4v = __builtin_bit_cast(h4, hi);
+      bf[j] = h8{l4[0], l4[1], l4[2], l4[3], h4v[0], h4v[1], h4v[2], h4v[3]};
+    }
+  };
+  auto mfma_all = [&](const h8 (&af)[4], const h8 (&bf)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+  };
+
   const int T = K / BK;
   load_tiles(0);
   store_tiles(0);
   __syncthreads();
+  h8 af0[4], bf0[4], af1[4], bf1[4];
   for (int t = 0; t < T; ++t) {
     const int buf = t & 1;
-    if (t + 1 < T) load_tiles(t + 1);
     const _Float16* as = As + buf * A_TILE;
     const _Float16* bs = Bs + buf * B_TILE;
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      h8 af[4], bf[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const h8*>(as + (a_row + i * 32) * A_LD + kk * 16 + a_k);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const _Float16* p = bs + (kk * 16 + b_k) * B_LD + b_n + j * 32;
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * B_LD));
-        const h4 l4 = __builtin_bit_cast(h4, lo), h4v = __builtin_bit_cast(h4, hi);
-        bf[j] = h8{l4[0], l4[1], l4[2], l4[3], h4v[0], h4v[1], h4v[2], h4v[3]};
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-    }
+    // The scheduler is told not to move anything across these fences: without them it sinks every
+    // operand read next to its first use and the matrix cores wait for LDS sixteen times per tile.
+#define ART_FENCE() __builtin_amdgcn_sched_barrier(0)
+    load_frags(af0, bf0, as, bs, 0);
+    ART_FENCE();
+    if (t + 1 < T) load_tiles(t + 1);
+    ART_FENCE();
+    load_frags(af1, bf1, as, bs, 1);     // operands of k-step kk+1 are requested before the MFMAs of k-step kk
+    ART_FENCE();
+    mfma_all(af0, bf0);
+    ART_FENCE();
+    load_frags(af0, bf0, as, bs, 2);
+    ART_FENCE();
+    mfma_all(af1, bf1);
+    ART_FENCE();
+    load_frags(af1, bf1, as, bs, 3);
+    ART_FENCE();
+    mfma_all(af0, bf0);
+    ART_FENCE();
+    mfma_all(af1, bf1);
+    ART_FENCE();
+#undef ART_FENCE
     if (t + 1 < T) store_tiles(buf ^ 1);
     __syncthreads();
   }

@@ -95,13 +95,39 @@ __device__ __forceinline__ float sum_k_lanes_of_wave(float v) {
   return v;
 }
 
+// sum over the 64 lanes of a wavefront; every lane gets the result
+__device__ __forceinline__ float wave_sum_all(float v) {
+#define ART_DPP_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false))
+  ART_DPP_ADD(0xB1);    // quad_perm [1,0,3,2]
+  ART_DPP_ADD(0x4E);    // quad_perm [2,3,0,1]
+  ART_DPP_ADD(0x141);   // row_half_mirror
+  ART_DPP_ADD(0x140);   // row_mirror
+#undef ART_DPP_ADD
+  const int b = __builtin_bit_cast(int, v);
+  return (__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16))) +
+         (__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48)));
+}
+
+// Optional work fused around the product (decode, M = 1):
+//   norm_w   != NULL : x is replaced by RMSNorm(x) = fp16(x * rsqrt(sum(x^2) * inv_n + eps) * norm_w) before the product;
+//   residual != NULL : y = fp16(fp16(product) + residual), i.e. the residual add that follows the projection.
+//   gate_up  != NULL : x is not read; x[k] = fp16(silu(gate_up[k]) * gate_up[K + k]) (SwiGLU, line :171 of the sample).
+struct Fused {
+  const _Float16* norm_w;
+  const _Float16* residual;
+  const _Float16* gate_up;
+  float inv_n, eps;
+};
+
 template <int M>
 __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight, const _Float16* __restrict__ scales,
     const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y, int K, int N, int splits,
-    unsigned long long* __restrict__ slots, Magic magic) {
+    unsigned long long* __restrict__ slots, Magic magic, Fused fused) {
   __shared__ __align__(16) float red[M][KL][CT];        // 16 KiB per row of x
   __shared__ float aux[M][4][2];                        // per wavefront (= group): magic-number term, sum of x
+  __shared__ float s_ss[4];
+  __shared__ __align__(16) unsigned int s_x[KL][CL];    // SwiGLU input, one fp16 pair per lane
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cl = tid % CL, kl = tid / CL;
@@ -115,7 +141,30 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
   const int r0c = k_ok ? r0 : 0;
   const int n0c = (n0 < N) ? n0 : 0;
 
-  // ---- every global load of this lane goes out first
+  // ---- fused RMSNorm, part 1: the loads for the sum of squares go out BEFORE the weight loads.  Loads
+  // return in order, so these can be consumed (and the block-wide reduction done) while the weights are
+  // still in flight; issued after the weights they would wait for the whole stream.
+  const bool norm = (M == 1) && (fused.norm_w != nullptr);
+  u32x4 sq[2];
+  if (norm) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c = tid + i * kThreads;
+      sq[i] = (c < (K >> 3)) ? reinterpret_cast<const u32x4*>(x)[c] : u32x4{0, 0, 0, 0};
+    }
+  }
+
+  // ---- fused SwiGLU, part 1: the column lanes of a k lane share the same 16 values of x, so each
+  // computes one pair; its two loads also go out ahead of the weight stream.
+  const bool swiglu = (M == 1) && (fused.gate_up != nullptr);
+  unsigned int gpair = 0, upair = 0;
+  if (swiglu) {
+    const int k = 2 * r0c + 2 * cl;
+    gpair = *reinterpret_cast<const unsigned int*>(fused.gate_up + k);
+    upair = *reinterpret_cast<const unsigned int*>(fused.gate_up + K + k);
+  }
+
+  // ---- every other global load of this lane
   u32x4 w[R];
   {
     const unsigned char* wp = qweight + (size_t)r0c * N + n0c;
@@ -125,9 +174,21 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
   u32x4 xv[M][2];                                         // 16 halves of x per row of x
 #pragma unroll
   for (int m = 0; m < M; ++m) {
+    if (swiglu) continue;
     const u32x4* xp = reinterpret_cast<const u32x4*>(x + (size_t)m * K + 2 * r0c);
     xv[m][0] = xp[0];
     xv[m][1] = xp[1];
+  }
+  if (swiglu) {       // part 2: pair -> LDS -> all 16 values of the k lane (same wavefront: no block barrier needed)
+    const half2_t g = as_h2(gpair), u = as_h2(upair);
+    const float g0f = (float)g.x, g1f = (float)g.y;
+    const half2_t o = {(_Float16)(g0f / (1.0f + expf(0.0f - g0f)) * (float)u.x), (_Float16)(g1f / (1.0f + expf(0.0f - g1f)) * (float)u.y)};
+    s_x[kl][cl] = __builtin_bit_cast(unsigned int, o);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    xv[0][0] = *reinterpret_cast<const u32x4*>(&s_x[kl][0]);
+    xv[0][1] = *reinterpret_cast<const u32x4*>(&s_x[kl][4]);
   }
   // column owners (tid < 128) fetch scale and zero point of their column for the four groups of the block
   const int col = tile * CT + tid;
@@ -148,6 +209,49 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
       xv[m][0] = u32x4{0, 0, 0, 0};
       xv[m][1] = u32x4{0, 0, 0, 0};
     }
+  }
+
+  // ---- fused RMSNorm, part 2 (while the weight loads are in flight): sum of squares over all of x.
+  // Every block recomputes it from the 2*K bytes of x (served by L2) rather than waiting for another kernel.
+  if (norm) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const unsigned int wds[4] = {sq[i][0], sq[i][1], sq[i][2], sq[i][3]};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const half2_t h = as_h2(wds[j]);
+        ss = fmaf((float)h.x, (float)h.x, ss);
+        ss = fmaf((float)h.y, (float)h.y, ss);
+      }
+    }
+    for (int c = tid + 2 * kThreads; c < (K >> 3); c += kThreads) {      // K > 4096
+      const u32x4 v = reinterpret_cast<const u32x4*>(x)[c];
+      const unsigned int wds[4] = {v[0], v[1], v[2], v[3]};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const half2_t h = as_h2(wds[j]);
+        ss = fmaf((float)h.x, (float)h.x, ss);
+        ss = fmaf((float)h.y, (float)h.y, ss);
+      }
+    }
+    ss = wave_sum_all(ss);
+    if (lane == 0) s_ss[wave] = ss;
+    __syncthreads();
+    const float r = 1.0f / sqrtf(((s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3])) * fused.inv_n + fused.eps);
+    const u32x4* np = reinterpret_cast<const u32x4*>(fused.norm_w + 2 * r0c);
+    const u32x4 n0v = np[0], n1v = np[1];
+    const unsigned int nw[8] = {n0v[0], n0v[1], n0v[2], n0v[3], n1v[0], n1v[1], n1v[2], n1v[3]};
+    const unsigned int xw[8] = {xv[0][0][0], xv[0][0][1], xv[0][0][2], xv[0][0][3], xv[0][1][0], xv[0][1][1], xv[0][1][2], xv[0][1][3]};
+    unsigned int out[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const half2_t xh = as_h2(xw[i]), wh = as_h2(nw[i]);
+      const half2_t o = {(_Float16)((float)xh.x * r * (float)wh.x), (_Float16)((float)xh.y * r * (float)wh.y)};
+      out[i] = __builtin_bit_cast(unsigned int, o);
+    }
+    xv[0][0] = u32x4{out[0], out[1], out[2], out[3]};
+    xv[0][1] = u32x4{out[4], out[5], out[6], out[7]};
   }
 
   // ---- multiply-accumulate
@@ -203,7 +307,9 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
       r += (float)sc[g] * (a - aux[m][g][0] - z * aux[m][g][1]);
     }
     if (splits == 1) {
-      y[(size_t)m * N + col] = (_Float16)r;
+      _Float16 o = (_Float16)r;
+      if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)fused.residual[col]);
+      y[(size_t)m * N + col] = o;
       continue;
     }
     // one returning atomic: [arrival count : 8][2^-30 fixed-point sum : 56]
@@ -212,14 +318,17 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     const long long old = (long long)__hip_atomic_fetch_add(slot, (unsigned long long)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (((old + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
       const long long total = old + mine - ((long long)splits << 56);
-      y[(size_t)m * N + col] = (_Float16)((float)total * (1.f / kFix));
+ _Float16 o = (_Float16)((float)total * (1.f / kFix));
+      if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)fused.residual[col]);
+      y[(size_t)m * N + col] = o;
       *slot = 0ull;                     // ready for the next launch (stream order makes this visible)
     }
   }
 }
 
 template <int M>
-int launch(const void* x, const void* qw, const void* sc, const void* qz, void* y, int K, int N, hipStream_t stream) {
+int launch(const void* x, const void* qw, const void* sc, const void* qz, void* y, int K, int N, hipStream_t stream,
+           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f}) {
   const int rows = K / 2;
   const int tiles = (N + CT - 1) / CT;
   const int splits = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
@@ -230,7 +339,7 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
   unsigned long long* slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(ws.base) + art::kSlotOffset);
   gemv_w4a16_kernel<M><<<dim3(tiles, splits), dim3(kThreads), 0, stream>>>(
       (const _Float16*)x, (const unsigned char*)qw, (const _Float16*)sc, (const unsigned char*)qz, (_Float16*)y, K, N,
-      splits, slots, Magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u});
+      splits, slots, Magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u}, fused);
   ART_LAUNCH_CHECK();
   return 0;
 }
@@ -256,4 +365,18 @@ extern "C" int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const 
     m += step;
   }
   return 0;
+}
+
+extern "C" int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                                    void* y_dev, int K, int N, const void* norm_weight_dev, float eps, const void* residual_dev,
+                                    int swiglu_input, void* stream) {
+  ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16_fused: null pointer");
+  ART_REQUIRE(!(swiglu_input && norm_weight_dev), "art_gemv_w4a16_fused: SwiGLU input and RMSNorm cannot be combined");
+  ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_fused: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
+  ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0 && ((uintptr_t)norm_weight_dev % 16) == 0,
+              "art_gemv_w4a16_fused: x, qweight and the norm weight must be 16-byte aligned");
+  ART_REQUIRE(x_dev != y_dev || norm_weight_dev == nullptr, "art_gemv_w4a16_fused: y may alias the residual, not a normalised x");
+  Fused f{(const _Float16*)norm_weight_dev, (const _Float16*)residual_dev, swiglu_input ? (const _Float16*)x_dev : nullptr,
+          1.0f / (float)K, eps};
+  return launch<1>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, (hipStream_t)stream, f);
 }

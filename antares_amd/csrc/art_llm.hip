@@ -133,43 +133,84 @@ template <> struct Row16<float> {
 constexpr int kAttThreads = 256;
 constexpr int kAttGroups = kAttThreads / 8;   // 32 position groups per block
 
-template <class QT, class KT, class OT>
-__global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __restrict__ q, const KT* __restrict__ k,
-                                                                 const KT* __restrict__ v, const float* __restrict__ att_f,
-                                                                 OT* __restrict__ out, int heads, const int* __restrict__ len_dev,
-                                                                 int len_host) {
-  constexpr int D = 128;
+// ROPE = true: the block first rotates its head's q and k (rotate-half form) from the token's q|k|v vector,
+// writes k and v into cache row `pos` and attends over rows 0..pos; q_or_qkv then points at q|k|v.
+template <class QT, class KT, class OT, bool ROPE>
+__global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __restrict__ q_or_qkv, KT* __restrict__ k, KT* __restrict__ v,
+                                                                 const float* __restrict__ att_f, OT* __restrict__ out, int heads,
+                                                                 const int* __restrict__ len_dev, int len_host,
+                                                                 const _Float16* __restrict__ inv_freq) {
+  constexpr int D = 128, U = 4;
   __shared__ float s_m[kAttGroups], s_l[kAttGroups];
   __shared__ float s_acc[kAttGroups][D];
+  __shared__ float s_q[D];
   const int S = len_dev ? (*len_dev + 1) : len_host;     // device form carries the position, length = pos + 1
   const int h = blockIdx.x, tid = threadIdx.x;
   const int sub = tid & 7, group = tid >> 3;
   const float scale = att_f[0];
+  const size_t row = (size_t)heads * D;
   float qf[16];
+  if (ROPE) {
+    const int pos = S - 1, dim = heads * D;
+    if (tid < 128) {                                      // 64 pairs of q, 64 pairs of k
+      const bool is_k = tid >= 64;
+      const int j = tid & 63;
+      const QT* src = q_or_qkv + (is_k ? dim : 0) + (size_t)h * D;
+      float sn, cs;
+      sincosf((float)pos * (float)inv_freq[j], &sn, &cs);
+      const float xa = ld(src, j), xb = ld(src, j + 64);
+      const float ra = xa * cs - xb * sn, rb = xb * cs + xa * sn;
+      if (is_k) {
+        st(k + (size_t)pos * row + (size_t)h * D, j, ra);
+        st(k + (size_t)pos * row + (size_t)h * D, j + 64, rb);
+      } else {                                            // q goes through the output dtype like the separate operator
+        s_q[j] = (float)(QT)ra;
+        s_q[j + 64] = (float)(QT)rb;
+      }
+    } else {
+      const int e = tid - 128;
+      v[(size_t)pos * row + (size_t)h * D + e] = (KT)q_or_qkv[2 * (size_t)dim + (size_t)h * D + e];
+    }
+    __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 16; ++i) qf[i] = ld(q, (size_t)h * D + sub * 16 + i) * scale;
+    for (int i = 0; i < 16; ++i) qf[i] = s_q[sub * 16 + i] * scale;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) qf[i] = ld(q_or_qkv, (size_t)h * D + sub * 16 + i) * scale;
+  }
 
   float m = -INFINITY, l = 0.f, acc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-  const size_t row = (size_t)heads * D;
-  for (int s = group; s < S; s += kAttGroups) {
-    float kf[16], vf[16];
-    Row16<KT>::load(k + (size_t)s * row + (size_t)h * D + sub * 16, kf);
-    Row16<KT>::load(v + (size_t)s * row + (size_t)h * D + sub * 16, vf);
-    float d = 0.f;
+  // U positions per group are requested before the first is used: S/128 round trips instead of S/32
+  for (int s0 = group; s0 < S; s0 += kAttGroups * U) {
+    float kf[U][16], vf[U][16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kf[i], d);
-    // sum over the 8 lanes of the group (xor 1, xor 2 inside a quad, then the neighbouring quad)
-    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xf, 0xf, false));
-    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xf, 0xf, false));
-    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xf, 0xf, false));
-    const float mn = fmaxf(m, d);
-    const float corr = __expf(m - mn), p = __expf(d - mn);
-    l = l * corr + p;
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * kAttGroups;
+      const int sc = s < S ? s : s0;                      // past the end: re-read a valid row, weight 0 below
+      Row16<KT>::load(k + (size_t)sc * row + (size_t)h * D + sub * 16, kf[u]);
+      Row16<KT>::load(v + (size_t)sc * row + (size_t)h * D + sub * 16, vf[u]);
+    }
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * vf[i]);
-    m = mn;
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * kAttGroups;
+      float d = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kf[u][i], d);
+      // sum over the 8 lanes of the group (xor 1, xor 2 inside a quad, then the neighbouring quad)
+      d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xf, 0xf, false));
+      d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xf, 0xf, false));
+      d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xf, 0xf, false));
+      if (s < S) {
+        const float mn = fmaxf(m, d);
+        const float corr = __expf(m - mn), p = __expf(d - mn);
+        l = l * corr + p;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * vf[u][i]);
+        m = mn;
+      }
+    }
   }
   if (sub == 0) { s_m[group] = m; s_l[group] = l; }
 #pragma unroll
@@ -187,6 +228,38 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
       o = fmaf(s_acc[g][tid], wgt, o);
     }
     st(out, (size_t)h * D + tid, o / ll);
+  }
+}
+
+}  // namespace
+
+namespace {
+
+// q | k | v of one token (3 * heads * head_dim values) -> rotated q, rotated k into its cache row, v into its cache row.
+// One launch instead of two rotary launches and a row copy; the position comes from the device.
+template <class T, class FT>
+__global__ __launch_bounds__(256) void rope_qkv_store_kernel(const T* __restrict__ qkv, const FT* __restrict__ freq, T* __restrict__ q_out,
+                                                              T* __restrict__ key_cache, T* __restrict__ val_cache, int heads, int half,
+                                                              const int* __restrict__ pos_dev) {
+  const int pos = *pos_dev;
+  const int dim = heads * half * 2;
+  const int pairs = heads * half;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < 2 * pairs) {                       // q pairs, then k pairs
+    const bool is_k = i >= pairs;
+    const int p = is_k ? i - pairs : i;
+    const int h = p / half, j = p % half;
+    const T* src = qkv + (is_k ? dim : 0);
+    T* dst = is_k ? key_cache + (size_t)pos * dim : q_out;
+    float s, c;
+    sincosf((float)pos * ld(freq, j), &s, &c);
+    const size_t a = (size_t)h * 2 * half + j, b = a + half;
+    const float xa = ld(src, a), xb = ld(src, b);
+    st(dst, a, xa * c - xb * s);
+    st(dst, b, xb * c + xa * s);
+  } else if (i < 2 * pairs + dim) {          // v row copy
+    const int e = i - 2 * pairs;
+    val_cache[(size_t)pos * dim + e] = qkv[2 * (size_t)dim + e];
   }
 }
 
@@ -254,10 +327,42 @@ extern "C" int art_decode_attention(const void* q_dev, const void* k_dev, const 
   hipStream_t st = (hipStream_t)stream;
   const int* pd = (const int*)pos_dev;
   const float* af = (const float*)att_f_dev;
-#define ART_ATT(QT, KT) attention_kernel<QT, KT, QT><<<dim3(heads), dim3(kAttThreads), 0, st>>>((const QT*)q_dev, (const KT*)k_dev, (const KT*)v_dev, af, (QT*)out_dev, heads, pd, seq_len)
+#define ART_ATT(QT, KT) attention_kernel<QT, KT, QT, false><<<dim3(heads), dim3(kAttThreads), 0, st>>>((const QT*)q_dev, (KT*)k_dev, (KT*)v_dev, af, (QT*)out_dev, heads, pd, seq_len, nullptr)
   if (q_dtype == 0) { if (kv_dtype == 0) ART_ATT(float, float); else ART_ATT(float, _Float16); }
   else { if (kv_dtype == 0) ART_ATT(_Float16, float); else ART_ATT(_Float16, _Float16); }
 #undef ART_ATT
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, void* q_out_dev, void* key_cache_dev, void* val_cache_dev,
+                                  int heads, int head_dim, const void* pos_dev, int dtype, int freq_dtype, void* stream) {
+  ART_REQUIRE(qkv_dev && freq_dev && q_out_dev && key_cache_dev && val_cache_dev && pos_dev, "art_rope_qkv_store: null pointer");
+  ART_REQUIRE(heads >= 1 && head_dim >= 2 && head_dim % 2 == 0, "art_rope_qkv_store: bad shape");
+  ART_REQUIRE(ART_DT_OK(dtype) && ART_DT_OK(freq_dtype), "art_rope_qkv_store: dtype codes are 0 (f32) / 1 (f16)");
+  const int half = head_dim / 2, dim = heads * head_dim;
+  const dim3 grid((2 * heads * half + dim + 255) / 256), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const int* pd = (const int*)pos_dev;
+#define ART_RQS(T, FT) rope_qkv_store_kernel<T, FT><<<grid, block, 0, st>>>((const T*)qkv_dev, (const FT*)freq_dev, (T*)q_out_dev, (T*)key_cache_dev, (T*)val_cache_dev, heads, half, pd)
+  if (dtype == 0) { if (freq_dtype == 0) ART_RQS(float, float); else ART_RQS(float, _Float16); }
+  else { if (freq_dtype == 0) ART_RQS(_Float16, float); else ART_RQS(_Float16, _Float16); }
+#undef ART_RQS
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int art_decode_attention_rope(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev, void* val_cache_dev,
+                                         const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev,
+                                         void* stream) {
+  ART_REQUIRE(qkv_dev && inv_freq_dev && key_cache_dev && val_cache_dev && att_f_dev && out_dev && pos_dev,
+              "art_decode_attention_rope: null pointer");
+  ART_REQUIRE(head_dim == 128 && heads >= 1, "art_decode_attention_rope: head_dim must be 128 (got %d)", head_dim);
+  ART_REQUIRE(((uintptr_t)key_cache_dev % 16) == 0 && ((uintptr_t)val_cache_dev % 16) == 0,
+              "art_decode_attention_rope: caches must be 16-byte aligned");
+  attention_kernel<_Float16, _Float16, _Float16, true><<<dim3(heads), dim3(kAttThreads), 0, (hipStream_t)stream>>>(
+      (const _Float16*)qkv_dev, (_Float16*)key_cache_dev, (_Float16*)val_cache_dev, (const float*)att_f_dev, (_Float16*)out_dev,
+      heads, (const int*)pos_dev, 0, (const _Float16*)inv_freq_dev);
   ART_LAUNCH_CHECK();
   return 0;
 }

@@ -94,8 +94,9 @@ class LlamaInt4Decoder:
     """One-token-per-step decoder.  ``step()`` enqueues a whole forward pass on the
     current stream; ``capture()`` records it once in a HIP graph."""
 
-    def __init__(self, cfg: LlamaConfig, weights: Dict[str, object], device=None):
+    def __init__(self, cfg: LlamaConfig, weights: Dict[str, object], device=None, fused: bool = True):
         import autort
+        self.fused = fused
         self.autort = autort
         self.cfg = cfg
         self.dev = device or autort.device()
@@ -139,6 +140,29 @@ class LlamaInt4Decoder:
 
     def step(self) -> torch.Tensor:
         """Forward pass for (self.token, self.pos); leaves fp16 logits in self.logits."""
+        return self.step_fused() if self.fused else self.step_plain()
+
+    def step_fused(self) -> torch.Tensor:
+        """Five launches per layer: RMSNorm, SwiGLU and the residual adds ride inside the projections; rotary of
+        q and k and both cache writes ride inside the attention.  Same roundings as ``step_plain``."""
+        cfg, ops = self.cfg, self.autort.ops
+        H, D = cfg.n_heads, cfg.head_dim
+        gemv = ops.gemv_w4a16_fused
+        self.embed(self.w['embed'], self.token, out=self.x)
+        for l, lw in enumerate(self.w['layers']):
+            a, o, gu, dn = lw['qkv'], lw['o'], lw['gate_up'], lw['down']
+            gemv(self.x, a['qweight'], a['scales'], a['qzeros'], self.qkv, norm_weight=lw['att_norm'], eps=cfg.rms_eps)
+            ops.attention_rope_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f, self.att,
+                                   extra=[self.pos])
+            gemv(self.att.view(-1), o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
+            gemv(self.x, gu['qweight'], gu['scales'], gu['qzeros'], self.gu, norm_weight=lw['ffn_norm'], eps=cfg.rms_eps)
+            gemv(self.gu, dn['qweight'], dn['scales'], dn['qzeros'], self.x, residual=self.x, swiglu=True)
+        h = self.w['lm_head']
+        gemv(self.x, h['qweight'], h['scales'], h['qzeros'], self.logits, norm_weight=self.w['final_norm'], eps=cfg.rms_eps)
+        return self.logits
+
+    def step_plain(self) -> torch.Tensor:
+        """One launch per operator of the sample's forward pass (thirteen per layer)."""
         cfg, ops = self.cfg, self.autort.ops
         d, H, D = cfg.dim, cfg.n_heads, cfg.head_dim
         self.embed(self.w['embed'], self.token, out=self.x)

@@ -48,6 +48,10 @@ _SIGNATURES = {
     'art_gemv_w4a16': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_gemv_gptq': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     'art_partition_even_first_i32': (c_int, [c_void_p, c_void_p, c_longlong, c_void_p]),
+    'art_gemv_w4a16_fused': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p,
+                                     c_int, c_void_p]),
+    'art_decode_attention_rope': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
+    'art_rope_qkv_store': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p]),
     'art_gemm_f16': (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_rmsnorm': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_float, c_int, c_int, c_int, c_void_p]),
     'art_rotary': (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_longlong, c_int, c_int, c_int,

@@ -101,6 +101,18 @@ int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* strea
 int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                    void* y_dev, int M, int K, int N, void* stream);
 
+/* The same GEMV (M = 1) with the operators that surround a projection in the
+ * decode step of samples/05_llama2_7b_int4.py:146-177 folded in:
+ *   norm_weight_dev != NULL: x is first replaced by
+ *       fp16(x * rsqrt(sum(x^2)/K + eps) * norm_weight)                     (lines :128-131,:150,:169)
+ *   residual_dev != NULL:    y = fp16(fp16(product) + residual)             (lines :168,:173)
+ *   swiglu_input != 0:       x_dev holds gate | up (2*K values) and the product is taken with
+ *       fp16(silu(gate[k]) * up[k])                                         (line :171)
+ * y may alias residual.  Same roundings as the separate operators. */
+int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                         void* y_dev, int K, int N, const void* norm_weight_dev, float eps, const void* residual_dev,
+                         int swiglu_input, void* stream);
+
 /* The reference's own weight format (samples/05_llama2_7b_int4.py:135-139):
  * qweight int32 [K/8,N], eight nibbles per word along K (least significant
  * first), zero point fixed at 8, scales fp32 or fp16 [K/128,N], x and y fp32
@@ -145,6 +157,15 @@ int art_rmsnorm(const void* x_dev, const void* vsum_dev, const void* w_dev, void
 int art_rotary(const void* x_dev, const void* freq_dev, void* out_dev, int heads, int head_dim, int interleaved,
                const void* pos_dev, int pos, long long out_row_stride, int x_dtype, int freq_dtype, int out_dtype,
                void* stream);
+/* One token's q | k | v (3 * heads * head_dim values): q rotated into q_out, k rotated into row
+ * *pos_dev of key_cache, v copied into row *pos_dev of val_cache (caches: [positions, heads*head_dim]).
+ * One launch for lines :155-158 and the v part of :151-152 of samples/05_llama2_7b_int4.py. */
+int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, void* q_out_dev, void* key_cache_dev, void* val_cache_dev,
+                       int heads, int head_dim, const void* pos_dev, int dtype, int freq_dtype, void* stream);
+/* art_rope_qkv_store and art_decode_attention in one launch (fp16): block h rotates its head's q and k,
+ * writes k and v into cache row *pos_dev and attends over rows 0..*pos_dev. */
+int art_decode_attention_rope(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev, void* val_cache_dev,
+                              const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev, void* stream);
 int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev, const void* att_f_dev, void* out_dev,
                          int seq_len, int heads, int head_dim, const void* pos_dev, int q_dtype, int kv_dtype, int out_dtype,
                          void* stream);

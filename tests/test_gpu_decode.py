@@ -15,13 +15,14 @@ def small_config():
     return LlamaConfig(n_layers=2, dim=512, n_heads=4, ffn=1024, vocab=1024, max_seq=32)
 
 
-def test_decode_matches_oracle_eager_and_graph():
+@pytest.mark.parametrize('fused', [False, True])
+def test_decode_matches_oracle_eager_and_graph(fused):
     from antares_amd.llama import LlamaInt4Decoder, random_weights
     from oracle.llama_ref import LlamaRef
     cfg = small_config()
     w = random_weights(cfg, seed=3)
     ref = LlamaRef(cfg, w)
-    dec = LlamaInt4Decoder(cfg, w)
+    dec = LlamaInt4Decoder(cfg, w, fused=fused)
     steps = 10
     tokens, ref_logits = [5], []
     for pos in range(steps):
@@ -56,3 +57,34 @@ def test_decode_matches_oracle_eager_and_graph():
             assert int(dec.token.item()) == tokens[pos + 1]
         dec.reset(tokens[pos + 1], pos + 1)             # keep both sides on the oracle's token stream
     assert torch.allclose(dec.key_cache.float(), eager_keys.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_fused_projection_matches_operator_chain():
+    """gemv_w4a16_fused against rmsnorm -> gemv -> add through the separate operators and against the oracle."""
+    import autort
+    from antares_amd import workloads
+    from antares_amd.autort import patterns
+    from oracle import hot_ops
+    dev = autort.device()
+    for K, N in [(512, 256), (4096, 4096), (11008, 4096), (4096, 12288)]:
+        print(f'[case] fused projection K={K} N={N}', flush=True)
+        p = workloads.w4_problem(K + N, 1, K, N)
+        g = torch.Generator().manual_seed(K)
+        nw = (1 + 0.1 * torch.randn(K, generator=g)).half()
+        res = torch.randn(N, generator=g).half()
+        x = p['x'].view(-1)
+        d = {k: v.to(dev) for k, v in p.items()}
+        got = autort.ops.gemv_w4a16_fused(x.to(dev), d['qweight'], d['scales'], d['qzeros'], norm_weight=nw.to(dev), residual=res.to(dev))
+        xn = hot_ops.rmsnorm(x.numpy(), None, nw.numpy(), 1.0 / K, 1e-5, np.float16)
+        y = hot_ops.gemm_w4a16(xn.reshape(1, K), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy()).reshape(-1)
+        want = (y.astype(np.float32) + res.numpy().astype(np.float32)).astype(np.float16)
+        assert np.allclose(got.cpu().numpy().astype(np.float32), want.astype(np.float32), rtol=1e-2, atol=1e-2)
+        # the chain of separate operators
+        f = autort.export(ir=patterns.W4A16_IR, inputs=patterns.W4A16_INPUTS, name='gemv_w4a16')
+        xb = autort.ops.rmsnorm_f16(x.to(dev), None, nw.to(dev))
+        chain = f(xb.view(1, -1), d['qweight'], d['scales'], d['qzeros']).view(-1) + res.to(dev)
+        assert torch.allclose(got.float(), chain.float(), rtol=2e-3, atol=2e-3)
+        # in place on the residual
+        buf = res.to(dev).clone()
+        autort.ops.gemv_w4a16_fused(x.to(dev), d['qweight'], d['scales'], d['qzeros'], buf, norm_weight=nw.to(dev), residual=buf)
+        assert torch.equal(buf, got)
