@@ -51,8 +51,8 @@ struct art_func {
   hipFunction_t handle;
 };
 
-// 16 MiB: split-K partial sums and tile states of the scan kernels.
-static constexpr size_t kWorkspaceBytes = 16u << 20;
+// 64 MiB: split-K accumulators, partial tiles of the split-K GEMM and tile states of the scan kernels.
+static constexpr size_t kWorkspaceBytes = 64u << 20;
 
 extern "C" {
 

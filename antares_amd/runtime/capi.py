@@ -46,6 +46,7 @@ _SIGNATURES = {
     'art_copy_bytes': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     'art_workspace_bytes': (c_size_t, []),
     'art_gemv_w4a16': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    'art_gemm_w4a16': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_gemv_gptq': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     'art_partition_even_first_i32': (c_int, [c_void_p, c_void_p, c_longlong, c_void_p]),
     'art_gemv_w4a16_fused': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p,

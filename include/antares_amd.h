@@ -101,6 +101,13 @@ int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* strea
 int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                    void* y_dev, int M, int K, int N, void* stream);
 
+/* The same product for any M >= 1 on the matrix cores (prefill batches; the samples' decode loop uses
+ * M = 1): operands, layouts and constraints as for art_gemv_w4a16, plus qzeros and y 8-byte aligned.
+ * Rows are processed 64 at a time; each pass reads the weights once.  K-splits are combined through the
+ * library workspace in a fixed order, so results do not depend on timing. */
+int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                   void* y_dev, int M, int K, int N, void* stream);
+
 /* The same GEMV (M = 1) with the operators that surround a projection in the
  * decode step of samples/05_llama2_7b_int4.py:146-177 folded in:
  *   norm_weight_dev != NULL: x is first replaced by

@@ -51,18 +51,27 @@ int ref_sort_even_first_i32(const int32_t* data, int32_t* output, long long m) {
  *   y[m,n]  = fp16( sum_k float(x[m,k]) * float(w[k,n]) )   fp32 accumulate in k order */
 void ref_gemm_w4a16(const uint16_t* x, const uint8_t* qweight, const uint16_t* scales, const uint8_t* qzeros,
                     uint16_t* y, int M, int K, int N) {
-  for (int m = 0; m < M; ++m)
-    for (int n = 0; n < N; ++n) {
+  /* The column of dequantised weights and the rows of x are widened once; every y[m,n] is still the
+   * k-ordered fp32 sum written above. */
+  float* w = (float*)malloc((size_t)K * sizeof(float));
+  float* xf = (float*)malloc((size_t)M * K * sizeof(float));
+  for (size_t i = 0; i < (size_t)M * K; ++i) xf[i] = ref_h2f(x[i]);
+  for (int n = 0; n < N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const int q = (qweight[(size_t)(k / 2) * N + n] >> (k % 2 * 4)) & 15;
+      const int z = (qzeros[(size_t)(k / 128) * (N / 2) + n / 2] >> (n % 2 * 4)) & 15;
+      const float s = ref_h2f(scales[(size_t)(k / 128) * N + n]);
+      w[k] = ref_h2f(ref_f2h(s * ref_h2f(ref_f2h((float)(q - z)))));
+    }
+    for (int m = 0; m < M; ++m) {
+      const float* xr = xf + (size_t)m * K;
       float acc = 0.0f;
-      for (int k = 0; k < K; ++k) {
-        const int q = (qweight[(size_t)(k / 2) * N + n] >> (k % 2 * 4)) & 15;
-        const int z = (qzeros[(size_t)(k / 128) * (N / 2) + n / 2] >> (n % 2 * 4)) & 15;
-        const float s = ref_h2f(scales[(size_t)(k / 128) * N + n]);
-        const float w = ref_h2f(ref_f2h(s * ref_h2f(ref_f2h((float)(q - z)))));
-        acc += ref_h2f(x[(size_t)m * K + k]) * w;
-      }
+      for (int k = 0; k < K; ++k) acc += xr[k] * w[k];
       y[(size_t)m * N + n] = ref_f2h(acc);
     }
+  }
+  free(w);
+  free(xf);
 }
 
 /* The sample's own program (samples/05_llama2_7b_int4.py:135-139), fp32 x:
