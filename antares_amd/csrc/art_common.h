@@ -28,6 +28,11 @@ constexpr size_t kScratchOffset = 4 * 1024 * 1024;       // partial sums, tile c
 
 }  // namespace art
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global load of the wave (vmcnt(0)), which drains register prefetches at each barrier; this one
+// leaves them in flight.  Use it only where the data exchanged through the barrier lives in LDS.
+__device__ __forceinline__ void art_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 #define ART_HIP(expr)                                                                   \
   do {                                                                                  \
     hipError_t _e = (expr);                                                             \

@@ -1,12 +1,12 @@
-// Weight-only int4 GEMM for a batch of rows (prefill, 9 <= M): the same arithmetic as the GEMV of
+// Weight-only int4 GEMM for a batch of rows (prefill, M > 8): the same arithmetic as the GEMV of
 // art_gemv_w4.hip,
 //     y[m,n] = sum_g s[g,n] * sum_{k in group g} x[m,k] * (q[k,n] - z[g,n]),      group = 128 k,
 // with the inner sums on the matrix cores.  Replaces the kernel the reference generates when the
 // dequant + matmul program of samples/05_llama2_7b_int4.py:135-144 is exported with a batch axis.
 //
 // Design for MI355X:
-//   * the weights are read from HBM exactly once; a block owns 128 columns (one full 128-byte line of
-//     every packed row) and a contiguous range of k groups, and streams them two groups ahead;
+//   * the weights are read from HBM exactly once; a work item owns 128 columns (one full 128-byte line
+//     of every packed row) and a contiguous range of k groups, and streams them two groups ahead;
 //   * unpacking is fused into the LDS staging: 16 bytes (16 columns x 2 k) become two rows of fp16
 //     (q - z) values - exact small integers - with one shift, four and-or and four packed subtractions
 //     per word.  The columns of every group of four land in LDS in the order 0,2,1,3, which costs nothing:
@@ -14,6 +14,9 @@
 //   * v_mfma_f32_32x32x16_f16 per wave: 32 columns x 64 rows, B operand through ds_read_b64_tr_b16;
 //     the group sum is scaled by s[g,n] in fp32 afterwards (one scalar per lane, since an accumulator
 //     lane owns one column), so no scale is rounded to fp16;
+//   * a block is two independent work items of four waves each that alternate phases: while one half
+//     unpacks its next group on the vector units, the other half multiplies its current group on the
+//     matrix cores.  One wave of each half sits on every SIMD, so both pipes stay busy;
 //   * split-K without atomics (5.6 M float atomics cost 75 us on this chip): each K-split writes its
 //     fp32 tile to the library workspace and a second small kernel adds the splits in a fixed order
 //     and rounds once to fp16 - results do not depend on timing.
@@ -34,8 +37,11 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 constexpr int BM = 64, BN = 128, GK = 128;     // rows, columns and k per staged tile
-constexpr int W_LD = BN + 16;                  // halves per weight row in LDS (288 bytes)
+constexpr int W_LD = BN + 32;                  // halves per weight row in LDS: 320 bytes, so the four k rows
+                                               // a transposing read touches fall on disjoint banks
 constexpr int X_LD = GK + 8;                   // halves per x row in LDS (272 bytes)
+constexpr int HALF_LDS = GK * W_LD + BM * X_LD;                 // halves of LDS per work item
+constexpr size_t kLdsBytes = (size_t)2 * HALF_LDS * sizeof(_Float16);
 
 struct Magic {
   unsigned int mask_lo, mask_hi, bias_lo, bias_hi;   // 0x000F000F 0x00F000F0 0x64006400 0x54005400
@@ -44,27 +50,41 @@ struct Magic {
 __device__ __forceinline__ h2 as_h2(unsigned int v) { return __builtin_bit_cast(h2, v); }
 __device__ __forceinline__ unsigned int as_u32(h2 v) { return __builtin_bit_cast(unsigned int, v); }
 
-// (w & mask) | bias for disjoint mask and bias.
+// (w & mask) | bias in one v_bitop3_b32 (truth table 0xEA = (a & b) | c).
 __device__ __forceinline__ unsigned int and_or(unsigned int w, unsigned int mask, unsigned int bias) {
-  return (w & mask) | (~mask & bias);
+  return __builtin_amdgcn_bitop3_b32(w, mask, bias, 0xEA);
 }
 
 // Position p of a staged column <-> column of the matrix: bits 0 and 1 swapped.
 __device__ __forceinline__ int unpermute(int p) { return (p & ~3) | ((p & 1) << 1) | ((p >> 1) & 1); }
 
 template <int MT>   // MT accumulator tiles of 32 rows: 1 for M <= 32, 2 for M <= 64
-__global__ __launch_bounds__(256) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
+__global__ __launch_bounds__(512) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
                                                           const _Float16* __restrict__ scales,
                                                           const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y,
                                                           float* __restrict__ partial, int M, int K, int N, int splits,
-                                                          Magic mg) {
-  __shared__ __align__(16) _Float16 Ws[GK * W_LD];
-  __shared__ __align__(16) _Float16 Xs[MT * 32 * X_LD];
+                                                          int col_tiles, Magic mg) {
+  extern __shared__ __align__(16) _Float16 smem[];
+  const int half = threadIdx.x >> 8;             // which of the block's two work items this wave serves
+  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+  _Float16* Ws = smem + half * HALF_LDS;         // [GK][W_LD]
+  _Float16* Xs = Ws + GK * W_LD;                 // [BM][X_LD]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * BN;
-  const int G = K / GK;
-  const int g_begin = (int)((long long)G * blockIdx.y / splits), g_end = (int)((long long)G * (blockIdx.y + 1) / splits);
+  // work item -> (column tile, K split); the two halves of a block take neighbouring column tiles
+  const int G = K / GK, items = col_tiles * splits;
+  auto group_range = [&](int item, int& begin, int& end) {
+    const int split = item / col_tiles;
+    begin = item < items ? (int)((long long)G * split / splits) : 0;
+    end = item < items ? (int)((long long)G * (split + 1) / splits) : 0;
+  };
+  const int item = blockIdx.x * 2 + half;
+  int g_begin, g_end, o_begin, o_end;
+  group_range(item, g_begin, g_end);
+  group_range(blockIdx.x * 2 + (1 - half), o_begin, o_end);
+  const int steps = g_end - g_begin;
+  const int T = steps > o_end - o_begin ? steps : o_end - o_begin;      // both halves pass the same barriers
+  const int split = item / col_tiles;
+  const int n0 = (item % col_tiles) * BN;
 
   // ---- global -> register staging
   // weights: 64 packed rows x 128 bytes per group = 512 chunks of 16 bytes, two per thread
@@ -90,14 +110,14 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const _Float16* __restr
   const int b_n = wave * 32 + ((lane & 31) >> 4) * 16 + (s16 & 3) * 4;
   const int my_col = n0 + unpermute(wave * 32 + (lane & 31));       // the column this lane accumulates
   const bool my_ok = my_col < N;
+  const int sc_col = my_ok ? my_col : 0;
 
-  // Two register stages: the loads of group g + 2 are issued while group g is unpacked and multiplied.
+  // Two register stages: the loads of group g + 2 are issued while group g is unpacked.
   // Stages are indexed statically (a run-time index would put the arrays in scratch memory).
   u32x4 wq[2][2];      // [stage][chunk]
   u32x4 xr[2][2 * MT];
   u32x2 zq[2];
   _Float16 sc16[2];
-  const int sc_col = my_ok ? my_col : 0;
   auto load_stage = [&](int g, auto tag) {
     constexpr int S = decltype(tag)::value;
 #pragma unroll
@@ -109,16 +129,19 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const _Float16* __restr
     sc16[S] = scales[(size_t)g * N + sc_col];
   };
 
-  f16v total[MT], grp[MT];
+  f16v total[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) total[i][r] = 0.f;
+  float sc_staged = 0.f;     // scale of the group that currently sits in LDS
 
-  auto step = [&](int g, auto tag) {
+  // Phase D: unpack step i of this work item into LDS and refill its register stage.
+  auto unpack = [&](int i, auto tag) {
     constexpr int S = decltype(tag)::value;
+    if (i >= steps) return;
+    sc_staged = my_ok ? (float)sc16[S] : 0.f;
     // zero points of this thread's 16 columns, paired (c0,c2) and (c1,c3), on both nibble biases
-    const float sc = my_ok ? (float)sc16[S] : 0.f;
     h2 z_lo[8], z_hi[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -130,13 +153,13 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const _Float16* __restr
       z_hi[2 * j] = as_h2(and_or(e << 4, mg.mask_hi, mg.bias_hi));
       z_hi[2 * j + 1] = as_h2(and_or(o << 4, mg.mask_hi, mg.bias_hi));
     }
-    // unpack: chunk c holds packed row pr + 32c = k rows 2*(pr+32c) and 2*(pr+32c)+1
+    // chunk c holds packed row pr + 32c = k rows 2*(pr+32c) and 2*(pr+32c)+1
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
       u32x4 even[2], odd[2];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const unsigned int w = col_ok ? wq[S][c][j] : 0u, w8 = w >> 8;
+        const unsigned int w = wq[S][c][j], w8 = w >> 8;    // columns past N hold finite garbage and are never stored
         const h2 e02 = as_h2(and_or(w, mg.mask_lo, mg.bias_lo)) - z_lo[2 * j];
         const h2 e13 = as_h2(and_or(w8, mg.mask_lo, mg.bias_lo)) - z_lo[2 * j + 1];
         const h2 o02 = as_h2(and_or(w, mg.mask_hi, mg.bias_hi)) - z_hi[2 * j];
@@ -153,14 +176,18 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const _Float16* __restr
       *reinterpret_cast<u32x4*>(row + W_LD + 8) = odd[1];
     }
 #pragma unroll
-    for (int i = 0; i < 2 * MT; ++i) *reinterpret_cast<u32x4*>(Xs + xs_off[i]) = xr[S][i];
-    if (g + 2 < g_end) load_stage(g + 2, tag);     // refill the stage just consumed
-    __syncthreads();
+    for (int j = 0; j < 2 * MT; ++j) *reinterpret_cast<u32x4*>(Xs + xs_off[j]) = xr[S][j];
+    if (i + 2 < steps) load_stage(g_begin + i + 2, tag);     // refill the stage just consumed
+  };
 
+  // Phase M: multiply the group that sits in LDS (step i) and add it, scaled, to the totals.
+  auto multiply = [&](int i) {
+    if (i < 0 || i >= steps) return;
+    f16v grp[MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) grp[i][r] = 0.f;
+      for (int r = 0; r < 16; ++r) grp[t][r] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < GK / 16; ++kk) {
       const _Float16* p = Ws + (kk * 16 + b_k) * W_LD + b_n;
@@ -169,37 +196,48 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const _Float16* __restr
       const h4 l4 = __builtin_bit_cast(h4, lo), h4v = __builtin_bit_cast(h4, hi);
       const h8 bf = h8{l4[0], l4[1], l4[2], l4[3], h4v[0], h4v[1], h4v[2], h4v[3]};
 #pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        const h8 af = *reinterpret_cast<const h8*>(Xs + (a_row + i * 32) * X_LD + kk * 16 + a_k);
-        grp[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, grp[i], 0, 0, 0);
+      for (int t = 0; t < MT; ++t) {
+        const h8 af = *reinterpret_cast<const h8*>(Xs + (a_row + t * 32) * X_LD + kk * 16 + a_k);
+        grp[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, grp[t], 0, 0, 0);
       }
     }
+    const float sc = sc_staged;
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) total[i][r] += grp[i][r] * sc;
-    __syncthreads();
+      for (int r = 0; r < 16; ++r) total[t][r] += grp[t][r] * sc;
   };
 
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
-  if (g_begin < g_end) load_stage(g_begin, S0{});
-  if (g_begin + 1 < g_end) load_stage(g_begin + 1, S1{});
-  for (int g = g_begin; g < g_end; g += 2) {
-    step(g, S0{});
-    if (g + 1 < g_end) step(g + 1, S1{});
+  if (steps > 0) load_stage(g_begin, S0{});
+  if (steps > 1) load_stage(g_begin + 1, S1{});
+  // Time slots, one barrier after each:   half 0:  D(0) M(0) D(1) M(1) ...
+  //                                        half 1:   -   D(0) M(0) D(1) ...  M(T-1)
+  auto iteration = [&](int i, auto tag) {
+    if (half == 0) unpack(i, tag);
+    else multiply(i - 1);
+    art_lds_barrier();
+    if (half == 0) multiply(i);
+    else unpack(i, tag);
+    art_lds_barrier();
+  };
+  for (int i = 0; i < T; i += 2) {
+    iteration(i, S0{});
+    if (i + 1 < T) iteration(i + 1, S1{});
   }
+  if (half == 1) multiply(T - 1);
 
-  // ---- epilogue: accumulator element r of tile i is row i*32 + (r/4)*8 + (lane/32)*4 + r%4, column my_col
-  if (!my_ok) return;
+  // ---- epilogue: accumulator element r of tile t is row t*32 + (r/4)*8 + (lane/32)*4 + r%4, column my_col
+  if (!my_ok || steps == 0) return;
 #pragma unroll
-  for (int i = 0; i < MT; ++i)
+  for (int t = 0; t < MT; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int row = i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+      const int row = t * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
       if (row < M) {
-        if (splits == 1) y[(size_t)row * N + my_col] = (_Float16)total[i][r];
-        else partial[((size_t)blockIdx.y * M + row) * N + my_col] = total[i][r];
+        if (splits == 1) y[(size_t)row * N + my_col] = (_Float16)total[t][r];
+        else partial[((size_t)split * M + row) * N + my_col] = total[t][r];
       }
     }
 }
@@ -215,15 +253,16 @@ __global__ __launch_bounds__(256) void gemm_w4a16_combine_kernel(const float* __
   *reinterpret_cast<h4*>(y + i * 4) = out;
 }
 
-// Number of K-splits: enough blocks to occupy every compute unit about twice, bounded by the
-// number of groups and by the scratch space the partial tiles need.
-int choose_splits(int rows, int N, int G, size_t scratch_bytes) {
+// Number of K-splits: as many work items as fit the chip in one round (two per compute unit), but at
+// least four groups per item, and no more than the scratch space for the partial tiles allows.
+// Measured on MI355X at M = 64: N=4096 K=4096 -> 8, N=11008 -> 5, N=4096 K=11008 -> 16, N=32000 -> 2.
+int choose_splits(int rows, int N, int G, size_t scratch_bytes, int compute_units) {
   const int col_tiles = (N + BN - 1) / BN;
-  int s = (512 + col_tiles - 1) / col_tiles;
+  int s = 2 * compute_units / col_tiles;
+  if (s > G / 4) s = G / 4;
   const size_t per_split = (size_t)rows * N * sizeof(float);
   const int cap = (int)(scratch_bytes / per_split);
   if (s > cap) s = cap;
-  if (s > G) s = G;
   return s < 1 ? 1 : s;
 }
 
@@ -241,21 +280,33 @@ extern "C" int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const 
   ART_REQUIRE(ws.base != nullptr, "art_gemm_w4a16: art_init has not been called on this device");
   float* scratch = reinterpret_cast<float*>((char*)ws.base + art::kScratchOffset);
   const size_t scratch_bytes = ws.bytes - art::kScratchOffset;
+  static int compute_units = 0;
+  if (compute_units == 0) {
+    int dev = 0;
+    ART_HIP(hipGetDevice(&dev));
+    ART_HIP(hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, dev));
+    ART_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_w4a16_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)kLdsBytes));
+    ART_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_w4a16_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)kLdsBytes));
+  }
   const Magic mg{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
   hipStream_t st = (hipStream_t)stream;
-  const int G = K / GK;
+  const int G = K / GK, col_tiles = (N + BN - 1) / BN;
   for (int m0 = 0; m0 < M; m0 += BM) {      // 64 rows of x per pass over the weights
     const int rows = M - m0 < BM ? M - m0 : BM;
-    const int splits = choose_splits(rows, N, G, scratch_bytes);
+    const int splits = choose_splits(rows, N, G, scratch_bytes, compute_units);
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m0 * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m0 * N;
-    const dim3 grid((N + BN - 1) / BN, splits);
+    const dim3 grid((col_tiles * splits + 1) / 2);
     if (rows <= 32)
-      gemm_w4a16_kernel<1><<<grid, 256, 0, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
-                                                 (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits, mg);
+      gemm_w4a16_kernel<1><<<grid, 512, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
+                                                         (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
+                                                         col_tiles, mg);
     else
-      gemm_w4a16_kernel<2><<<grid, 256, 0, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
-                                                 (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits, mg);
+      gemm_w4a16_kernel<2><<<grid, 512, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
+                                                         (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
+                                                         col_tiles, mg);
     ART_LAUNCH_CHECK();
     if (splits > 1) {
       const long long count4 = (long long)rows * N / 4;

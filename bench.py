@@ -30,6 +30,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
 LAYERS = 32
 # HBM bytes per launch of the headline GEMV kernel, from FETCH_SIZE / WRITE_SIZE counters scaled by
 # the copy-kernel calibration (profiles/gemv_w4a16_4096x11008_traffic_pmc.md): 23.80 MB read + 0.81 MB written.
@@ -92,8 +93,20 @@ def bench_gemv(torch, autort, capi, workloads, K, N, M, steps, warmup, seed, lay
     sec = time_graph(torch, capi, one_pass, steps, warmup)
     per_launch = sec / layers
     by = workloads.w4_bytes(M, K, N)
-    return {'workload': f'int4 g128 GEMV M={M} K={K} N={N}', 'bytes_per_launch': by, 'launches_per_step': layers,
+    return {'workload': f"int4 g128 {'GEMV' if M <= 8 else 'GEMM'} M={M} K={K} N={N}", 'bytes_per_launch': by, 'launches_per_step': layers,
             'sec_per_step': sec, 'us_per_launch': per_launch * 1e6, 'gbps': by / per_launch / 1e9}
+
+
+def bench_gemm_f16(torch, autort, capi, workloads, steps, warmup, seed, n):
+    from antares_amd.autort import patterns
+    dev = autort.device()
+    op = autort.export(ir=patterns.GEMM_F16_IR, inputs=patterns.GEMM_F16_INPUTS, name='gemm_f16')
+    a, b = (t.to(dev) for t in workloads.gemm_inputs(seed, n))
+    c = torch.empty(n, n, dtype=torch.float16, device=dev)
+    sec = time_graph(torch, capi, lambda: op(a, b, out=c), steps, warmup)
+    tflops = 2.0 * n * n * n / sec / 1e12
+    return {'workload': f'fp16 GEMM M=N=K={n} (fp32 accumulate)', 'us_per_launch': sec * 1e6, 'tflops': tflops,
+            'roofline_bound': 'mfma', 'roofline_frac': tflops / MFMA_F16_PEAK_TFLOPS}
 
 
 def bench_sigmoid(torch, autort, capi, workloads, steps, warmup, seed, n=4_096_000, copies=16):
@@ -242,6 +255,13 @@ def main():
                            layers=32 if n < 32000 else 8)
             extra.append({'workload': r['workload'], 'us_per_launch': round(r['us_per_launch'], 3), 'gbps': round(r['gbps'], 1),
                           'roofline_frac': round(r['gbps'] / HBM_PEAK_GBPS, 4)})
+        for (k, n) in [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 32000)]:
+            r = bench_gemv(torch, autort, capi, workloads, k, n, 64, max(10, args.steps // 2), args.warmup, args.seed, layers=8)
+            extra.append({'workload': r['workload'], 'us_per_launch': round(r['us_per_launch'], 3), 'gbps': round(r['gbps'], 1),
+                          'roofline_frac': round(r['gbps'] / HBM_PEAK_GBPS, 4)})
+        for n in (4096, 8192):
+            r = bench_gemm_f16(torch, autort, capi, workloads, max(5, args.steps // 4), args.warmup, args.seed, n)
+            extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
         for fn in (bench_sigmoid, bench_partition):
             r = fn(torch, autort, capi, workloads, args.steps, args.warmup, args.seed)
             extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
