@@ -99,9 +99,11 @@ __global__ __launch_bounds__(256) void rotary_kernel(const XT* __restrict__ x, c
 
 // ------------------------------------------------------------------ attention (one query)
 // att[h,s] = (sum_m q[h,m] k[s,h,m]) * att_f ; p = softmax_s(att) ; out[h,m] = sum_s p[h,s] v[s,h,m]
-// One block per head.  Eight lanes share a position (16 dims = 32 bytes of fp16 each), so a wavefront
-// reads eight 256-byte rows per step; every 8-lane group keeps an online-softmax state (max, sum, 16
-// partial outputs) for the positions it visits; the 32 groups of the block are merged through LDS.
+// One block of 512 threads per head.  Eight lanes share a position (16 dims = 32 bytes of fp16 each), so
+// a wavefront reads eight 256-byte rows per step; every 8-lane group keeps an online-softmax state (max,
+// sum, 16 partial outputs) for the positions it visits and has four positions in flight, 256 positions
+// (128 KiB) per block - a compute unit needs that much outstanding to stream at its full rate.  The
+// eight groups of a wavefront are merged with lane exchanges, the eight wavefronts through LDS.
 template <class T> struct Row16;   // 16 consecutive elements as floats
 template <> struct Row16<_Float16> {
   static __device__ __forceinline__ void load(const _Float16* p, float (&f)[16]) {
@@ -130,8 +132,20 @@ template <> struct Row16<float> {
   }
 };
 
-constexpr int kAttThreads = 256;
-constexpr int kAttGroups = kAttThreads / 8;   // 32 position groups per block
+constexpr int kAttThreads = 512;
+constexpr int kAttGroups = kAttThreads / 8;   // 64 position groups per block
+constexpr int kAttWaves = kAttThreads / 64;
+
+// Merge the online-softmax state of the lane `mask` away (same dims, other positions) into this lane's.
+__device__ __forceinline__ void att_merge_lane(float& m, float& l, float (&acc)[16], int mask) {
+  const float m2 = __shfl_xor(m, mask), l2 = __shfl_xor(l, mask);
+  const float mn = fmaxf(m, m2);
+  const float c1 = (m == -INFINITY) ? 0.f : __expf(m - mn), c2 = (m2 == -INFINITY) ? 0.f : __expf(m2 - mn);
+  l = l * c1 + l2 * c2;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = acc[i] * c1 + __shfl_xor(acc[i], mask) * c2;
+  m = mn;
+}
 
 // ROPE = true: the block first rotates its head's q and k (rotate-half form) from the token's q|k|v vector,
 // writes k and v into cache row `pos` and attends over rows 0..pos; q_or_qkv then points at q|k|v.
@@ -141,37 +155,69 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
                                                                  const int* __restrict__ len_dev, int len_host,
                                                                  const _Float16* __restrict__ inv_freq) {
   constexpr int D = 128, U = 4;
-  __shared__ float s_m[kAttGroups], s_l[kAttGroups];
-  __shared__ float s_acc[kAttGroups][D];
+  __shared__ float s_m[kAttWaves], s_l[kAttWaves];
+  __shared__ float s_acc[kAttWaves][D];
   __shared__ float s_q[D];
+  __shared__ float s_k[D], s_v[D];
   const int S = len_dev ? (*len_dev + 1) : len_host;     // device form carries the position, length = pos + 1
   const int h = blockIdx.x, tid = threadIdx.x;
   const int sub = tid & 7, group = tid >> 3;
   const float scale = att_f[0];
   const size_t row = (size_t)heads * D;
+  // With ROPE the newest position is served from LDS: the block does not wait for its own cache write.
+  const int Sc = ROPE ? S - 1 : S;                        // positions read from the cache
+
+  // this thread's share of the token's q|k|v, requested before anything else
+  float xa = 0.f, xb = 0.f, xv = 0.f;
+  if (ROPE) {
+    const int dim = heads * D;
+    if (tid < 128) {                                      // 64 pairs of q, 64 pairs of k
+      const QT* src = q_or_qkv + (tid >= 64 ? dim : 0) + (size_t)h * D;
+      xa = ld(src, tid & 63);
+      xb = ld(src, (tid & 63) + 64);
+    } else if (tid < 256) {
+      xv = ld(q_or_qkv, 2 * (size_t)dim + (size_t)h * D + (tid - 128));
+    }
+  }
+  // U positions per group are requested before the first is used, and the first round is requested
+  // before the rotary phase, which does not depend on it
+  float kf[U][16], vf[U][16];
+  auto request = [&](int s0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * kAttGroups;
+      const int sc = s < Sc ? s : s0;                     // past the end: re-read a valid row, weight 0 below
+      Row16<KT>::load(k + (size_t)sc * row + (size_t)h * D + sub * 16, kf[u]);
+      Row16<KT>::load(v + (size_t)sc * row + (size_t)h * D + sub * 16, vf[u]);
+    }
+  };
+  if (group < Sc) request(group);
+
   float qf[16];
   if (ROPE) {
-    const int pos = S - 1, dim = heads * D;
-    if (tid < 128) {                                      // 64 pairs of q, 64 pairs of k
+    const int pos = S - 1;
+    if (tid < 128) {
       const bool is_k = tid >= 64;
       const int j = tid & 63;
-      const QT* src = q_or_qkv + (is_k ? dim : 0) + (size_t)h * D;
       float sn, cs;
       sincosf((float)pos * (float)inv_freq[j], &sn, &cs);
-      const float xa = ld(src, j), xb = ld(src, j + 64);
       const float ra = xa * cs - xb * sn, rb = xb * cs + xa * sn;
-      if (is_k) {
-        st(k + (size_t)pos * row + (size_t)h * D, j, ra);
-        st(k + (size_t)pos * row + (size_t)h * D, j + 64, rb);
+      if (is_k) {                                         // the cache gets the rounded value, and so does this step
+        KT* dst = k + (size_t)pos * row + (size_t)h * D;
+        st(dst, j, ra);
+        st(dst, j + 64, rb);
+        s_k[j] = (float)(KT)ra;
+        s_k[j + 64] = (float)(KT)rb;
       } else {                                            // q goes through the output dtype like the separate operator
         s_q[j] = (float)(QT)ra;
         s_q[j + 64] = (float)(QT)rb;
       }
-    } else {
+    } else if (tid < 256) {
       const int e = tid - 128;
-      v[(size_t)pos * row + (size_t)h * D + e] = (KT)q_or_qkv[2 * (size_t)dim + (size_t)h * D + e];
+      v[(size_t)pos * row + (size_t)h * D + e] = (KT)xv;
+      s_v[e] = (float)(KT)xv;
     }
-    __syncthreads();
+    art_lds_barrier();
 #pragma unroll
     for (int i = 0; i < 16; ++i) qf[i] = s_q[sub * 16 + i] * scale;
   } else {
@@ -182,47 +228,61 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
   float m = -INFINITY, l = 0.f, acc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-  // U positions per group are requested before the first is used: S/128 round trips instead of S/32
-  for (int s0 = group; s0 < S; s0 += kAttGroups * U) {
-    float kf[U][16], vf[U][16];
+  auto group_sum = [](float d) {   // sum over the 8 lanes of a group (xor 1, xor 2 inside a quad, then the neighbouring quad)
+    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xf, 0xf, false));
+    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xf, 0xf, false));
+    d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xf, 0xf, false));
+    return d;
+  };
+  auto absorb = [&](float d, const float (&vrow)[16]) {   // one position into this group's online softmax
+    const float mn = fmaxf(m, d);
+    const float corr = __expf(m - mn), p = __expf(d - mn);
+    l = l * corr + p;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * vrow[i]);
+    m = mn;
+  };
+  for (int s0 = group; s0 < Sc; s0 += kAttGroups * U) {
+    if (s0 != group) request(s0);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int s = s0 + u * kAttGroups;
-      const int sc = s < S ? s : s0;                      // past the end: re-read a valid row, weight 0 below
-      Row16<KT>::load(k + (size_t)sc * row + (size_t)h * D + sub * 16, kf[u]);
-      Row16<KT>::load(v + (size_t)sc * row + (size_t)h * D + sub * 16, vf[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int s = s0 + u * kAttGroups;
       float d = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kf[u][i], d);
-      // sum over the 8 lanes of the group (xor 1, xor 2 inside a quad, then the neighbouring quad)
-      d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xf, 0xf, false));
-      d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xf, 0xf, false));
-      d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xf, 0xf, false));
-      if (s < S) {
-        const float mn = fmaxf(m, d);
-        const float corr = __expf(m - mn), p = __expf(d - mn);
-        l = l * corr + p;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * vf[u][i]);
-        m = mn;
-      }
+      d = group_sum(d);
+      if (s0 + u * kAttGroups < Sc) absorb(d, vf[u]);
     }
   }
-  if (sub == 0) { s_m[group] = m; s_l[group] = l; }
+  if (ROPE) {                                             // the newest position, from LDS, joins group 0
+    float kn[16], vn[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) s_acc[group][sub * 16 + i] = acc[i];
-  __syncthreads();
+    for (int i = 0; i < 16; ++i) {
+      kn[i] = s_k[sub * 16 + i];
+      vn[i] = s_v[sub * 16 + i];
+    }
+    float d = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kn[i], d);
+    d = group_sum(d);
+    if (group == 0) absorb(d, vn);
+  }
+  att_merge_lane(m, l, acc, 8);       // the eight groups of a wavefront: lanes that differ in bits 3..5
+  att_merge_lane(m, l, acc, 16);
+  att_merge_lane(m, l, acc, 32);
+  const int wave = tid >> 6;
+  if ((tid & 63) < 8) {
+    if (sub == 0) { s_m[wave] = m; s_l[wave] = l; }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s_acc[wave][sub * 16 + i] = acc[i];
+  }
+  art_lds_barrier();                  // LDS only: the cache-row stores above need not have landed
   if (tid < D) {
     float mm = -INFINITY;
 #pragma unroll
-    for (int g = 0; g < kAttGroups; ++g) mm = fmaxf(mm, s_m[g]);
+    for (int g = 0; g < kAttWaves; ++g) mm = fmaxf(mm, s_m[g]);
     float ll = 0.f, o = 0.f;
 #pragma unroll
-    for (int g = 0; g < kAttGroups; ++g) {
+    for (int g = 0; g < kAttWaves; ++g) {
       const float wgt = (s_m[g] == -INFINITY) ? 0.f : __expf(s_m[g] - mm);
       ll = fmaf(s_l[g], wgt, ll);
       o = fmaf(s_acc[g][tid], wgt, o);
