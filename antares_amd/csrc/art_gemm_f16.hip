@@ -6,21 +6,25 @@
 // scalar loads through LDS, one FMA per element, no matrix instructions).
 //
 // Design for MI355X:
-//   * block tile 256 x 256 x 64, 256 threads = 2 x 2 wavefronts, each wavefront owns 128 x 128 of C as
+//   * block tile 256 x 256 x 32, 256 threads = 2 x 2 wavefronts, each wavefront owns 128 x 128 of C as
 //     4 x 4 accumulator tiles of v_mfma_f32_32x32x16_f16 (256 accumulator registers per lane, one
 //     wavefront per SIMD); 16 MFMAs (512 matrix-core cycles) per 8 KiB of LDS reads;
 //   * A tile in LDS as [m][k] (k contiguous, rows padded by 16 bytes): one ds_read_b128 gives a lane
 //     its 8 consecutive k of one row;
-//   * B tile in LDS exactly as it lies in memory, [k][n] (n contiguous, rows padded by 32 bytes); the
+//   * B tile in LDS exactly as it lies in memory, [k][n] (n contiguous, rows padded by 64 bytes); the
 //     MFMA wants 8 consecutive k per lane for ONE column, which is the transpose: ds_read_b64_tr_b16
 //     (new in gfx950) reads a 4(k) x 16(n) patch with 16 lanes and hands lane L the four k of column L.
-//     Two such reads make one B operand; the 32-byte row padding spreads the four k rows over all banks;
-//   * global -> registers -> LDS, double buffered: the loads of tile t+1 are issued before the MFMAs of
-//     tile t and stored to the other LDS buffer after them; one barrier per 64 k;
+//     Two such reads make one B operand; the row padding puts the four k rows on disjoint banks;
+//   * global -> registers -> LDS with two register stages (indexed statically) and two LDS buffers;
+//     the one barrier per tile waits for LDS only, so global loads stay in flight across it;
+//   * one wavefront per SIMD means nothing else hides a stall, so every LDS read, LDS write and global
+//     load is issued between two MFMAs of the other k-step (sched_group_barrier pins the order);
 //   * block -> tile mapping is XCD aware: the 32 blocks that run on one XCD at a time cover a 4 x 8
 //     super-tile, so they share 4 A panels and 8 B panels through that XCD's L2;
 //   * C goes through LDS once more so that it leaves as 128-bit row-contiguous stores.
 #include "art_common.h"
+
+#include <type_traits>
 
 namespace {
 
@@ -30,14 +34,15 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int A_LD = BK + 8;             // halves per A row in LDS (144 bytes)
-constexpr int B_LD = BN + 16;            // halves per B row in LDS (544 bytes)
+constexpr int BM = 256, BN = 256, BK = 32;
+constexpr int A_LD = BK + 8;             // halves per A row in LDS (80 bytes)
+constexpr int B_LD = BN + 32;            // halves per B row in LDS (576 bytes = 16 banks past a multiple of 64)
 constexpr int A_TILE = BM * A_LD;        // halves
 constexpr int B_TILE = BK * B_LD;
 constexpr int C_LD = BN + 8;             // halves per C row while staging the output
-constexpr size_t kLdsBytes = (size_t)(2 * A_TILE + 2 * B_TILE) * 2;
-static_assert((size_t)BM * C_LD * 2 <= kLdsBytes, "output staging must fit in the operand buffers");
+constexpr size_t kOperandBytes = (size_t)(2 * A_TILE + 2 * B_TILE) * 2;
+constexpr size_t kOutputBytes = (size_t)BM * C_LD * 2;
+constexpr size_t kLdsBytes = kOperandBytes > kOutputBytes ? kOperandBytes : kOutputBytes;
 
 __device__ __forceinline__ int xcd_tile(int b, int nb) {
   const int q = nb >> 3, r = nb & 7, xcd = b & 7, idx = b >> 3;
@@ -67,22 +72,34 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
   const _Float16* Ag = A + (size_t)tm * BM * K;
   const _Float16* Bg = B + (size_t)tn * BN;
 
-  // global -> register staging: 8 chunks of 16 bytes per thread for each operand
-  u32x4 ga[8], gb[8];
-  auto load_tiles = [&](int kt) {
+  // global -> register staging: 4 chunks of 16 bytes per thread for each operand and stage.  The
+  // per-thread part of every address is computed once; a tile only adds a wave-uniform offset.
+  u32x4 ga[2][4], gb[2][4];
+  const _Float16* pa[4];
+  const _Float16* pb[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int c = tid + 256 * i;
-      ga[i] = *reinterpret_cast<const u32x4*>(Ag + (size_t)(c >> 3) * K + (size_t)kt * BK + (c & 7) * 8);
-      gb[i] = *reinterpret_cast<const u32x4*>(Bg + ((size_t)kt * BK + (c >> 5)) * N + (c & 31) * 8);
+  for (int i = 0; i < 4; ++i) {
+    const int c = tid + 256 * i;
+    pa[i] = Ag + (size_t)(c >> 2) * K + (c & 3) * 8;
+    pb[i] = Bg + (size_t)(c >> 5) * N + (c & 31) * 8;
+  }
+  const size_t b_step = (size_t)BK * N;
+  auto load_tiles = [&](int kt, auto tag) {
+    constexpr int S = decltype(tag)::value;
+    const size_t oa = (size_t)kt * BK, ob = (size_t)kt * b_step;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ga[S][i] = *reinterpret_cast<const u32x4*>(pa[i] + oa);
+      gb[S][i] = *reinterpret_cast<const u32x4*>(pb[i] + ob);
     }
   };
-  auto store_tiles = [&](int buf) {
+  auto store_tiles = [&](int buf, auto tag) {
+    constexpr int S = decltype(tag)::value;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < 4; ++i) {
       const int c = tid + 256 * i;
-      *reinterpret_cast<u32x4*>(As + buf * A_TILE + (c >> 3) * A_LD + (c & 7) * 8) = ga[i];
-      *reinterpret_cast<u32x4*>(Bs + buf * B_TILE + (c >> 5) * B_LD + (c & 31) * 8) = gb[i];
+      *reinterpret_cast<u32x4*>(As + buf * A_TILE + (c >> 2) * A_LD + (c & 3) * 8) = ga[S][i];
+      *reinterpret_cast<u32x4*>(Bs + buf * B_TILE + (c >> 5) * B_LD + (c & 31) * 8) = gb[S][i];
     }
   };
 
@@ -121,39 +138,61 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
   };
 
   const int T = K / BK;
-  load_tiles(0);
-  store_tiles(0);
-  __syncthreads();
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  load_tiles(0, S0{});
+  load_tiles(1, S1{});                     // K >= 64: there are at least two tiles
+  store_tiles(0, S0{});
+  load_tiles(T > 2 ? 2 : T - 1, S0{});
+  art_lds_barrier();
   h8 af0[4], bf0[4], af1[4], bf1[4];
-  for (int t = 0; t < T; ++t) {
+  load_frags(af0, bf0, As, Bs, 0);
+  // One tile = two k-steps of 16 MFMAs.  Tile t sits in LDS buffer t & 1.  Register stage `nxt` holds
+  // tile t + 1 (requested a tile and a half ago); once it is written to LDS it is refilled with tile
+  // t + 3, while stage `cur` keeps tile t + 2 in flight.  Every LDS and global
+  // instruction is issued between two MFMAs of the other k-step, so the single wavefront of a SIMD
+  // never leaves the matrix core idle while it waits for operands:
+  //   first half:   MFMAs of k-step 0  |  operand reads of k-step 1, tile t+1 written to the other buffer
+  //   barrier (LDS only)
+  //   second half:  MFMAs of k-step 1  |  operand reads of k-step 0 of tile t+1, global loads of tile t+3
+  // The sched_group_barrier sequences pin that interleaving (0x008 MFMA, 0x080 LDS, 0x020 global load); sched_barrier(0) closes each half.
+  auto k_tile = [&](int t, auto cur, auto nxt, auto last_tag) {
+    constexpr bool LAST = decltype(last_tag)::value;
     const int buf = t & 1;
     const _Float16* as = As + buf * A_TILE;
     const _Float16* bs = Bs + buf * B_TILE;
-    // The scheduler is told not to move anything across these fences: without them it sinks every
-    // operand read next to its first use and the matrix cores wait for LDS sixteen times per tile.
-#define ART_FENCE() __builtin_amdgcn_sched_barrier(0)
-    load_frags(af0, bf0, as, bs, 0);
-    ART_FENCE();
-    if (t + 1 < T) load_tiles(t + 1);
-    ART_FENCE();
-    load_frags(af1, bf1, as, bs, 1);     // operands of k-step kk+1 are requested before the MFMAs of k-step kk
-    ART_FENCE();
+    load_frags(af1, bf1, as, bs, 1);
+    if (!LAST) store_tiles(buf ^ 1, nxt);
     mfma_all(af0, bf0);
-    ART_FENCE();
-    load_frags(af0, bf0, as, bs, 2);
-    ART_FENCE();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);                   // 12 reads + 8 writes
+      if (i < 4) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    art_lds_barrier();
+    if (!LAST) {
+      load_frags(af0, bf0, As + (buf ^ 1) * A_TILE, Bs + (buf ^ 1) * B_TILE, 0);
+      load_tiles(t + 3 < T ? t + 3 : T - 1, nxt);      // past the end: a harmless repeat of the last tile
+    }
     mfma_all(af1, bf1);
-    ART_FENCE();
-    load_frags(af1, bf1, as, bs, 3);
-    ART_FENCE();
-    mfma_all(af0, bf0);
-    ART_FENCE();
-    mfma_all(af1, bf1);
-    ART_FENCE();
-#undef ART_FENCE
-    if (t + 1 < T) store_tiles(buf ^ 1);
-    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (i < 12) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);      // 12 reads
+      if (i >= 4 && i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using No = std::false_type;
+  // K is a multiple of 64, so T is even.  The last tile stores and reads a repeat of itself: harmless,
+  // and it keeps the loop body free of branches, which the instruction interleaving needs.
+  for (int t = 0; t < T; t += 2) {
+    k_tile(t, S0{}, S1{}, No{});
+    k_tile(t + 1, S1{}, S0{}, No{});
   }
+  __syncthreads();          // every wavefront is done with the operand buffers before they are reused for C
 
   // ---- output: registers -> LDS (fp16, [256][C_LD]) -> 128-bit stores
   _Float16* cs = smem;
@@ -181,7 +220,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
 
 extern "C" int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream) {
   ART_REQUIRE(a_dev && b_dev && c_dev, "art_gemm_f16: null pointer");
-  ART_REQUIRE(M > 0 && N > 0 && K > 0 && M % BM == 0 && N % BN == 0 && K % BK == 0,
+  ART_REQUIRE(M > 0 && N > 0 && K > 0 && M % BM == 0 && N % BN == 0 && K % 64 == 0,
               "art_gemm_f16: M and N must be multiples of 256 and K of 64 (M=%d N=%d K=%d)", M, N, K);
   ART_REQUIRE(((uintptr_t)a_dev % 16) == 0 && ((uintptr_t)b_dev % 16) == 0 && ((uintptr_t)c_dev % 16) == 0,
               "art_gemm_f16: operands must be 16-byte aligned");
