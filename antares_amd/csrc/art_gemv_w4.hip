@@ -237,7 +237,7 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     }
     ss = wave_sum_all(ss);
     if (lane == 0) s_ss[wave] = ss;
-    __syncthreads();
+    art_lds_barrier();      // LDS only: the weight loads issued above stay in flight
     const float r = 1.0f / sqrtf(((s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3])) * fused.inv_n + fused.eps);
     const u32x4* np = reinterpret_cast<const u32x4*>(fused.norm_w + 2 * r0c);
     const u32x4 n0v = np[0], n1v = np[1];
