@@ -119,7 +119,7 @@ struct Fused {
   float inv_n, eps;
 };
 
-template <int M>
+template <int M, int MODE>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused
 __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight, const _Float16* __restrict__ scales,
     const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y, int K, int N, int splits,
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
   // ---- fused RMSNorm, part 1: the loads for the sum of squares go out BEFORE the weight loads.  Loads
   // return in order, so these can be consumed (and the block-wide reduction done) while the weights are
   // still in flight; issued after the weights they would wait for the whole stream.
-  const bool norm = (M == 1) && (fused.norm_w != nullptr);
+  constexpr bool norm = (M == 1) && (MODE == 1);
   u32x4 sq[2];
   if (norm) {
 #pragma unroll
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
 
   // ---- fused SwiGLU, part 1: the column lanes of a k lane share the same 16 values of x, so each
   // computes one pair; its two loads also go out ahead of the weight stream.
-  const bool swiglu = (M == 1) && (fused.gate_up != nullptr);
+  constexpr bool swiglu = (M == 1) && (MODE == 2);
   unsigned int gpair = 0, upair = 0;
   if (swiglu) {
     const int k = 2 * r0c + 2 * cl;
@@ -337,9 +337,16 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
   ART_REQUIRE(ws.base != nullptr, "art_gemv_w4a16: call art_init first");
   ART_REQUIRE(art::kSlotOffset + (size_t)M * N * 8 <= art::kScratchOffset, "art_gemv_w4a16: N too large (%d)", N);
   unsigned long long* slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(ws.base) + art::kSlotOffset);
-  gemv_w4a16_kernel<M><<<dim3(tiles, splits), dim3(kThreads), 0, stream>>>(
-      (const _Float16*)x, (const unsigned char*)qw, (const _Float16*)sc, (const unsigned char*)qz, (_Float16*)y, K, N,
-      splits, slots, Magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u}, fused);
+  const Magic magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+  const dim3 grid(tiles, splits), block(kThreads);
+#define ART_GEMV_LAUNCH(MODE)                                                                                          \
+  gemv_w4a16_kernel<M, MODE><<<grid, block, 0, stream>>>((const _Float16*)x, (const unsigned char*)qw, (const _Float16*)sc, \
+                                                         (const unsigned char*)qz, (_Float16*)y, K, N, splits, slots, magic, fused)
+  // the plain product is its own instantiation: it carries none of the fused prologues
+  if (M == 1 && fused.norm_w != nullptr) ART_GEMV_LAUNCH(1);
+  else if (M == 1 && fused.gate_up != nullptr) ART_GEMV_LAUNCH(2);
+  else ART_GEMV_LAUNCH(0);
+#undef ART_GEMV_LAUNCH
   ART_LAUNCH_CHECK();
   return 0;
 }
