@@ -21,8 +21,9 @@ from .op import ExportedOp, parse_config
 
 
 class _Ops:
-    """``autort.ops.<name>``: operators exported in this process plus the
-    built-in ones."""
+    """``autort.ops.<name>``: operators exported in this process, operators
+    persisted by an earlier session or by the command line (module files, see
+    ``store.py``), and the built-in ones."""
 
     def __init__(self):
         object.__setattr__(self, '_table', {})
@@ -34,7 +35,13 @@ class _Ops:
         table = object.__getattribute__(self, '_table')
         if name in table:
             return table[name]
-        from . import builtin
+        from . import builtin, store
+        record = None if name.startswith('_') else store.load(name)
+        if record is not None:
+            op = ExportedOp(record['ir'], list(record['inputs']), config=record['config'], name=record['name'],
+                            extra_outputs=record['extra_outputs'], tuned=record.get('tuned') or None)
+            table[name] = op
+            return op
         op = builtin.lookup(name)
         if op is None:
             raise AttributeError(f'autort.ops has no operator `{name}`; create it with autort.export(..., name="{name}")')
@@ -42,8 +49,8 @@ class _Ops:
         return op
 
     def __dir__(self):
-        from . import builtin
-        return sorted(set(self._table) | set(builtin.names()))
+        from . import builtin, store
+        return sorted(set(self._table) | set(builtin.names()) | set(store.names()))
 
 
 ops = _Ops()
@@ -55,9 +62,11 @@ def export(ir: str, inputs: Sequence[str] = (), config: Optional[str] = None, na
     calling order as ``"name=dtype[dims]"``; a dimension may be an integer, a
     named run-time dimension with a default (``N:4096``) or a bare name.  The
     operator is also registered as ``autort.ops.<name>`` (default: the name of
-    the last output tensor)."""
+    the last output tensor) and written to a module file, so that later sessions
+    find it under the same name (README.md:75-86)."""
     op = ExportedOp(ir, list(inputs), config=config, name=name, extra_outputs=extra_outputs)
     ops._register(op.name, op)
+    op.persist()
     return op
 
 

@@ -61,8 +61,12 @@ class ExportedOp:
     """One einstein_v2 program bound to gfx950 kernels."""
 
     def __init__(self, ir: str, inputs, config: Optional[str] = None, name: Optional[str] = None,
-                 extra_outputs: Sequence[str] = ()):
+                 extra_outputs: Sequence[str] = (), tuned: Optional[Dict[str, object]] = None):
         self.ir = ir
+        self.input_specs = list(inputs)
+        self.config_text = config
+        self.extra_outputs = list(extra_outputs)
+        self.tuned: Dict[str, object] = dict(tuned or {})    # choices of a tuning run, keyed by kernel
         self.config = parse_config(config)
         self.graph: Graph = parse_program(ir, inputs, extra_outputs)
         self.fused: Graph = fuse_elementwise(self.graph)
@@ -76,6 +80,17 @@ class ExportedOp:
         self._image: Optional[bytes] = None
         from . import patterns
         self.fast_path = patterns.match(self.fused)
+
+    # -- persistence ---------------------------------------------------------
+    def persist(self) -> Optional[str]:
+        """Writes the operator's module file (see store.py); returns its path, or
+        None when the directory is not writable (the operator still works)."""
+        from . import store
+        try:
+            return store.save(self.name, self.ir, self.input_specs, self.config_text, self.extra_outputs,
+                              tuned=self.tuned, source=self.source)
+        except OSError:
+            return None
 
     # -- compilation ---------------------------------------------------------
     def compile(self) -> 'ExportedOp':

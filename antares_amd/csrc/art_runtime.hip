@@ -218,3 +218,27 @@ extern "C" int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, 
   ART_LAUNCH_CHECK();
   return 0;
 }
+
+// ---- device memory for callers that own no allocator (the reference's evaluator; the torch plugin uses torch's)
+extern "C" int art_alloc(size_t bytes, void** out_dev) {
+  ART_REQUIRE(out_dev != nullptr, "art_alloc: null output");
+  *out_dev = nullptr;
+  if (bytes == 0) return 0;
+  ART_HIP(hipMalloc(out_dev, bytes));
+  return 0;
+}
+
+extern "C" int art_free(void* dev) {
+  if (dev) ART_HIP(hipFree(dev));
+  return 0;
+}
+
+extern "C" int art_memcpy_htod(void* dst_dev, const void* src_host, size_t bytes, void* stream) {
+  if (bytes) ART_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+  return 0;
+}
+
+extern "C" int art_memcpy_dtoh(void* dst_host, const void* src_dev, size_t bytes, void* stream) {
+  if (bytes) ART_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+  return 0;
+}

@@ -33,7 +33,7 @@ ART_DEV half_t fp16_ceil(half_t x) { return (half_t)ceilf((float)x); }
 ART_DEV half_t fp16_max(half_t a, half_t b) { return a < b ? b : a; }
 ART_DEV half_t fp16_min(half_t a, half_t b) { return b < a ? b : a; }
 
-// ---- reduce operators ------------------------------------------------------
+// ---- reduce operators
 struct OpAdd { template <class T> ART_MEM T operator()(T a, T b) const { return (T)(a + b); } };
 struct OpMul { template <class T> ART_MEM T operator()(T a, T b) const { return (T)(a * b); } };
 struct OpMax { template <class T> ART_MEM T operator()(T a, T b) const { return a < b ? b : a; } };
@@ -41,7 +41,7 @@ struct OpMin { template <class T> ART_MEM T operator()(T a, T b) const { return 
 struct OpAny { template <class T> ART_MEM T operator()(T a, T b) const { return (T)((a != (T)0) || (b != (T)0)); } };
 struct OpAll { template <class T> ART_MEM T operator()(T a, T b) const { return (T)((a != (T)0) && (b != (T)0)); } };
 
-// ---- wavefront reduction -----------------------------------------------------
+// ---- wavefront reduction
 // 32-bit payloads move through DPP inside each 16-lane row (xor 1, xor 2,
 // half-mirror, mirror), then the four row results are read with v_readlane and
 // combined in a fixed order, so every lane ends with the same, run-to-run

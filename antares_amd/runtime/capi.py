@@ -45,6 +45,10 @@ _SIGNATURES = {
     'art_stream_synchronize': (c_int, [c_void_p]),
     'art_copy_bytes': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     'art_workspace_bytes': (c_size_t, []),
+    'art_alloc': (c_int, [c_size_t, POINTER(c_void_p)]),
+    'art_free': (c_int, [c_void_p]),
+    'art_memcpy_htod': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    'art_memcpy_dtoh': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     'art_gemv_w4a16': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_gemm_w4a16': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_gemv_gptq': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),

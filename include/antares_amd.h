@@ -85,6 +85,15 @@ int art_event_elapsed_ms(void* start, void* stop, float* ms);   /* synchronises 
 int art_event_destroy(void* event);
 int art_stream_synchronize(void* stream);
 
+/* Device memory and host<->device copies for callers that bring no allocator of their own (the
+ * reference's evaluator).  Replace ab::alloc / release / memcpyHtoD / memcpyDtoH (backend.hpp:92-114,
+ * 221-232); the power-of-two bucket cache of ab::alloc stays on the caller's side (include/c-mi355x/backend.hpp).
+ * The copies are asynchronous on `stream`; pair them with art_stream_synchronize. */
+int art_alloc(size_t bytes, void** out_dev);
+int art_free(void* dev);
+int art_memcpy_htod(void* dst_dev, const void* src_host, size_t bytes, void* stream);
+int art_memcpy_dtoh(void* dst_host, const void* src_dev, size_t bytes, void* stream);
+
 /* Plain device copy kernel (dst, src: 16-byte aligned, bytes % 16 == 0); used
  * as the calibration workload for memory-traffic counters. */
 int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* stream);

@@ -83,6 +83,21 @@ int g_threads = 0;
 
 }  // namespace
 
+// The harness's own half conversions (graph_evaluator/execute_module.hpp:46-55): bit moves without
+// rounding, subnormal or zero handling.  They are part of what fill and digest produce - a float 0.0
+// becomes the half 0x4000 (2.0), and the half 0x0000 reads back as 2^-14 - so they are restated as they are.
+static inline float harness_h2f(uint16_t in) {
+  const uint32_t f = ((uint32_t)(in & 0x8000) << 16) | ((((uint32_t)(in & 0x7c00)) + 0x1C000u) << 13) | ((uint32_t)(in & 0x03FF) << 13);
+  float out;
+  memcpy(&out, &f, sizeof(out));
+  return out;
+}
+static inline uint16_t harness_f2h(float in) {
+  uint32_t x;
+  memcpy(&x, &in, sizeof(x));
+  return (uint16_t)(((x >> 16) & 0x8000) | ((((x & 0x7f800000u) - 0x38000000u) >> 13) & 0x7c00) | ((x >> 13) & 0x03ff));
+}
+
 extern "C" {
 
 // Number of worker threads a launch will use (CPU_THREADS env, else all cores).
@@ -115,7 +130,7 @@ int ref_fill(void* data, long long count, const char* dtype, int arg_index) {
   if (!strcmp(dtype, "int32")) { for (long long x = 0; x < count; ++x) ((int*)data)[x] = 0; }
   else if (!strcmp(dtype, "int16")) { for (long long x = 0; x < count; ++x) ((short*)data)[x] = 0; }
   else if (!strcmp(dtype, "int64")) { for (long long x = 0; x < count; ++x) ((long long*)data)[x] = 0; }
-  else if (!strcmp(dtype, "float16")) { for (long long x = 0; x < count; ++x) ((uint16_t*)data)[x] = ref_f2h((float)((x + i + 1) % 71)); }
+  else if (!strcmp(dtype, "float16")) { for (long long x = 0; x < count; ++x) ((uint16_t*)data)[x] = harness_f2h((float)((x + i + 1) % 71)); }
   else if (!strcmp(dtype, "float32")) { for (long long x = 0; x < count; ++x) ((float*)data)[x] = (float)((x + i + 1) % 71); }
   else if (!strcmp(dtype, "float64")) { for (long long x = 0; x < count; ++x) ((double*)data)[x] = (double)((x + i + 1) % 71); }
   else if (!strcmp(dtype, "int8") || !strcmp(dtype, "uint8")) {
@@ -132,7 +147,7 @@ int ref_digest(const void* data, long long count, const char* dtype, double* out
   double d = 0.0;
   if (!strcmp(dtype, "int32")) { for (long long x = 0; x < count; ++x) d += (double)((x + 1) % 83) * ((const int*)data)[x]; }
   else if (!strcmp(dtype, "int64")) { for (long long x = 0; x < count; ++x) d += (double)((x + 1) % 83) * ((const long long*)data)[x]; }
-  else if (!strcmp(dtype, "float16")) { for (long long x = 0; x < count; ++x) d += (double)((x + 1) % 83) * ref_h2f(((const uint16_t*)data)[x]); }
+  else if (!strcmp(dtype, "float16")) { for (long long x = 0; x < count; ++x) d += (double)((x + 1) % 83) * harness_h2f(((const uint16_t*)data)[x]); }
   else if (!strcmp(dtype, "float32")) { for (long long x = 0; x < count; ++x) d += (double)((x + 1) % 83) * ((const float*)data)[x]; }
   else if (!strcmp(dtype, "float64")) { for (long long x = 0; x < count; ++x) d += (double)((x + 1) % 83) * ((const double*)data)[x]; }
   else if (!strcmp(dtype, "int8") || !strcmp(dtype, "uint8") || !strcmp(dtype, "int16")) {

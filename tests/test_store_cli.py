@@ -1,0 +1,106 @@
+"""Persisted operators, the command line and the legacy CustomOp surface (CPU parts: no launch)."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SIGMOID = 'sigmoid_f32[N] = 1 - 1 / (1 + data[N].call(strs.exp))'
+
+
+@pytest.fixture()
+def ops_dir(tmp_path, monkeypatch):
+    monkeypatch.setenv('AUTORT_OPS_DIR', str(tmp_path / 'ops'))
+    monkeypatch.setenv('AUTORT_CACHE_DIR', str(tmp_path / 'cache'))
+    return tmp_path / 'ops'
+
+
+def test_export_writes_a_module_file_and_a_new_session_finds_it(ops_dir):
+    import autort
+    from antares_amd.autort import store
+    op = autort.export(ir=SIGMOID, inputs=['data=float32[N:4096000]'], config='tune:5')
+    path = store.module_path('sigmoid_f32')
+    assert os.path.isfile(path)
+    text = open(path).read()
+    assert text.startswith('// MODULE: ') and '// GLOBALS: ' in text        # record first, kernel container after it
+    record = store.load('sigmoid_f32')
+    assert record['ir'] == SIGMOID and record['inputs'] == ['data=float32[N:4096000]'] and record['config'] == 'tune:5'
+    # a later session: nothing registered in the process, the name resolves from the file
+    fresh = type(autort.ops)()
+    again = fresh.sigmoid_f32
+    assert again is not op and again.ir == SIGMOID and again.declared == ['data']
+    assert 'sigmoid_f32' in dir(fresh)
+    with pytest.raises(AttributeError):
+        fresh.no_such_operator_anywhere
+
+
+def test_module_name_is_checked(ops_dir):
+    from antares_amd.autort import store
+    for bad in ('', '../x', 'a/b', '.hidden'):
+        with pytest.raises(ValueError):
+            store.module_path(bad)
+    assert store.load('../x') is None
+
+
+def test_command_line_creates_the_operator(ops_dir):
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    r = subprocess.run([sys.executable, '-m', 'autort', '--ir', SIGMOID, '-i', 'data=float32[N:4096000]', '-c', 'tune:5'],
+                       cwd=ROOT, env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert 'Module file for operator `sigmoid_f32` has been exported to' in r.stdout
+    assert os.path.isfile(ops_dir / 'sigmoid_f32.mod')
+    bad = subprocess.run([sys.executable, '-m', 'autort', '--ir', 'out[N] = nothing[N', '-i', 'data=float32[N]'],
+                         cwd=ROOT, env=env, capture_output=True, text=True, timeout=300)
+    assert bad.returncode == 1 and 'autort:' in bad.stderr
+
+
+def test_custom_op_emit_reports_outputs(ops_dir):
+    from antares_amd.autort.custom_op import CustomOp
+    a = torch.zeros(8, 16)
+    with pytest.raises(RuntimeError):
+        CustomOp(ir='out[N, M] = a[N, M] + b[N, M]', input_orders={'a': a, 'b': a})      # device=None means CPU: refused
+    op = CustomOp(ir='mid[N, M] = a[N, M] * 2; out[N] +=! mid[N, M] * b[N, M]',
+                  input_orders={'a': a, 'b': ('b', torch.float32, [8, 16])}, extra_outputs=['mid'],
+                  device=torch.device('cuda')).tune(step=0).emit()
+    assert op.output_names == ['mid', 'out'] or op.output_names == ['out', 'mid']
+    infos = {n: (dt, shp) for n, dt, shp in op.output_infos}
+    assert infos['out'] == (torch.float32, [8]) and infos['mid'] == (torch.float32, [8, 16])
+    assert op.kernel_sources.startswith('// GLOBALS: ')
+    assert isinstance(op.custom_key, int)
+    with pytest.raises(Exception, match='Deprecated Usage'):
+        op.to('cuda')
+
+
+@pytest.mark.gpu
+def test_persisted_operator_runs_in_a_fresh_process(ops_dir):
+    """README.md:75-86: create on the command line, use from a later session."""
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    r = subprocess.run([sys.executable, '-m', 'autort', '--ir', SIGMOID, '-i', 'data=float32[N:4096000]', '-c', 'tune:5'],
+                       cwd=ROOT, env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    code = ('import torch, autort\n'
+            'data = torch.arange(0, 10, dtype=torch.float32, device=autort.device())\n'
+            'print(["%.4f" % v for v in autort.ops.sigmoid_f32(data).tolist()])\n')
+    r = subprocess.run([sys.executable, '-c', code], cwd=ROOT, env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    want = ['0.5000', '0.7311', '0.8808', '0.9526', '0.9820', '0.9933', '0.9975', '0.9991', '0.9997', '0.9999']   # README.md:68
+    assert str(want) in r.stdout
+
+
+@pytest.mark.gpu
+def test_custom_op_forward_matches_torch(ops_dir):
+    from antares_amd.autort.custom_op import CustomOp
+    import autort
+    dev = autort.device()
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(64, 48, generator=g).to(dev)
+    b = torch.randn(64, 48, generator=g).to(dev)
+    op = CustomOp(ir='mid[N, M] = a[N, M] * 2; out[N] +=! mid[N, M] * b[N, M]', input_orders={'a': a, 'b': b},
+                  extra_outputs=['mid'], device=dev).tune(step=0).emit()
+    outs = dict(zip(op.output_names, op(a, b)))
+    assert torch.allclose(outs['mid'], a * 2)
+    assert torch.allclose(outs['out'], (a * 2 * b).sum(1), rtol=1e-5, atol=1e-5)
+    single = CustomOp(ir='out[N, M] = a[N, M] + b[N, M]', input_orders={'a': a, 'b': b}, device=dev).emit()
+    assert torch.equal(single(a, b), a + b)
