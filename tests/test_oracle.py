@@ -170,8 +170,14 @@ def test_fill_and_digest_closed_form():
     a = fill(np.zeros(1000, np.float32), 'float32', 2)
     assert np.array_equal(a, (np.arange(1000) + 3) % 71)
     assert np.array_equal(fill(np.ones(10, np.int32), 'int32', 0), np.zeros(10))
+    # the harness converts with bare bit moves (execute_module.hpp:46-55): exact for 1..70, but a float 0.0
+    # becomes the half 0x4000 = 2.0, and a half 0x0000 is read back as 2^-15 by the digest
     h = fill(np.zeros(100, np.float16), 'float16', 0)
-    assert np.array_equal(h.astype(np.float32), (np.arange(100) + 1) % 71)
+    want16 = ((np.arange(100) + 1) % 71).astype(np.float32)
+    want16[want16 == 0] = 2.0
+    assert np.array_equal(h.astype(np.float32), want16) and h[70] == 2.0
+    assert digest(np.zeros(10, np.float16), 'float16') == pytest.approx(sum(range(1, 11)) * 2.0 ** -15, rel=1e-12)
+    assert digest(np.full(4, 1.5, np.float16), 'float16') == pytest.approx(1.5 * (1 + 2 + 3 + 4), rel=1e-12)
     out = np.linspace(-1, 1, 500).astype(np.float32)
     want = float(np.sum(((np.arange(500) + 1) % 83) * out.astype(np.float64)))
     assert digest(out, 'float32') == pytest.approx(want, rel=1e-12)
