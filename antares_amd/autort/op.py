@@ -159,16 +159,55 @@ class ExportedOp:
         module = self._load()
         g = self.fused
         dims = [env[d] for d in g.dim_names]
+        trials = self.config.get('tune')
+        trials = trials if isinstance(trials, int) and trials > 0 else 0
         for plan in self.plans:
             for n in plan.args:
                 if n not in bound:         # intermediate (reduce result) of a multi-kernel program
                     bound[n] = torch.empty(g.shape_of(n, env), dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)
             ptrs = {n: bound[n].data_ptr() for n in plan.args}
-            sym, grid, block = plan.choose(env, ptrs)
+            key = plan.name + '|' + ','.join(str(v) for v in dims) + '|' + ''.join('a' if ptrs[n] % 16 == 0 else 'u' for n in plan.args)
+            saved = self.tuned.get(key)
+            if saved is None and trials and not torch.cuda.is_current_stream_capturing():
+                saved = self._tune(plan, key, bound, dims, ptrs, env, module, trials)
+            if saved is not None and saved['variant'] in plan.variants:
+                sym, grid, block = plan.variants[saved['variant']], int(saved['grid']), 256
+            else:
+                sym, grid, block = plan.choose(env, ptrs)
             if grid == 0:
                 continue
             capi.launch(module.function(sym), (grid, 1, 1), (block, 1, 1), stream,
                         [ptrs[n] for n in plan.args] + dims)
+
+    def _tune(self, plan, key: str, bound, dims, ptrs, env, module, trials: int):
+        """``config="tune:N"``: times up to N launch configurations of one kernel for the extents of this call
+        (the reference searches its schedule space with OpEvo, tuner/OpEvo/main.py:467-616, N steps at a time;
+        the space here is small - kernel variant x grid size - so the walk is: the heuristic choice first, then
+        its neighbours, best first).  Written tensors are replaced by scratch copies while timing, so programs
+        that accumulate into their output are not disturbed.  The winner is kept in the module file."""
+        cands = plan.candidates(env, ptrs)
+        if len(cands) <= 1:
+            return None
+        base_sym, base_grid, _ = plan.choose(env, ptrs)
+        cands.sort(key=lambda c: (c[1] != base_sym, abs(c[2] - base_grid)))      # heuristic first, then nearest
+        scratch = {n: (torch.empty_like(bound[n]) if n == plan.output or n in self.inout else bound[n]) for n in plan.args}
+        args = [scratch[n].data_ptr() for n in plan.args] + dims
+        stream = current_stream_handle()
+        best = None
+        for tag, sym, grid in cands[:trials]:
+            fn = module.function(sym)
+            capi.launch(fn, (grid, 1, 1), (256, 1, 1), stream, args)            # warm-up
+            start, stop = capi.Event(), capi.Event()
+            start.record(stream)
+            for _ in range(5):
+                capi.launch(fn, (grid, 1, 1), (256, 1, 1), stream, args)
+            stop.record(stream)
+            us = start.elapsed_ms(stop) * 200.0
+            if best is None or us < best['us']:
+                best = {'variant': tag, 'grid': grid, 'us': round(us, 3)}
+        self.tuned[key] = best
+        self.persist()
+        return best
 
     def __repr__(self):
         return f'<autort op {self.name}: {" ".join(self.ir.split())[:80]}>'

@@ -161,6 +161,39 @@ class KernelPlan:
         return self.variants['thread'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
 
 
+    def candidates(self, env: Dict[str, int], pointers: Dict[str, int]) -> List[Tuple[str, str, int]]:
+        """Every launch configuration that computes the same result for these extents and addresses:
+        (variant tag, kernel symbol, grid.x).  All kernels are grid-stride, so any grid is valid; the
+        candidates cover each applicable variant at the heuristic grid and at smaller power-of-two caps."""
+        total = 1
+        for _, e in self.data_axes:
+            total *= e if isinstance(e, int) else env[e]
+        if total == 0:
+            return []
+        tags = []
+        if self.kind == 'map':
+            if 'vec' in self.variants and all(pointers[t] % 16 == 0 for t in self.vec_tensors) and total >= self.vec:
+                tags.append(('vec', (total + self.vec - 1) // self.vec))
+            tags.append(('scalar', total))
+        elif self.kind == 'scatter':
+            tags.append(('scalar', total))
+        else:
+            waves_per_block = BLOCK // 64
+            tags += [('thread', total), ('wave', (total + waves_per_block - 1) // waves_per_block * BLOCK), ('block', total * BLOCK)]
+        out = []
+        for tag, work in tags:
+            if tag not in self.variants:
+                continue
+            full = max(1, min((work + BLOCK - 1) // BLOCK, MAX_GRID))
+            grids = {full}
+            cap = 256
+            while cap < full:
+                grids.add(cap)
+                cap *= 2
+            out += [(tag, self.variants[tag], g) for g in sorted(grids, reverse=True)]
+        return out
+
+
 def _signature(name: str, args: List[str], tensors, dims: List[str], written: List[str]) -> str:
     ps = []
     for a in args:

@@ -257,8 +257,10 @@ def main():
                           'roofline_frac': round(r['gbps'] / HBM_PEAK_GBPS, 4)})
         for (k, n) in [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 32000)]:
             r = bench_gemv(torch, autort, capi, workloads, k, n, 64, max(10, args.steps // 2), args.warmup, args.seed, layers=8)
+            tflops = 2.0 * 64 * k * n / (r['us_per_launch'] * 1e-6) / 1e12
             extra.append({'workload': r['workload'], 'us_per_launch': round(r['us_per_launch'], 3), 'gbps': round(r['gbps'], 1),
-                          'roofline_frac': round(r['gbps'] / HBM_PEAK_GBPS, 4)})
+                          'roofline_frac': round(r['gbps'] / HBM_PEAK_GBPS, 4), 'tflops': round(tflops, 1),
+                          'mfma_frac': round(tflops / MFMA_F16_PEAK_TFLOPS, 4)})
         for n in (4096, 8192):
             r = bench_gemm_f16(torch, autort, capi, workloads, max(5, args.steps // 4), args.warmup, args.seed, n)
             extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})

@@ -104,3 +104,33 @@ def test_custom_op_forward_matches_torch(ops_dir):
     assert torch.allclose(outs['out'], (a * 2 * b).sum(1), rtol=1e-5, atol=1e-5)
     single = CustomOp(ir='out[N, M] = a[N, M] + b[N, M]', input_orders={'a': a, 'b': b}, device=dev).emit()
     assert torch.equal(single(a, b), a + b)
+
+
+@pytest.mark.gpu
+def test_tune_config_times_candidates_and_keeps_the_winner(ops_dir):
+    """config="tune:N" (README.md:66): the first call searches launch configurations, the choice is stored in the
+    module file and reused by later sessions; results are the same before and after."""
+    import autort
+    from antares_amd.autort import store
+    dev = autort.device()
+    x = (torch.rand(1_000_000, generator=torch.Generator().manual_seed(0)) * 16 - 8).to(dev)
+    plain = autort.export(ir=SIGMOID, inputs=['data=float32[N:4096000]'], name='sigmoid_plain')
+    tuned = autort.export(ir=SIGMOID, inputs=['data=float32[N:4096000]'], config='tune:6', name='sigmoid_tuned')
+    want = plain(x)
+    got = tuned(x)
+    assert torch.equal(got, want)
+    assert len(tuned.tuned) == 1
+    (key, choice), = tuned.tuned.items()
+    assert key.startswith('autort_sigmoid_tuned_k0|1000000|') and choice['variant'] in ('vec', 'scalar') and choice['grid'] >= 1
+    assert store.load('sigmoid_tuned')['tuned'] == tuned.tuned
+    # a later session starts from the stored choice and does not search again
+    again = type(autort.ops)().sigmoid_tuned
+    assert again.tuned == tuned.tuned
+    assert torch.equal(again(x), want) and again.tuned == tuned.tuned
+    # a program that accumulates into an in-out tensor is timed on scratch copies, not on the live tensor
+    acc = autort.export(ir='hist[data[N] % 16] +=. one[0]', inputs=['data=int32[N]', 'one=int32[1]', 'hist=int32[16]'],
+                        config='tune:4', name='hist_tuned')
+    data = torch.arange(4096, dtype=torch.int32, device=dev)
+    hist = torch.zeros(16, dtype=torch.int32, device=dev)
+    acc(data, torch.ones(1, dtype=torch.int32, device=dev), hist)
+    assert hist.tolist() == [256] * 16
