@@ -3,12 +3,13 @@
 // Replaces the reference's three-step pipeline of samples/01_sort_even_first.py:9-27
 // (classify scatter into a [2,N] flag plane, torch cumsum over 2N flags, bucket
 // scatter; about 64 bytes of traffic per element) by two launches that move
-// 12 bytes per element and need no atomics, fences or zeroed state:
+// 12 bytes per element and need no atomics, fences or zeroed state (the barriers
+// inside the scatter kernel order LDS only, so the next tile's loads stay in flight):
 //
 //   count    block b reads its span of the input (a whole number of
 //            4096-element tiles) and stores the number of even values in
 //            counts[b].
-//   scatter  block b adds up counts[0..b) and counts[b..B) (B <= 8192 words,
+//   scatter  block b adds up counts[0..b) and counts[b..B) (B <= 1024 words,
 //            served by L2) to get the number of evens before its span and the
 //            total; then, tile by tile, it ranks the even values with a
 //            wavefront prefix + a 4-wave prefix through LDS, compacts evens
@@ -51,11 +52,16 @@ __global__ __launch_bounds__(kThreads) void partition_count_kernel(const int* __
   __shared__ unsigned int s_wave[4];
   const int tid = threadIdx.x;
   unsigned int c = 0;
-  for (int s = 0; s < tiles_per_block; ++s) {
-    const long long base = ((long long)blockIdx.x * tiles_per_block + s) * kTile;
-    if (base >= n) break;
+  const long long first = (long long)blockIdx.x * tiles_per_block * kTile;
+  for (int s = 0; s < tiles_per_block; s += 2) {       // two tiles (eight 16-byte loads per thread) in flight at a time
+    i32x4 a[kVecPerThread], b2[kVecPerThread];
+    const long long base = first + (long long)s * kTile;
 #pragma unroll
-    for (int j = 0; j < kVecPerThread; ++j) c += even_count4(load_vec(in, base, j, n));
+    for (int j = 0; j < kVecPerThread; ++j) a[j] = load_vec(in, base, j, n);                 // past n: reads as odd, counts 0
+#pragma unroll
+    for (int j = 0; j < kVecPerThread; ++j) b2[j] = (s + 1 < tiles_per_block) ? load_vec(in, base + kTile, j, n) : i32x4{1, 1, 1, 1};
+#pragma unroll
+    for (int j = 0; j < kVecPerThread; ++j) c += even_count4(a[j]) + even_count4(b2[j]);
   }
 #pragma unroll
   for (int m = 1; m < 64; m <<= 1) c += __shfl_xor(c, m, 64);
@@ -92,16 +98,19 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
     total_sum += __shfl_xor(total_sum, m, 64);
   }
   if (lane == 0) { s_sum[wave][0] = before_sum; s_sum[wave][1] = total_sum; }
-  __syncthreads();
+  art_lds_barrier();
   long long even_before = (long long)(s_sum[0][0] + s_sum[1][0] + s_sum[2][0] + s_sum[3][0]);
   const long long total_even = (long long)(s_sum[0][1] + s_sum[1][1] + s_sum[2][1] + s_sum[3][1]);
 
   for (int s = 0; s < tiles_per_block; ++s) {
     const long long base = span_base + (long long)s * kTile;
     if (base >= n) break;
-    if (s > 0) {
+    // the next tile's loads go out before this tile is ranked and written
+    i32x4 vn[kVecPerThread];
+    const bool more = (s + 1 < tiles_per_block) && (base + kTile < n);
+    if (more) {
 #pragma unroll
-      for (int j = 0; j < kVecPerThread; ++j) v[j] = load_vec(in, base, j, n);
+      for (int j = 0; j < kVecPerThread; ++j) vn[j] = load_vec(in, base + kTile, j, n);
     }
     const long long valid = (n - base < kTile) ? (n - base) : kTile;      // elements of this tile that exist
     unsigned int cnt[kVecPerThread], incl[kVecPerThread];
@@ -118,7 +127,7 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
       incl[j] = p;
       if (lane == 63) s_wave[wave][j] = p;
     }
-    __syncthreads();
+    art_lds_barrier();
     // evens before (j, wave, lane) in tile order (j outermost, then thread id)
     unsigned int tile_even = 0, before[kVecPerThread];
 #pragma unroll
@@ -145,13 +154,17 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
         ev += is_even ? 1u : 0u;
       }
     }
-    __syncthreads();
+    art_lds_barrier();
     const long long odd_base = total_even + (base - even_before);
     const unsigned int tile_odd = (unsigned int)valid - tile_even;     // padding was counted as odd and sits last
     for (unsigned int i = tid; i < tile_even; i += kThreads) out[even_before + i] = s_items[i];
     for (unsigned int i = tid; i < tile_odd; i += kThreads) out[odd_base + i] = s_items[tile_even + i];
     even_before += tile_even;
-    __syncthreads();                                            // s_items / s_wave are reused by the next tile
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < kVecPerThread; ++j) v[j] = vn[j];
+    }
+    art_lds_barrier();                                            // s_items / s_wave are reused by the next tile
   }
 }
 
@@ -165,7 +178,7 @@ extern "C" int art_partition_even_first_i32(const void* in_dev, void* out_dev, l
   art::Workspace& ws = art::workspace();
   ART_REQUIRE(ws.base != nullptr, "art_partition_even_first_i32: call art_init first");
   const long long tiles = (n + kTile - 1) / kTile;
-  constexpr long long kMaxBlocks = 8192;                        // bounds the counts every block adds up
+  constexpr long long kMaxBlocks = 1024;                        // bounds the counts every block adds up (4 KiB from L2)
   const int tiles_per_block = (int)((tiles + kMaxBlocks - 1) / kMaxBlocks);
   const int blocks = (int)((tiles + tiles_per_block - 1) / tiles_per_block);
   unsigned int* counts = reinterpret_cast<unsigned int*>(reinterpret_cast<char*>(ws.base) + art::kScratchOffset);

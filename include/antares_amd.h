@@ -144,7 +144,8 @@ int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, int M, int N
 
 /* Stable even-first partition of int32 values: all even values in input order,
  * then all odd values in input order.  Two launches (count, then rank + scatter),
- * 12 bytes of traffic per element, no atomics.
+ * 12 bytes of traffic per element, no atomics; at most 1024 blocks, each walking its span tile by tile
+ * with the next tile's loads in flight.
  * Replaces the classify -> cumsum -> bucket pipeline of
  * samples/01_sort_even_first.py:9-27. */
 int art_partition_even_first_i32(const void* in_dev, void* out_dev, long long n, void* stream);
