@@ -5,18 +5,21 @@
 // dequant + matmul program of samples/05_llama2_7b_int4.py:135-144 is exported with a batch axis.
 //
 // Design for MI355X:
-//   * the weights are read from HBM exactly once; a work item owns 128 columns (one full 128-byte line
-//     of every packed row) and a contiguous range of k groups, and streams them two groups ahead;
+//   * the weights are read from HBM exactly once; a block owns 128 columns (one full 128-byte line of
+//     every packed row) and a contiguous range of k groups;
 //   * unpacking is fused into the LDS staging: 16 bytes (16 columns x 2 k) become two rows of fp16
-//     (q - z) values - exact small integers - with one shift, four and-or and four packed subtractions
-//     per word.  The columns of every group of four land in LDS in the order 0,2,1,3, which costs nothing:
-//     the column an accumulator lane owns is permuted the same way and undone in the epilogue;
+//     (q - z) values - exact small integers - with one shift, four v_bitop3_b32 and four packed
+//     subtractions per word.  The columns of every group of four land in LDS in the order 0,2,1,3,
+//     which costs nothing: the column an accumulator lane owns is permuted the same way and undone
+//     in the epilogue;
 //   * v_mfma_f32_32x32x16_f16 per wave: 32 columns x 64 rows, B operand through ds_read_b64_tr_b16;
 //     the group sum is scaled by s[g,n] in fp32 afterwards (one scalar per lane, since an accumulator
 //     lane owns one column), so no scale is rounded to fp16;
-//   * a block is two independent work items of four waves each that alternate phases: while one half
-//     unpacks its next group on the vector units, the other half multiplies its current group on the
-//     matrix cores.  One wave of each half sits on every SIMD, so both pipes stay busy;
+//   * a step is 64 k.  LDS holds two steps: while the matrix cores work on step t, the same waves
+//     unpack step t+1 into the other buffer; one barrier per step, and it waits for LDS only, so the
+//     register stages (a whole group = two steps each, two of them) keep their global loads in flight
+//     across it.  58 KiB of LDS and < 256 registers: two blocks per compute unit, whose phases drift
+//     apart and fill each other's gaps;
 //   * split-K without atomics (5.6 M float atomics cost 75 us on this chip): each K-split writes its
 //     fp32 tile to the library workspace and a second small kernel adds the splits in a fixed order
 //     and rounds once to fp16 - results do not depend on timing.
@@ -36,12 +39,13 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
-constexpr int BM = 64, BN = 128, GK = 128;     // rows, columns and k per staged tile
+constexpr int BM = 64, BN = 128, GK = 128;     // rows and columns of a block, k of a quantisation group
+constexpr int SK = 64;                         // k of a step (half a group)
 constexpr int W_LD = BN + 32;                  // halves per weight row in LDS: 320 bytes, so the four k rows
                                                // a transposing read touches fall on disjoint banks
-constexpr int X_LD = GK + 8;                   // halves per x row in LDS (272 bytes)
-constexpr int HALF_LDS = GK * W_LD + BM * X_LD;                 // halves of LDS per work item
-constexpr size_t kLdsBytes = (size_t)2 * HALF_LDS * sizeof(_Float16);
+constexpr int X_LD = SK + 8;                   // halves per x row in LDS (144 bytes)
+constexpr int W_TILE = SK * W_LD, X_TILE = BM * X_LD;
+constexpr size_t kLdsBytes = (size_t)2 * (W_TILE + X_TILE) * sizeof(_Float16);
 
 struct Magic {
   unsigned int mask_lo, mask_hi, bias_lo, bias_hi;   // 0x000F000F 0x00F000F0 0x64006400 0x54005400
@@ -59,46 +63,36 @@ __device__ __forceinline__ unsigned int and_or(unsigned int w, unsigned int mask
 __device__ __forceinline__ int unpermute(int p) { return (p & ~3) | ((p & 1) << 1) | ((p >> 1) & 1); }
 
 template <int MT>   // MT accumulator tiles of 32 rows: 1 for M <= 32, 2 for M <= 64
-__global__ __launch_bounds__(512) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
-                                                          const _Float16* __restrict__ scales,
-                                                          const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y,
-                                                          float* __restrict__ partial, int M, int K, int N, int splits,
-                                                          int col_tiles, Magic mg) {
+__global__ __launch_bounds__(256, 2) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
+                                                             const _Float16* __restrict__ scales,
+                                                             const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y,
+                                                             float* __restrict__ partial, int M, int K, int N, int splits,
+                                                             int col_tiles, Magic mg) {
   extern __shared__ __align__(16) _Float16 smem[];
-  const int half = threadIdx.x >> 8;             // which of the block's two work items this wave serves
-  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
-  _Float16* Ws = smem + half * HALF_LDS;         // [GK][W_LD]
-  _Float16* Xs = Ws + GK * W_LD;                 // [BM][X_LD]
+  _Float16* Ws = smem;                           // [2][SK][W_LD]
+  _Float16* Xs = smem + 2 * W_TILE;              // [2][BM][X_LD]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-  // work item -> (column tile, K split); the two halves of a block take neighbouring column tiles
-  const int G = K / GK, items = col_tiles * splits;
-  auto group_range = [&](int item, int& begin, int& end) {
-    const int split = item / col_tiles;
-    begin = item < items ? (int)((long long)G * split / splits) : 0;
-    end = item < items ? (int)((long long)G * (split + 1) / splits) : 0;
-  };
-  const int item = blockIdx.x * 2 + half;
-  int g_begin, g_end, o_begin, o_end;
-  group_range(item, g_begin, g_end);
-  group_range(blockIdx.x * 2 + (1 - half), o_begin, o_end);
-  const int steps = g_end - g_begin;
-  const int T = steps > o_end - o_begin ? steps : o_end - o_begin;      // both halves pass the same barriers
-  const int split = item / col_tiles;
-  const int n0 = (item % col_tiles) * BN;
+  // block -> (column tile, K split)
+  const int G = K / GK;
+  const int split = blockIdx.x / col_tiles;
+  const int n0 = (blockIdx.x % col_tiles) * BN;
+  const int g_begin = (int)((long long)G * split / splits), g_end = (int)((long long)G * (split + 1) / splits);
+  const int groups = g_end - g_begin;
 
-  // ---- global -> register staging
-  // weights: 64 packed rows x 128 bytes per group = 512 chunks of 16 bytes, two per thread
+  // ---- global -> register staging, one quantisation group (two steps) per stage
+  // weights of a step: 32 packed rows x 128 bytes = 256 chunks of 16 bytes, one per thread
   const int cc = tid & 7;                       // 16-column chunk
-  const int pr = tid >> 3;                      // packed row (+32 for the second chunk)
+  const int pr = tid >> 3;                      // packed row of the step
   const bool col_ok = n0 + cc * 16 < N;         // N % 16 == 0: a chunk is inside or outside as a whole
-  const int wcol = col_ok ? n0 + cc * 16 : 0;
+  const int wcol = col_ok ? n0 + cc * 16 : 0;   // columns past N: load valid memory, results are never stored
   const unsigned char* wp = qweight + (size_t)pr * N + wcol;
-  // x: MT*32 rows x 128 k = MT*512 chunks of 16 bytes, 2*MT per thread; rows past M repeat row M-1
-  const _Float16* xp[2 * MT];
-  int xs_off[2 * MT];
+  // x of a step: MT*32 rows x 64 k = MT*256 chunks of 16 bytes, MT per thread; rows past M repeat row M-1
+  const _Float16* xp[MT];
+  int xs_off[MT];
 #pragma unroll
-  for (int i = 0; i < 2 * MT; ++i) {
-    const int c = tid + 256 * i, row = c >> 4, kc = c & 15;
+  for (int i = 0; i < MT; ++i) {
+    const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
     xp[i] = x + (size_t)(row < M ? row : M - 1) * K + kc * 8;
     xs_off[i] = row * X_LD + kc * 8;
   }
@@ -112,37 +106,32 @@ __global__ __launch_bounds__(512) void gemm_w4a16_kernel(const _Float16* __restr
   const bool my_ok = my_col < N;
   const int sc_col = my_ok ? my_col : 0;
 
-  // Two register stages: the loads of group g + 2 are issued while group g is unpacked.
   // Stages are indexed statically (a run-time index would put the arrays in scratch memory).
-  u32x4 wq[2][2];      // [stage][chunk]
-  u32x4 xr[2][2 * MT];
+  u32x4 wq[2][2];      // [stage][step of the group]
+  u32x4 xr[2][2][MT];
   u32x2 zq[2];
   _Float16 sc16[2];
-  auto load_stage = [&](int g, auto tag) {
+  auto load_group = [&](int g, auto tag) {
     constexpr int S = decltype(tag)::value;
 #pragma unroll
-    for (int i = 0; i < 2 * MT; ++i) xr[S][i] = *reinterpret_cast<const u32x4*>(xp[i] + (size_t)g * GK);
-    const unsigned char* p = wp + (size_t)g * (GK / 2) * N;
-    wq[S][0] = *reinterpret_cast<const u32x4*>(p);
-    wq[S][1] = *reinterpret_cast<const u32x4*>(p + (size_t)32 * N);
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) xr[S][h][i] = *reinterpret_cast<const u32x4*>(xp[i] + (size_t)g * GK + h * SK);
+      wq[S][h] = *reinterpret_cast<const u32x4*>(wp + ((size_t)g * (GK / 2) + h * (SK / 2)) * N);
+    }
     zq[S] = *reinterpret_cast<const u32x2*>(qzeros + (size_t)g * (N / 2) + (wcol >> 1));
     sc16[S] = scales[(size_t)g * N + sc_col];
   };
 
-  f16v total[MT];
+  f16v total[MT], grp[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) total[i][r] = 0.f;
-  float sc_staged = 0.f;     // scale of the group that currently sits in LDS
 
-  // Phase D: unpack step i of this work item into LDS and refill its register stage.
-  auto unpack = [&](int i, auto tag) {
+  h2 z_lo[8], z_hi[8];   // zero points of this thread's 16 columns, paired (c0,c2) and (c1,c3), on both nibble biases
+  auto prepare_zeros = [&](auto tag) {
     constexpr int S = decltype(tag)::value;
-    if (i >= steps) return;
-    sc_staged = my_ok ? (float)sc16[S] : 0.f;
-    // zero points of this thread's 16 columns, paired (c0,c2) and (c1,c3), on both nibble biases
-    h2 z_lo[8], z_hi[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const unsigned int zw = (zq[S][j >> 1] >> ((j & 1) * 16)) & 0xffffu;   // z0 | z1<<4 | z2<<8 | z3<<12
@@ -153,83 +142,134 @@ __global__ __launch_bounds__(512) void gemm_w4a16_kernel(const _Float16* __restr
       z_hi[2 * j] = as_h2(and_or(e << 4, mg.mask_hi, mg.bias_hi));
       z_hi[2 * j + 1] = as_h2(and_or(o << 4, mg.mask_hi, mg.bias_hi));
     }
-    // chunk c holds packed row pr + 32c = k rows 2*(pr+32c) and 2*(pr+32c)+1
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      u32x4 even[2], odd[2];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const unsigned int w = wq[S][c][j], w8 = w >> 8;    // columns past N hold finite garbage and are never stored
-        const h2 e02 = as_h2(and_or(w, mg.mask_lo, mg.bias_lo)) - z_lo[2 * j];
-        const h2 e13 = as_h2(and_or(w8, mg.mask_lo, mg.bias_lo)) - z_lo[2 * j + 1];
-        const h2 o02 = as_h2(and_or(w, mg.mask_hi, mg.bias_hi)) - z_hi[2 * j];
-        const h2 o13 = as_h2(and_or(w8, mg.mask_hi, mg.bias_hi)) - z_hi[2 * j + 1];
-        even[j >> 1][(j & 1) * 2] = as_u32(e02);
-        even[j >> 1][(j & 1) * 2 + 1] = as_u32(e13);
-        odd[j >> 1][(j & 1) * 2] = as_u32(o02);
-        odd[j >> 1][(j & 1) * 2 + 1] = as_u32(o13);
-      }
-      _Float16* row = Ws + (2 * (pr + 32 * c)) * W_LD + cc * 16;
-      *reinterpret_cast<u32x4*>(row) = even[0];
-      *reinterpret_cast<u32x4*>(row + 8) = even[1];
-      *reinterpret_cast<u32x4*>(row + W_LD) = odd[0];
-      *reinterpret_cast<u32x4*>(row + W_LD + 8) = odd[1];
-    }
-#pragma unroll
-    for (int j = 0; j < 2 * MT; ++j) *reinterpret_cast<u32x4*>(Xs + xs_off[j]) = xr[S][j];
-    if (i + 2 < steps) load_stage(g_begin + i + 2, tag);     // refill the stage just consumed
   };
+  // Unpack one step (half H of the group in stage S) into LDS buffer `buf`.
+  auto unpack = [&](int buf, auto tag, auto half_tag) {
+    constexpr int S = decltype(tag)::value, H = decltype(half_tag)::value;
+    u32x4 even[2], odd[2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const unsigned int w = wq[S][H][j], w8 = w >> 8;
+      const h2 e02 = as_h2(and_or(w, mg.mask_lo, mg.bias_lo)) - z_lo[2 * j];
+      const h2 e13 = as_h2(and_or(w8, mg.mask_lo, mg.bias_lo)) - z_lo[2 * j + 1];
+      const h2 o02 = as_h2(and_or(w, mg.mask_hi, mg.bias_hi)) - z_hi[2 * j];
+      const h2 o13 = as_h2(and_or(w8, mg.mask_hi, mg.bias_hi)) - z_hi[2 * j + 1];
+      even[j >> 1][(j & 1) * 2] = as_u32(e02);
+      even[j >> 1][(j & 1) * 2 + 1] = as_u32(e13);
+      odd[j >> 1][(j & 1) * 2] = as_u32(o02);
+      odd[j >> 1][(j & 1) * 2 + 1] = as_u32(o13);
+    }
+    _Float16* row = Ws + buf * W_TILE + (2 * pr) * W_LD + cc * 16;       // packed row pr = k rows 2*pr, 2*pr+1 of the step
+    *reinterpret_cast<u32x4*>(row) = even[0];
+    *reinterpret_cast<u32x4*>(row + 8) = even[1];
+    *reinterpret_cast<u32x4*>(row + W_LD) = odd[0];
+    *reinterpret_cast<u32x4*>(row + W_LD + 8) = odd[1];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) *reinterpret_cast<u32x4*>(Xs + buf * X_TILE + xs_off[i]) = xr[S][H][i];
+  };
+  // Operand fragments of two k-steps of 16 (kk0, kk0 + 1) of the step in LDS buffer `buf`.
+  auto read_frags = [&](h8 (&fa)[2][MT], h8 (&fb)[2], int buf, int kk0) {
+    const _Float16* ws = Ws + buf * W_TILE;
+    const _Float16* xs = Xs + buf * X_TILE;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const _Float16* p = ws + ((kk0 + k) * 16 + b_k) * W_LD + b_n;
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * W_LD));
+      const h4 l4 = __builtin_bit_cast(h4, lo), h4v = __builtin_bit_cast(h4, hi);
+      fb[k] = h8{l4[0], l4[1], l4[2], l4[3], h4v[0], h4v[1], h4v[2], h4v[3]};
+#pragma unroll
+      for (int t = 0; t < MT; ++t) fa[k][t] = *reinterpret_cast<const h8*>(xs + (a_row + t * 32) * X_LD + (kk0 + k) * 16 + a_k);
+    }
+  };
+  auto mfma2 = [&](const h8 (&fa)[2][MT], const h8 (&fb)[2]) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) grp[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[k][t], fb[k], grp[t], 0, 0, 0);
+  };
+  // Scheduling masks of sched_group_barrier: 0x008 MFMA, 0x002 VALU, 0x100 LDS read, 0x200 LDS write, 0x020 global load.
+  // First half of a step: the MFMAs of k-steps 0,1 with, between them, the operand reads of k-steps 2,3 and the
+  // unpacking of the next step into the other buffer.
+#define ART_FIRST_HALF()                                        \
+  do {                                                          \
+    __builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * MT, 0); \
+    for (int m_ = 0; m_ < 2 * MT; ++m_) {                       \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
+      __builtin_amdgcn_sched_group_barrier(0x002, 24, 0);       \
+    }                                                           \
+    __builtin_amdgcn_sched_group_barrier(0x200, 4 + MT, 0);     \
+    __builtin_amdgcn_sched_barrier(0);                          \
+  } while (0)
+  // Second half: the MFMAs of k-steps 2,3 with the first operand reads of the next step (and the global loads) between them.
+#define ART_SECOND_HALF()                                       \
+  do {                                                          \
+    __builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * MT, 0); \
+    for (int m_ = 0; m_ < 2 * MT; ++m_) {                       \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
+      __builtin_amdgcn_sched_group_barrier(0x020, 3, 0);        \
+    }                                                           \
+    __builtin_amdgcn_sched_barrier(0);                          \
+  } while (0)
 
-  // Phase M: multiply the group that sits in LDS (step i) and add it, scaled, to the totals.
-  auto multiply = [&](int i) {
-    if (i < 0 || i >= steps) return;
-    f16v grp[MT];
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  using H0 = std::integral_constant<int, 0>;
+  using H1 = std::integral_constant<int, 1>;
+  const int last = groups - 1;
+  if (groups > 0) {
+    load_group(g_begin, S0{});
+    load_group(g_begin + (groups > 1 ? 1 : 0), S1{});
+    prepare_zeros(S0{});
+    unpack(0, S0{}, H0{});
+  }
+  art_lds_barrier();
+  h8 fa01[2][MT], fb01[2], fa23[2][MT], fb23[2];
+  if (groups > 0) read_frags(fa01, fb01, 0, 0);
+  // Group i (stage S): its first step sits in LDS buffer 0 and the operands of its k-steps 0,1 in registers.
+  // The body has no branches (the scheduling directives work inside one basic block): past the last group it
+  // reloads and unpacks the last group again, which nobody multiplies.
+  auto group_body = [&](int i, auto tag, auto next_tag) {
+    constexpr int S = decltype(tag)::value;
+    const float sc = my_ok ? (float)sc16[S] : 0.f;
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) grp[t][r] = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < GK / 16; ++kk) {
-      const _Float16* p = Ws + (kk * 16 + b_k) * W_LD + b_n;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * W_LD));
-      const h4 l4 = __builtin_bit_cast(h4, lo), h4v = __builtin_bit_cast(h4, hi);
-      const h8 bf = h8{l4[0], l4[1], l4[2], l4[3], h4v[0], h4v[1], h4v[2], h4v[3]};
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        const h8 af = *reinterpret_cast<const h8*>(Xs + (a_row + t * 32) * X_LD + kk * 16 + a_k);
-        grp[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, grp[t], 0, 0, 0);
-      }
-    }
-    const float sc = sc_staged;
+    // step 0 of the group (buffer 0); step 1 is unpacked into buffer 1
+    read_frags(fa23, fb23, 0, 2);
+    unpack(1, tag, H1{});
+    mfma2(fa01, fb01);
+    ART_FIRST_HALF();
+    art_lds_barrier();
+    read_frags(fa01, fb01, 1, 0);
+    load_group(g_begin + (i + 2 < groups ? i + 2 : last), tag);          // stage S is consumed: refill it
+    mfma2(fa23, fb23);
+    ART_SECOND_HALF();
+    // step 1 of the group (buffer 1); step 0 of the next group is unpacked into buffer 0
+    read_frags(fa23, fb23, 1, 2);
+    prepare_zeros(next_tag);
+    unpack(0, next_tag, H0{});
+    mfma2(fa01, fb01);
+    ART_FIRST_HALF();
+    art_lds_barrier();
+    read_frags(fa01, fb01, 0, 0);
+    mfma2(fa23, fb23);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) total[t][r] += grp[t][r] * sc;
   };
-
-  using S0 = std::integral_constant<int, 0>;
-  using S1 = std::integral_constant<int, 1>;
-  if (steps > 0) load_stage(g_begin, S0{});
-  if (steps > 1) load_stage(g_begin + 1, S1{});
-  // Time slots, one barrier after each:   half 0:  D(0) M(0) D(1) M(1) ...
-  //                                        half 1:   -   D(0) M(0) D(1) ...  M(T-1)
-  auto iteration = [&](int i, auto tag) {
-    if (half == 0) unpack(i, tag);
-    else multiply(i - 1);
-    art_lds_barrier();
-    if (half == 0) multiply(i);
-    else unpack(i, tag);
-    art_lds_barrier();
-  };
-  for (int i = 0; i < T; i += 2) {
-    iteration(i, S0{});
-    if (i + 1 < T) iteration(i + 1, S1{});
+  for (int i = 0; i < groups; i += 2) {
+    group_body(i, S0{}, S1{});
+    if (i + 1 < groups) group_body(i + 1, S1{}, S0{});
   }
-  if (half == 1) multiply(T - 1);
+#undef ART_FIRST_HALF
+#undef ART_SECOND_HALF
 
   // ---- epilogue: accumulator element r of tile t is row t*32 + (r/4)*8 + (lane/32)*4 + r%4, column my_col
-  if (!my_ok || steps == 0) return;
+  if (!my_ok || groups == 0) return;
 #pragma unroll
   for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -253,14 +293,17 @@ __global__ __launch_bounds__(256) void gemm_w4a16_combine_kernel(const float* __
   *reinterpret_cast<h4*>(y + i * 4) = out;
 }
 
-// Number of K-splits: as many work items as fit the chip in one round (two per compute unit), but at
-// least four groups per item, and no more than the scratch space for the partial tiles allows.
-// Measured on MI355X at M = 64: N=4096 K=4096 -> 8, N=11008 -> 5, N=4096 K=11008 -> 16, N=32000 -> 2.
-int choose_splits(int rows, int N, int G, size_t scratch_bytes, int compute_units) {
-  const int col_tiles = (N + BN - 1) / BN;
+// Number of K-splits: as many blocks as the chip holds at once (two per compute unit), but at least
+// two groups per block, no more partial-tile bytes than weight bytes (every split adds an fp32 copy of
+// the output to the traffic), and no more than the scratch space allows.  Measured optimum at M = 64 on
+// MI355X: 8 splits for 4096x4096 and 11008x4096, 5 for 4096x11008, 2 for 4096x32000.
+int choose_splits(int rows, int N, int K, size_t scratch_bytes, int compute_units) {
+  const int col_tiles = (N + BN - 1) / BN, G = K / GK;
   int s = 2 * compute_units / col_tiles;
-  if (s > G / 4) s = G / 4;
+  if (s > G / 2) s = G / 2;
   const size_t per_split = (size_t)rows * N * sizeof(float);
+  const size_t weight_bytes = (size_t)K * N / 2;
+  if ((size_t)s * per_split > weight_bytes) s = (int)(weight_bytes / per_split);
   const int cap = (int)(scratch_bytes / per_split);
   if (s > cap) s = cap;
   return s < 1 ? 1 : s;
@@ -295,16 +338,16 @@ extern "C" int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const 
   const int G = K / GK, col_tiles = (N + BN - 1) / BN;
   for (int m0 = 0; m0 < M; m0 += BM) {      // 64 rows of x per pass over the weights
     const int rows = M - m0 < BM ? M - m0 : BM;
-    const int splits = choose_splits(rows, N, G, scratch_bytes, compute_units);
+    const int splits = choose_splits(rows, N, K, scratch_bytes, compute_units);
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m0 * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m0 * N;
-    const dim3 grid((col_tiles * splits + 1) / 2);
+    const dim3 grid(col_tiles * splits);
     if (rows <= 32)
-      gemm_w4a16_kernel<1><<<grid, 512, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
+      gemm_w4a16_kernel<1><<<grid, 256, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
                                                          col_tiles, mg);
     else
-      gemm_w4a16_kernel<2><<<grid, 512, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
+      gemm_w4a16_kernel<2><<<grid, 256, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
                                                          col_tiles, mg);
     ART_LAUNCH_CHECK();
