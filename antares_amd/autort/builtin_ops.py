@@ -266,6 +266,30 @@ class RopeQkvStore:
         return q_out
 
 
+class GreedyNext:
+    """``greedy_next_f16(logits[V], prompt[L] or None, token[1], pos[1], embed[V, D], x[D])``: the bookkeeping
+    between two decode steps in one launch - pos += 1; token = prompt[pos] while the prompt lasts, else
+    argmax(logits); x = embed[token].  token, pos and prompt are int32 GPU tensors."""
+    name = 'greedy_next_f16'
+
+    def __call__(self, logits, prompt, token, pos, embed, x):
+        vocab, dim = embed.shape
+        if logits.numel() != vocab or x.numel() != dim or token.numel() != 1 or pos.numel() != 1:
+            raise ValueError('greedy_next_f16: shapes do not fit together')
+        if not (logits.dtype == embed.dtype == x.dtype == torch.float16):
+            raise TypeError('greedy_next_f16: logits, embed and x must be float16')
+        ints = [token, pos] + ([prompt] if prompt is not None and prompt.numel() else [])
+        if any(t.dtype != torch.int32 for t in ints):
+            raise TypeError('greedy_next_f16: token, pos and prompt must be int32')
+        _require_cuda(logits, embed, x, *ints)
+        has_prompt = len(ints) == 3
+        capi.check(capi.lib().art_greedy_next(c_void_p(logits.data_ptr()), vocab, c_void_p(prompt.data_ptr() if has_prompt else 0),
+                                             prompt.numel() if has_prompt else 0, c_void_p(token.data_ptr()), c_void_p(pos.data_ptr()),
+                                             c_void_p(embed.data_ptr()), dim, c_void_p(x.data_ptr()), c_void_p(current_stream_handle())))
+        return token
+
+
+builtin('greedy_next_f16')(lambda: GreedyNext())
 builtin('gemv_w4a16_fused')(lambda: GemvW4Fused())
 builtin('attention_rope_f16')(lambda: AttentionRope())
 builtin('rope_qkv_store_f16')(lambda: RopeQkvStore('rope_qkv_store_f16'))

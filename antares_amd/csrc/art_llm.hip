@@ -426,3 +426,92 @@ extern "C" int art_decode_attention_rope(const void* qkv_dev, const void* inv_fr
   ART_LAUNCH_CHECK();
   return 0;
 }
+
+// ------------------------------------------------------------------ greedy step bookkeeping
+// The tail of one decode step of samples/05_llama2_7b_int4.py:196-201 in a single block:
+//   pos <- pos + 1;  token <- prompt[pos] while the prompt lasts, else argmax(logits);  x <- embedding[token].
+// Replaces an argmax, five elementwise launches and the embedding gather of the next step.
+namespace {
+
+constexpr int kGreedyThreads = 1024;
+
+__global__ __launch_bounds__(kGreedyThreads) void greedy_next_kernel(const _Float16* __restrict__ logits, int vocab,
+                                                                      const int* __restrict__ prompt, int prompt_len,
+                                                                      int* __restrict__ token, int* __restrict__ pos,
+                                                                      const _Float16* __restrict__ embed, int dim,
+                                                                      _Float16* __restrict__ x_out) {
+  __shared__ float s_val[kGreedyThreads / 64];
+  __shared__ int s_idx[kGreedyThreads / 64];
+  __shared__ int s_token;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int next_pos = *pos + 1;
+  // largest logit, smallest index among equals (what torch.argmax returns)
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  // 16-byte chunks, four of them requested before the first is looked at (one round trip for 32768 logits)
+  const int chunks = vocab >> 3;
+  for (int c0 = tid; c0 < chunks; c0 += 4 * kGreedyThreads) {
+    u32x4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = c0 + j * kGreedyThreads;
+      v[j] = *reinterpret_cast<const u32x4*>(logits + 8 * (size_t)(c < chunks ? c : c0));
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = c0 + j * kGreedyThreads;
+      if (c >= chunks) break;
+      const unsigned int wds[4] = {v[j][0], v[j][1], v[j][2], v[j][3]};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 pair = __builtin_bit_cast(h2, wds[e >> 1]);
+        const float f = (float)((e & 1) ? pair.y : pair.x);
+        if (f > best) { best = f; best_i = 8 * c + e; }      // indices grow: the first maximum of this thread stays
+      }
+    }
+  }
+  for (int i = (chunks << 3) + tid; i < vocab; i += kGreedyThreads) {      // vocab % 8 leftovers
+    const float f = (float)logits[i];
+    if (f > best || (f == best && i < best_i)) { best = f; best_i = i; }
+  }
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+    const float ov = __shfl_xor(best, m, 64);
+    const int oi = __shfl_xor(best_i, m, 64);
+    if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+  }
+  if (lane == 0) { s_val[wave] = best; s_idx[wave] = best_i; }
+  __syncthreads();
+  if (tid == 0) {
+    float b = s_val[0];
+    int bi = s_idx[0];
+    for (int w = 1; w < kGreedyThreads / 64; ++w)
+      if (s_val[w] > b || (s_val[w] == b && s_idx[w] < bi)) { b = s_val[w]; bi = s_idx[w]; }
+    if (bi == 0x7fffffff) bi = 0;                 // every logit was NaN or -inf
+    const int t = (next_pos < prompt_len) ? prompt[next_pos] : bi;
+    s_token = t;
+    *token = t;
+    *pos = next_pos;
+  }
+  __syncthreads();
+  const _Float16* row = embed + (size_t)s_token * dim;
+  for (int i = tid * 8; i < dim; i += kGreedyThreads * 8)
+    *reinterpret_cast<u32x4*>(x_out + i) = *reinterpret_cast<const u32x4*>(row + i);
+}
+
+}  // namespace
+
+extern "C" int art_greedy_next(const void* logits_dev, int vocab, const void* prompt_dev, int prompt_len, void* token_dev,
+                               void* pos_dev, const void* embed_dev, int dim, void* x_out_dev, void* stream) {
+  ART_REQUIRE(logits_dev && token_dev && pos_dev && embed_dev && x_out_dev, "art_greedy_next: null pointer");
+  ART_REQUIRE(vocab >= 1 && dim >= 8 && dim % 8 == 0, "art_greedy_next: need vocab >= 1 and dim %% 8 == 0 (vocab=%d dim=%d)", vocab, dim);
+  ART_REQUIRE(prompt_len == 0 || prompt_dev != nullptr, "art_greedy_next: prompt_len > 0 needs a prompt");
+  ART_REQUIRE(((uintptr_t)embed_dev % 16) == 0 && ((uintptr_t)x_out_dev % 16) == 0 && ((uintptr_t)logits_dev % 16) == 0,
+              "art_greedy_next: logits, embedding and x must be 16-byte aligned");
+  greedy_next_kernel<<<dim3(1), dim3(kGreedyThreads), 0, (hipStream_t)stream>>>((const _Float16*)logits_dev, vocab, (const int*)prompt_dev,
+                                                                                prompt_len, (int*)token_dev, (int*)pos_dev,
+                                                                                (const _Float16*)embed_dev, dim, (_Float16*)x_out_dev);
+  ART_LAUNCH_CHECK();
+  return 0;
+}

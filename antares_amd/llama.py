@@ -138,17 +138,19 @@ class LlamaInt4Decoder:
     def _linear(self, x: torch.Tensor, lin: Dict[str, torch.Tensor], out: torch.Tensor):
         self.gemv(x.view(1, -1), lin['qweight'], lin['scales'], lin['qzeros'], out=out.view(1, -1))
 
-    def step(self) -> torch.Tensor:
-        """Forward pass for (self.token, self.pos); leaves fp16 logits in self.logits."""
-        return self.step_fused() if self.fused else self.step_plain()
+    def step(self, embed: bool = True) -> torch.Tensor:
+        """Forward pass for (self.token, self.pos); leaves fp16 logits in self.logits.  ``embed=False`` skips the
+        embedding lookup: self.x already holds the row (the fused ``advance`` leaves it there)."""
+        return self.step_fused(embed) if self.fused else self.step_plain()
 
-    def step_fused(self) -> torch.Tensor:
+    def step_fused(self, embed: bool = True) -> torch.Tensor:
         """Five launches per layer: RMSNorm, SwiGLU and the residual adds ride inside the projections; rotary of
         q and k and both cache writes ride inside the attention.  Same roundings as ``step_plain``."""
         cfg, ops = self.cfg, self.autort.ops
         H, D = cfg.n_heads, cfg.head_dim
         gemv = ops.gemv_w4a16_fused
-        self.embed(self.w['embed'], self.token, out=self.x)
+        if embed:
+            self.embed(self.w['embed'], self.token, out=self.x)
         for l, lw in enumerate(self.w['layers']):
             a, o, gu, dn = lw['qkv'], lw['o'], lw['gate_up'], lw['down']
             gemv(self.x, a['qweight'], a['scales'], a['qzeros'], self.qkv, norm_weight=lw['att_norm'], eps=cfg.rms_eps)
@@ -188,7 +190,11 @@ class LlamaInt4Decoder:
 
     def advance(self, prompt: Optional[torch.Tensor] = None):
         """pos <- pos + 1; token <- prompt[pos] while the prompt lasts, else argmax(logits).
-        All on the device, so it can be part of the recorded graph."""
+        All on the device, so it can be part of the recorded graph.  The fused decoder does it in one launch,
+        which also leaves the embedding row of the new token in self.x."""
+        if self.fused:
+            self.autort.ops.greedy_next_f16(self.logits, prompt, self.token, self.pos, self.w['embed'], self.x)
+            return
         nxt = torch.argmax(self.logits).to(torch.int32).view(1)
         self.pos.add_(1)
         if prompt is not None and prompt.numel() > 0:
@@ -206,7 +212,7 @@ class LlamaInt4Decoder:
             stream.synchronize()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=stream):
-                self.step()
+                self.step(embed=not (greedy and self.fused))     # the fused advance has already fetched the row
                 if greedy:
                     self.advance(prompt)
         torch.cuda.synchronize()
@@ -216,3 +222,4 @@ class LlamaInt4Decoder:
     def reset(self, token: int = 0, pos: int = 0):
         self.token.fill_(token)
         self.pos.fill_(pos)
+        self.embed(self.w['embed'], self.token, out=self.x)      # a recorded greedy graph starts from self.x

@@ -187,6 +187,13 @@ int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev
                          int seq_len, int heads, int head_dim, const void* pos_dev, int q_dtype, int kv_dtype, int out_dtype,
                          void* stream);
 
+/* The bookkeeping between two decode steps of samples/05_llama2_7b_int4.py:196-201, one launch, all on the
+ * device:  *pos += 1;  *token = (*pos < prompt_len) ? prompt[*pos] : argmax(logits[0..vocab));
+ * x_out[0..dim) = embed[*token][0..dim).  logits, embed, x_out fp16; prompt, token, pos int32.  Ties of the
+ * argmax go to the smallest index.  prompt_dev may be NULL when prompt_len == 0. */
+int art_greedy_next(const void* logits_dev, int vocab, const void* prompt_dev, int prompt_len, void* token_dev,
+                    void* pos_dev, const void* embed_dev, int dim, void* x_out_dev, void* stream);
+
 /* Bytes of library workspace art_partition_even_first_i32 / split-K kernels may use. */
 size_t art_workspace_bytes(void);
 

@@ -124,3 +124,35 @@ def test_attention_on_cache_views(autort, dtype, S):
     pos_t = torch.tensor([S - 1], dtype=torch.int32, device=dev)
     out2 = op(q, key_cache.view(seq_len, H, D), val_cache.view(seq_len, H, D), att_f, extra=[pos_t])
     assert torch.equal(out, out2)
+
+
+def test_greedy_next_matches_torch():
+    """pos += 1; token = prompt[pos] while the prompt lasts, else argmax(logits) (first maximum); x = embed[token]."""
+    import autort
+    dev = autort.device()
+    g = torch.Generator().manual_seed(4)
+    V, D = 32000, 4096
+    embed = (torch.randn(V, D, generator=g) * 0.02).half().to(dev)
+    prompt = torch.randint(0, V, (5,), generator=g, dtype=torch.int32).to(dev)
+    x = torch.zeros(D, dtype=torch.float16, device=dev)
+    for case in range(6):
+        note(f'greedy_next case {case}')
+        logits = torch.randn(V, generator=g).half()
+        if case == 1:                      # ties: the first maximum wins
+            logits[[777, 20000, 31999]] = logits.max() + 1
+        if case == 2:
+            logits[V - 1] = 100.0          # last element
+        if case == 3:
+            logits[0] = 100.0              # first element
+        logits = logits.to(dev)
+        for start_pos, use_prompt in ((0, True), (3, True), (4, True), (9, True), (7, False)):
+            token = torch.full((1,), -1, dtype=torch.int32, device=dev)
+            pos = torch.full((1,), start_pos, dtype=torch.int32, device=dev)
+            autort.ops.greedy_next_f16(logits, prompt if use_prompt else None, token, pos, embed, x)
+            torch.cuda.synchronize()
+            new_pos = start_pos + 1
+            want = int(prompt[new_pos]) if (use_prompt and new_pos < prompt.numel()) else int(torch.argmax(logits.float().cpu()))
+            if case == 1 and not (use_prompt and new_pos < prompt.numel()):
+                want = 777
+            assert int(pos) == new_pos and int(token) == want, (case, start_pos, use_prompt, int(token), want)
+            assert torch.equal(x, embed[want])
