@@ -243,6 +243,56 @@ class AttentionRope:
         return out
 
 
+class AttentionRopeSplit:
+    """``attention_rope_split_f16(qkv[3*H*D], inv_freq[D], key_cache, val_cache, att_f[1], partial[H, P, 132], extra=[pos_tensor])``:
+    ``attention_rope_f16`` spread over P blocks per head.  ``partial`` (float32) receives, per head and part, 128
+    unnormalised sums, the running maximum and the running sum; ``gemv_w4a16_attn`` merges them while it loads x."""
+    name = 'attention_rope_split_f16'
+
+    def __call__(self, qkv, inv_freq, key_cache, val_cache, att_f, partial, extra=None):
+        if partial.dim() != 3 or partial.shape[2] != 132 or partial.dtype != torch.float32:
+            raise TypeError('attention_rope_split_f16: partial must be float32 [heads, parts, 132]')
+        heads, parts = partial.shape[0], partial.shape[1]
+        head_dim = key_cache.shape[-1] // heads
+        if qkv.numel() != 3 * heads * head_dim or val_cache.shape != key_cache.shape or not 2 <= parts <= 8:
+            raise ValueError('attention_rope_split_f16: shapes do not fit together (2..8 parts)')
+        for t in (qkv, inv_freq, key_cache, val_cache):
+            if t.dtype != torch.float16:
+                raise TypeError('attention_rope_split_f16: qkv, inv_freq and the caches must be float16')
+        if att_f.dtype != torch.float32 or att_f.numel() != 1:
+            raise TypeError('attention_rope_split_f16: att_f must be a 1-element float32 tensor')
+        _require_cuda(qkv, inv_freq, key_cache, val_cache, att_f, partial)
+        pos_dev, _ = _pos_args(extra, self.name)
+        if not pos_dev.value:
+            raise TypeError('attention_rope_split_f16: extra=[pos] must be a 1-element int32 GPU tensor')
+        capi.check(capi.lib().art_decode_attention_rope_split(
+            c_void_p(qkv.data_ptr()), c_void_p(inv_freq.data_ptr()), c_void_p(key_cache.data_ptr()), c_void_p(val_cache.data_ptr()),
+            c_void_p(att_f.data_ptr()), c_void_p(partial.data_ptr()), heads, head_dim, pos_dev, parts,
+            c_void_p(current_stream_handle())))
+        return partial
+
+
+class GemvW4Attn:
+    """``gemv_w4a16_attn(partial[H, P, 132], qweight, scales, qzeros, out[N], residual=None)``: the int4 projection of a
+    split attention's output (merged on the fly) with the residual add folded in."""
+    name = 'gemv_w4a16_attn'
+
+    def __call__(self, partial, qweight, scales, qzeros, out, residual=None):
+        K, N = qweight.shape[0] * 2, qweight.shape[1]
+        if partial.dim() != 3 or partial.shape[2] != 132 or partial.dtype != torch.float32 or partial.shape[0] * 128 != K:
+            raise TypeError('gemv_w4a16_attn: partial must be float32 [K/128, parts, 132]')
+        if scales.shape != (K // 128, N) or qzeros.shape != (K // 128, N // 2) or out.numel() != N:
+            raise ValueError('gemv_w4a16_attn: operand shapes do not match K, N')
+        if scales.dtype != torch.float16 or out.dtype != torch.float16 or (residual is not None and residual.dtype != torch.float16):
+            raise TypeError('gemv_w4a16_attn: scales, out and residual must be float16')
+        _require_cuda(*([partial, qweight, scales, qzeros, out] + ([residual] if residual is not None else [])))
+        capi.check(capi.lib().art_gemv_w4a16_attn(
+            c_void_p(partial.data_ptr()), partial.shape[1], c_void_p(qweight.data_ptr()), c_void_p(scales.data_ptr()),
+            c_void_p(qzeros.data_ptr()), c_void_p(out.data_ptr()), K, N,
+            c_void_p(residual.data_ptr() if residual is not None else 0), c_void_p(current_stream_handle())))
+        return out
+
+
 class RopeQkvStore:
     """``rope_qkv_store_f16(qkv[3*H*D], inv_freq[D], q_out[H,D], key_cache[S,H*D], val_cache[S,H*D], extra=[pos_tensor])``:
     rotary embedding of q and k (k straight into its cache row) and the copy of v into its cache row, one launch."""
@@ -292,5 +342,7 @@ class GreedyNext:
 builtin('greedy_next_f16')(lambda: GreedyNext())
 builtin('gemv_w4a16_fused')(lambda: GemvW4Fused())
 builtin('attention_rope_f16')(lambda: AttentionRope())
+builtin('attention_rope_split_f16')(lambda: AttentionRopeSplit())
+builtin('gemv_w4a16_attn')(lambda: GemvW4Attn())
 builtin('rope_qkv_store_f16')(lambda: RopeQkvStore('rope_qkv_store_f16'))
 builtin('rope_qkv_store_f32')(lambda: RopeQkvStore('rope_qkv_store_f32'))

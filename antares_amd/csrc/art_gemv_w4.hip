@@ -40,6 +40,7 @@ namespace {
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ half2_t as_h2(unsigned int v) { return __builtin_bit_cast(half2_t, v); }
 
@@ -117,9 +118,11 @@ struct Fused {
   const _Float16* residual;
   const _Float16* gate_up;
   float inv_n, eps;
+  const float* att_partial;   // != NULL: x is merged from the per-part records of a split decode attention (see MODE 3)
+  int att_parts;
 };
 
-template <int M, int MODE>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused
+template <int M, int MODE>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused, 3: x = merged split attention
 __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight, const _Float16* __restrict__ scales,
     const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y, int K, int N, int splits,
@@ -164,6 +167,23 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     upair = *reinterpret_cast<const unsigned int*>(fused.gate_up + K + k);
   }
 
+  // ---- fused attention merge, part 1: x is the output of a decode attention that ran as `att_parts` blocks per
+  // head and left, per (head, part), 128 unnormalised sums, the running maximum and the running sum of
+  // exp.  As with SwiGLU each column lane produces one pair of the k lane's 16 values.
+  constexpr bool attn = (M == 1) && (MODE == 3);
+  constexpr int kMaxParts = 8, kPartStride = 132;         // record layout of the attention kernel
+  f32x2 pacc[kMaxParts], pml[kMaxParts];
+  if (attn) {
+    const int k = 2 * r0c + 2 * cl, head = k >> 7, d = k & 127;
+    const float* rec = fused.att_partial + (size_t)head * fused.att_parts * kPartStride;
+#pragma unroll
+    for (int p = 0; p < kMaxParts; ++p) {
+      const int pc = p < fused.att_parts ? p : 0;         // unused parts re-read part 0 and get weight 0 below
+      pacc[p] = *reinterpret_cast<const f32x2*>(rec + pc * kPartStride + d);
+      pml[p] = *reinterpret_cast<const f32x2*>(rec + pc * kPartStride + 128);
+    }
+  }
+
   // ---- every other global load of this lane
   u32x4 w[R];
   {
@@ -174,15 +194,32 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
   u32x4 xv[M][2];                                         // 16 halves of x per row of x
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    if (swiglu) continue;
+    if (swiglu || attn) continue;
     const u32x4* xp = reinterpret_cast<const u32x4*>(x + (size_t)m * K + 2 * r0c);
     xv[m][0] = xp[0];
     xv[m][1] = xp[1];
   }
-  if (swiglu) {       // part 2: pair -> LDS -> all 16 values of the k lane (same wavefront: no block barrier needed)
-    const half2_t g = as_h2(gpair), u = as_h2(upair);
-    const float g0f = (float)g.x, g1f = (float)g.y;
-    const half2_t o = {(_Float16)(g0f / (1.0f + expf(0.0f - g0f)) * (float)u.x), (_Float16)(g1f / (1.0f + expf(0.0f - g1f)) * (float)u.y)};
+  if (swiglu || attn) {       // part 2: pair -> LDS -> all 16 values of the k lane (same wavefront: no block barrier needed)
+    half2_t o;
+    if (swiglu) {
+      const half2_t g = as_h2(gpair), u = as_h2(upair);
+      const float g0f = (float)g.x, g1f = (float)g.y;
+      o = half2_t{(_Float16)(g0f / (1.0f + expf(0.0f - g0f)) * (float)u.x), (_Float16)(g1f / (1.0f + expf(0.0f - g1f)) * (float)u.y)};
+    } else {                  // softmax merge: out = sum_p e^(m_p - M) acc_p / sum_p e^(m_p - M) l_p, rounded once to fp16
+      float mm = -INFINITY;
+#pragma unroll
+      for (int p = 0; p < kMaxParts; ++p)
+        if (p < fused.att_parts) mm = fmaxf(mm, pml[p][0]);
+      float n0f = 0.f, n1f = 0.f, den = 0.f;
+#pragma unroll
+      for (int p = 0; p < kMaxParts; ++p) {
+        const float wgt = (p < fused.att_parts && pml[p][0] != -INFINITY) ? __expf(pml[p][0] - mm) : 0.f;
+        n0f = fmaf(pacc[p][0], wgt, n0f);
+        n1f = fmaf(pacc[p][1], wgt, n1f);
+        den = fmaf(pml[p][1], wgt, den);
+      }
+      o = half2_t{(_Float16)(n0f / den), (_Float16)(n1f / den)};
+    }
     s_x[kl][cl] = __builtin_bit_cast(unsigned int, o);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -328,7 +365,7 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
 
 template <int M>
 int launch(const void* x, const void* qw, const void* sc, const void* qz, void* y, int K, int N, hipStream_t stream,
-           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f}) {
+           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0}) {
   const int rows = K / 2;
   const int tiles = (N + CT - 1) / CT;
   const int splits = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
@@ -345,6 +382,7 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
   // the plain product is its own instantiation: it carries none of the fused prologues
   if (M == 1 && fused.norm_w != nullptr) ART_GEMV_LAUNCH(1);
   else if (M == 1 && fused.gate_up != nullptr) ART_GEMV_LAUNCH(2);
+  else if (M == 1 && fused.att_partial != nullptr) ART_GEMV_LAUNCH(3);
   else ART_GEMV_LAUNCH(0);
 #undef ART_GEMV_LAUNCH
   ART_LAUNCH_CHECK();
@@ -384,6 +422,17 @@ extern "C" int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, 
               "art_gemv_w4a16_fused: x, qweight and the norm weight must be 16-byte aligned");
   ART_REQUIRE(x_dev != y_dev || norm_weight_dev == nullptr, "art_gemv_w4a16_fused: y may alias the residual, not a normalised x");
   Fused f{(const _Float16*)norm_weight_dev, (const _Float16*)residual_dev, swiglu_input ? (const _Float16*)x_dev : nullptr,
-          1.0f / (float)K, eps};
+          1.0f / (float)K, eps, nullptr, 0};
   return launch<1>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, (hipStream_t)stream, f);
+}
+
+extern "C" int art_gemv_w4a16_attn(const void* partial_dev, int parts, const void* qweight_dev, const void* scales_dev,
+                                   const void* qzeros_dev, void* y_dev, int K, int N, const void* residual_dev, void* stream) {
+  ART_REQUIRE(partial_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16_attn: null pointer");
+  ART_REQUIRE(parts >= 2 && parts <= 8, "art_gemv_w4a16_attn: parts must be in 2..8 (got %d)", parts);
+  ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_attn: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
+  ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)partial_dev % 16) == 0,
+              "art_gemv_w4a16_attn: partial records and qweight must be 16-byte aligned");
+  Fused f{nullptr, (const _Float16*)residual_dev, nullptr, 0.f, 0.f, (const float*)partial_dev, parts};
+  return launch<1>(partial_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, (hipStream_t)stream, f);
 }

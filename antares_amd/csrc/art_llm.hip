@@ -135,6 +135,7 @@ template <> struct Row16<float> {
 constexpr int kAttThreads = 512;
 constexpr int kAttGroups = kAttThreads / 8;   // 64 position groups per block
 constexpr int kAttWaves = kAttThreads / 64;
+constexpr int kAttPartialStride = 132;        // floats per (head, part) record: acc[128], max, sum, 2 of padding (16-byte rows)
 
 // Merge the online-softmax state of the lane `mask` away (same dims, other positions) into this lane's.
 __device__ __forceinline__ void att_merge_lane(float& m, float& l, float (&acc)[16], int mask) {
@@ -153,19 +154,27 @@ template <class QT, class KT, class OT, bool ROPE>
 __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __restrict__ q_or_qkv, KT* __restrict__ k, KT* __restrict__ v,
                                                                  const float* __restrict__ att_f, OT* __restrict__ out, int heads,
                                                                  const int* __restrict__ len_dev, int len_host,
-                                                                 const _Float16* __restrict__ inv_freq) {
+                                                                 const _Float16* __restrict__ inv_freq,
+                                                                 float* __restrict__ partial, int parts) {
+  // parts > 1: `parts` blocks share a head, each attends over a contiguous range of the cached positions and
+  // leaves its unnormalised state in partial[head][part][kAttPartialStride] = { acc[128], max, sum, -, - };
+  // whoever consumes the result merges them (the o-projection does it while it loads x).
   constexpr int D = 128, U = 4;
   __shared__ float s_m[kAttWaves], s_l[kAttWaves];
   __shared__ float s_acc[kAttWaves][D];
   __shared__ float s_q[D];
   __shared__ float s_k[D], s_v[D];
   const int S = len_dev ? (*len_dev + 1) : len_host;     // device form carries the position, length = pos + 1
-  const int h = blockIdx.x, tid = threadIdx.x;
+  const int h = blockIdx.x / parts, part = blockIdx.x % parts, tid = threadIdx.x;
   const int sub = tid & 7, group = tid >> 3;
   const float scale = att_f[0];
   const size_t row = (size_t)heads * D;
   // With ROPE the newest position is served from LDS: the block does not wait for its own cache write.
-  const int Sc = ROPE ? S - 1 : S;                        // positions read from the cache
+  const int cached = ROPE ? S - 1 : S;                    // positions read from the cache
+  const int span = (cached + parts - 1) / parts;          // ... of which this block takes [s_first, Sc)
+  const int s_first = part * span < cached ? part * span : cached;
+  const int Sc = s_first + span < cached ? s_first + span : cached;
+  const bool newest_here = ROPE && part == 0;             // one block of the head writes the cache row and attends to it
 
   // this thread's share of the token's q|k|v, requested before anything else
   float xa = 0.f, xb = 0.f, xv = 0.f;
@@ -191,7 +200,8 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
       Row16<KT>::load(v + (size_t)sc * row + (size_t)h * D + sub * 16, vf[u]);
     }
   };
-  if (group < Sc) request(group);
+  const int s_start = s_first + group;
+  if (s_start < Sc) request(s_start);
 
   float qf[16];
   if (ROPE) {
@@ -203,16 +213,18 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
       sincosf((float)pos * (float)inv_freq[j], &sn, &cs);
       const float ra = xa * cs - xb * sn, rb = xb * cs + xa * sn;
       if (is_k) {                                         // the cache gets the rounded value, and so does this step
-        KT* dst = k + (size_t)pos * row + (size_t)h * D;
-        st(dst, j, ra);
-        st(dst, j + 64, rb);
-        s_k[j] = (float)(KT)ra;
-        s_k[j + 64] = (float)(KT)rb;
+        if (newest_here) {
+          KT* dst = k + (size_t)pos * row + (size_t)h * D;
+          st(dst, j, ra);
+          st(dst, j + 64, rb);
+          s_k[j] = (float)(KT)ra;
+          s_k[j + 64] = (float)(KT)rb;
+        }
       } else {                                            // q goes through the output dtype like the separate operator
         s_q[j] = (float)(QT)ra;
         s_q[j + 64] = (float)(QT)rb;
       }
-    } else if (tid < 256) {
+    } else if (tid < 256 && newest_here) {
       const int e = tid - 128;
       v[(size_t)pos * row + (size_t)h * D + e] = (KT)xv;
       s_v[e] = (float)(KT)xv;
@@ -242,8 +254,8 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
     for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * vrow[i]);
     m = mn;
   };
-  for (int s0 = group; s0 < Sc; s0 += kAttGroups * U) {
-    if (s0 != group) request(s0);
+  for (int s0 = s_start; s0 < Sc; s0 += kAttGroups * U) {
+    if (s0 != s_start) request(s0);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       float d = 0.f;
@@ -253,7 +265,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
       if (s0 + u * kAttGroups < Sc) absorb(d, vf[u]);
     }
   }
-  if (ROPE) {                                             // the newest position, from LDS, joins group 0
+  if (newest_here) {                                      // the newest position, from LDS, joins group 0
     float kn[16], vn[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -287,7 +299,13 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
       ll = fmaf(s_l[g], wgt, ll);
       o = fmaf(s_acc[g][tid], wgt, o);
     }
-    st(out, (size_t)h * D + tid, o / ll);
+    if (parts == 1) {
+      st(out, (size_t)h * D + tid, o / ll);
+    } else {                                  // an empty range leaves max = -inf, sum = 0: weight 0 in the merge
+      float* dst = partial + ((size_t)h * parts + part) * kAttPartialStride;
+      dst[tid] = o;
+      if (tid == 0) { dst[D] = mm; dst[D + 1] = ll; }
+    }
   }
 }
 
@@ -387,7 +405,7 @@ extern "C" int art_decode_attention(const void* q_dev, const void* k_dev, const 
   hipStream_t st = (hipStream_t)stream;
   const int* pd = (const int*)pos_dev;
   const float* af = (const float*)att_f_dev;
-#define ART_ATT(QT, KT) attention_kernel<QT, KT, QT, false><<<dim3(heads), dim3(kAttThreads), 0, st>>>((const QT*)q_dev, (KT*)k_dev, (KT*)v_dev, af, (QT*)out_dev, heads, pd, seq_len, nullptr)
+#define ART_ATT(QT, KT) attention_kernel<QT, KT, QT, false><<<dim3(heads), dim3(kAttThreads), 0, st>>>((const QT*)q_dev, (KT*)k_dev, (KT*)v_dev, af, (QT*)out_dev, heads, pd, seq_len, nullptr, nullptr, 1)
   if (q_dtype == 0) { if (kv_dtype == 0) ART_ATT(float, float); else ART_ATT(float, _Float16); }
   else { if (kv_dtype == 0) ART_ATT(_Float16, float); else ART_ATT(_Float16, _Float16); }
 #undef ART_ATT
@@ -415,14 +433,23 @@ extern "C" int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, voi
 extern "C" int art_decode_attention_rope(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev, void* val_cache_dev,
                                          const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev,
                                          void* stream) {
+  return art_decode_attention_rope_split(qkv_dev, inv_freq_dev, key_cache_dev, val_cache_dev, att_f_dev, out_dev, heads, head_dim,
+                                         pos_dev, 1, stream);
+}
+
+extern "C" int art_decode_attention_rope_split(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev,
+                                               void* val_cache_dev, const void* att_f_dev, void* out_dev, int heads, int head_dim,
+                                               const void* pos_dev, int parts, void* stream) {
   ART_REQUIRE(qkv_dev && inv_freq_dev && key_cache_dev && val_cache_dev && att_f_dev && out_dev && pos_dev,
               "art_decode_attention_rope: null pointer");
   ART_REQUIRE(head_dim == 128 && heads >= 1, "art_decode_attention_rope: head_dim must be 128 (got %d)", head_dim);
-  ART_REQUIRE(((uintptr_t)key_cache_dev % 16) == 0 && ((uintptr_t)val_cache_dev % 16) == 0,
-              "art_decode_attention_rope: caches must be 16-byte aligned");
-  attention_kernel<_Float16, _Float16, _Float16, true><<<dim3(heads), dim3(kAttThreads), 0, (hipStream_t)stream>>>(
-      (const _Float16*)qkv_dev, (_Float16*)key_cache_dev, (_Float16*)val_cache_dev, (const float*)att_f_dev, (_Float16*)out_dev,
-      heads, (const int*)pos_dev, 0, (const _Float16*)inv_freq_dev);
+  ART_REQUIRE(parts >= 1 && parts <= 16, "art_decode_attention_rope: parts must be in 1..16 (got %d)", parts);
+  ART_REQUIRE(((uintptr_t)key_cache_dev % 16) == 0 && ((uintptr_t)val_cache_dev % 16) == 0 && ((uintptr_t)out_dev % 16) == 0,
+              "art_decode_attention_rope: caches and output must be 16-byte aligned");
+  attention_kernel<_Float16, _Float16, _Float16, true><<<dim3(heads * parts), dim3(kAttThreads), 0, (hipStream_t)stream>>>(
+      (const _Float16*)qkv_dev, (_Float16*)key_cache_dev, (_Float16*)val_cache_dev, (const float*)att_f_dev,
+      parts == 1 ? (_Float16*)out_dev : nullptr, heads, (const int*)pos_dev, 0, (const _Float16*)inv_freq_dev,
+      parts == 1 ? nullptr : (float*)out_dev, parts);
   ART_LAUNCH_CHECK();
   return 0;
 }

@@ -94,9 +94,10 @@ class LlamaInt4Decoder:
     """One-token-per-step decoder.  ``step()`` enqueues a whole forward pass on the
     current stream; ``capture()`` records it once in a HIP graph."""
 
-    def __init__(self, cfg: LlamaConfig, weights: Dict[str, object], device=None, fused: bool = True):
+    def __init__(self, cfg: LlamaConfig, weights: Dict[str, object], device=None, fused: bool = True, att_parts: int = 8):
         import autort
         self.fused = fused
+        self.att_parts = att_parts if fused else 1     # blocks per head in the decode attention (1 = unsplit)
         self.autort = autort
         self.cfg = cfg
         self.dev = device or autort.device()
@@ -116,6 +117,7 @@ class LlamaInt4Decoder:
         self.xb = torch.empty(d, **f16)
         self.qkv = torch.empty(3 * d, **f16)
         self.q_rot = torch.empty(H, D, **f16)
+        self.att_partial = torch.zeros(H, max(self.att_parts, 2), 132, dtype=torch.float32, device=self.dev)
         self.att = torch.empty(H, D, **f16)
         self.proj = torch.empty(d, **f16)
         self.gu = torch.empty(2 * cfg.ffn, **f16)
@@ -154,9 +156,14 @@ class LlamaInt4Decoder:
         for l, lw in enumerate(self.w['layers']):
             a, o, gu, dn = lw['qkv'], lw['o'], lw['gate_up'], lw['down']
             gemv(self.x, a['qweight'], a['scales'], a['qzeros'], self.qkv, norm_weight=lw['att_norm'], eps=cfg.rms_eps)
-            ops.attention_rope_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f, self.att,
-                                   extra=[self.pos])
-            gemv(self.att.view(-1), o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
+            if self.att_parts > 1:      # attention over several blocks per head, merged by the o-projection as it loads x
+                ops.attention_rope_split_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f,
+                                             self.att_partial, extra=[self.pos])
+                ops.gemv_w4a16_attn(self.att_partial, o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
+            else:
+                ops.attention_rope_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f, self.att,
+                                       extra=[self.pos])
+                gemv(self.att.view(-1), o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
             gemv(self.x, gu['qweight'], gu['scales'], gu['qzeros'], self.gu, norm_weight=lw['ffn_norm'], eps=cfg.rms_eps)
             gemv(self.gu, dn['qweight'], dn['scales'], dn['qzeros'], self.x, residual=self.x, swiglu=True)
         h = self.w['lm_head']

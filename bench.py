@@ -46,6 +46,7 @@ def parse_args():
     ap.add_argument('--no-extra', action='store_true', help='headline workload only')
     ap.add_argument('--no-decode', action='store_true', help='skip the 32-layer decode leg')
     ap.add_argument('--decode-cpu-steps', type=int, default=2, help='decode steps timed on the CPU oracle (0 = skip)')
+    ap.add_argument('--att-parts', type=int, default=8, help='blocks per head of the decode attention (1 = unsplit)')
     ap.add_argument('--seed', type=int, default=0)
     return ap.parse_args()
 
@@ -138,7 +139,7 @@ def bench_partition(torch, autort, capi, workloads, steps, warmup, seed, n=16_77
             'gbps': 8 * n / sec / 1e9, 'roofline_frac': 8 * n / sec / 1e9 / HBM_PEAK_GBPS, 'melem_per_s': n / sec / 1e6}
 
 
-def bench_decode(torch, autort, capi, seed, prompt_len=128, decode_steps=256, cpu_steps=0):
+def bench_decode(torch, autort, capi, seed, prompt_len=128, decode_steps=256, cpu_steps=0, att_parts=8):
     """BASELINE configuration 5: 32-layer Llama-2-7B-shaped int4 decode through autort.ops,
     batch 1, random-init weights, a 128-token random prompt fed token by token, then
     256 greedy steps; every step is one replay of the same recorded HIP graph.  The
@@ -148,7 +149,7 @@ def bench_decode(torch, autort, capi, seed, prompt_len=128, decode_steps=256, cp
     t0 = time.time()
     weights = random_weights(cfg, seed)
     gen_s = time.time() - t0
-    dec = LlamaInt4Decoder(cfg, weights)
+    dec = LlamaInt4Decoder(cfg, weights, att_parts=att_parts)
     g = torch.Generator().manual_seed(seed + 7)
     prompt = torch.randint(0, cfg.vocab, (prompt_len,), generator=g, dtype=torch.int64).to(torch.int32)
     prompt_dev = prompt.to(dec.dev)
@@ -269,7 +270,8 @@ def main():
             extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
         result['extra'] = extra
     if not args.no_decode:
-        result['decode'] = bench_decode(torch, autort, capi, args.seed, cpu_steps=0 if args.no_cpu else args.decode_cpu_steps)
+        result['decode'] = bench_decode(torch, autort, capi, args.seed, cpu_steps=0 if args.no_cpu else args.decode_cpu_steps,
+                                        att_parts=args.att_parts)
     if not args.no_cpu:
         result['cpu_baseline'] = cpu_baseline_gemv(workloads, K, N, M, args.seed)
         result['cpu_baseline']['value'] = round(result['cpu_baseline']['value'], 4)

@@ -183,6 +183,20 @@ int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, void* q_out_de
  * writes k and v into cache row *pos_dev and attends over rows 0..*pos_dev. */
 int art_decode_attention_rope(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev, void* val_cache_dev,
                               const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev, void* stream);
+/* art_decode_attention_rope spread over `parts` blocks per head (1..8), each attending over a contiguous share of
+ * the cached positions.  With parts == 1 out_dev receives the fp16 result as above.  With parts > 1 out_dev is a
+ * float buffer [heads][parts][132] that receives, per (head, part), 128 unnormalised sums, the running maximum and
+ * the running sum of exponentials (2 floats of padding); the merge
+ *     out[h,m] = sum_p e^(max_p - max) acc_p[m] / sum_p e^(max_p - max) sum_p
+ * is left to the consumer - art_gemv_w4a16_attn does it while it loads x, so the projection that follows the
+ * attention (samples/05_llama2_7b_int4.py:165-168) needs no extra launch. */
+int art_decode_attention_rope_split(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev, void* val_cache_dev,
+                                    const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev,
+                                    int parts, void* stream);
+/* y = fp16(product of the merged attention output with the int4 matrix) [+ residual]; partial_dev as written by
+ * art_decode_attention_rope_split with the same `parts` (2..8), K = heads * 128. */
+int art_gemv_w4a16_attn(const void* partial_dev, int parts, const void* qweight_dev, const void* scales_dev,
+                        const void* qzeros_dev, void* y_dev, int K, int N, const void* residual_dev, void* stream);
 int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev, const void* att_f_dev, void* out_dev,
                          int seq_len, int heads, int head_dim, const void* pos_dev, int q_dtype, int kv_dtype, int out_dtype,
                          void* stream);

@@ -15,14 +15,14 @@ def small_config():
     return LlamaConfig(n_layers=2, dim=512, n_heads=4, ffn=1024, vocab=1024, max_seq=32)
 
 
-@pytest.mark.parametrize('fused', [False, True])
-def test_decode_matches_oracle_eager_and_graph(fused):
+@pytest.mark.parametrize('fused,att_parts', [(False, 1), (True, 1), (True, 4), (True, 8)])
+def test_decode_matches_oracle_eager_and_graph(fused, att_parts):
     from antares_amd.llama import LlamaInt4Decoder, random_weights
     from oracle.llama_ref import LlamaRef
     cfg = small_config()
     w = random_weights(cfg, seed=3)
     ref = LlamaRef(cfg, w)
-    dec = LlamaInt4Decoder(cfg, w, fused=fused)
+    dec = LlamaInt4Decoder(cfg, w, fused=fused, att_parts=att_parts)
     steps = 10
     tokens, ref_logits = [5], []
     for pos in range(steps):

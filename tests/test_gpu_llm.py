@@ -156,3 +156,47 @@ def test_greedy_next_matches_torch():
                 want = 777
             assert int(pos) == new_pos and int(token) == want, (case, start_pos, use_prompt, int(token), want)
             assert torch.equal(x, embed[want])
+
+
+@pytest.mark.parametrize('parts', [2, 4, 8])
+@pytest.mark.parametrize('pos', [0, 1, 5, 130, 383])
+def test_split_attention_merged_by_the_projection(parts, pos):
+    """attention_rope_split_f16 + gemv_w4a16_attn against attention_rope_f16 + gemv_w4a16_fused (same caches, same
+    token): the cache rows written must be identical, the projected outputs equal up to fp32 reassociation."""
+    import autort
+    from antares_amd import workloads
+    dev = autort.device()
+    H, D, S = 32, 128, 384
+    g = torch.Generator().manual_seed(100 * parts + pos)
+    note(f'split attention parts={parts} pos={pos}')
+    qkv = torch.randn(3 * H * D, generator=g).half().to(dev)
+    inv = (1.0 / (10000 ** (torch.arange(0, D, 2).float() / D))).half()
+    inv_freq = torch.cat([inv, inv]).to(dev)
+    kc = (torch.randn(S, H * D, generator=g) * 0.5).half().to(dev)
+    vc = torch.randn(S, H * D, generator=g).half().to(dev)
+    att_f = torch.tensor([1 / math.sqrt(D)], dtype=torch.float32, device=dev)
+    pos_t = torch.tensor([pos], dtype=torch.int32, device=dev)
+    p = workloads.w4_problem(7, 1, H * D, 4096)
+    qw, sc, qz = (p[k].to(dev) for k in ('qweight', 'scales', 'qzeros'))
+    res = torch.randn(4096, generator=g).half().to(dev)
+    # reference path: one block per head, then the fused projection
+    kc1, vc1 = kc.clone(), vc.clone()
+    att = torch.empty(H, D, dtype=torch.float16, device=dev)
+    autort.ops.attention_rope_f16(qkv, inv_freq, kc1, vc1, att_f, att, extra=[pos_t])
+    y1 = torch.empty(4096, dtype=torch.float16, device=dev)
+    autort.ops.gemv_w4a16_fused(att.view(-1), qw, sc, qz, y1, residual=res)
+    # split path
+    kc2, vc2 = kc.clone(), vc.clone()
+    partial = torch.full((H, parts, 132), float('nan'), dtype=torch.float32, device=dev)
+    autort.ops.attention_rope_split_f16(qkv, inv_freq, kc2, vc2, att_f, partial, extra=[pos_t])
+    y2 = torch.empty(4096, dtype=torch.float16, device=dev)
+    autort.ops.gemv_w4a16_attn(partial, qw, sc, qz, y2, residual=res)
+    torch.cuda.synchronize()
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    # merging the records by hand reproduces the unsplit attention output
+    acc, mx, sm = partial[:, :, :128].double(), partial[:, :, 128].double(), partial[:, :, 129].double()
+    wgt = torch.exp(mx - mx.max(dim=1, keepdim=True).values)
+    wgt[torch.isinf(mx)] = 0
+    merged = (acc * wgt[:, :, None]).sum(1) / (sm * wgt).sum(1)[:, None]
+    assert torch.allclose(merged.float(), att.float(), rtol=2e-3, atol=2e-3)
+    assert torch.allclose(y2.float(), y1.float(), rtol=1e-2, atol=1e-2)
