@@ -5,11 +5,19 @@
 //
 // qweight is int32 [K/8, N] (eight nibbles of one column per word, least
 // significant first), scales fp32 or fp16 [K/128, N], x and y fp32 or fp16.
-// All arithmetic is fp32: nibble -> float through v_cvt_f32_ubyte after one
-// mask, one FMA per weight.  A lane owns 4 adjacent columns (one 128-bit load
-// per word row) and R word rows; k lanes meet in LDS, the column owner applies
-// scale and the fixed zero point 8 once per (group, column); K-splits are
-// added in a fixed order by the block that draws the last ticket.
+// The sample runs it in fp32, so all arithmetic here is fp32 and exact per product:
+//   * a lane owns 4 adjacent columns (one 128-bit load per word row) and 8 word rows (64 values of k);
+//     16 column lanes x 16 k lanes make a block of 64 columns x 1024 k = 32 KiB of weights, all eight loads
+//     of a lane in flight before the first is used; the grid is (N/64) x (K/1024): 688 blocks for 4096 x 11008;
+//   * the block's 1024 values of x go through LDS once (one 16-byte load per thread, an LDS-only barrier so
+//     the weight loads stay in flight) and are read back as broadcasts;
+//   * (w & 0x0F0F0F0F) and ((w >> 4) & 0x0F0F0F0F) put the even and the odd nibbles of a word into bytes;
+//     v_cvt_f32_ubyte0..3 turns each byte into a float, one FMA per weight: 2.4 VALU operations per weight;
+//   * the k lanes of a block meet in LDS; the owner of a column applies scale and the fixed zero point 8 once
+//     per (group, column): s * (acc - 8 * sum(x));
+//   * the K-splits of a column meet in one returning 64-bit atomic: a 2^-30 fixed-point partial sum with an
+//     arrival count in the top byte.  Integer addition is associative, so the result does not depend on the
+//     arrival order; the block that sees count == splits - 1 holds the total, writes y and clears the slot.
 #include "art_common.h"
 
 namespace {
@@ -20,113 +28,112 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 256;
 constexpr int CL = 16;                 // column lanes  -> 64 columns per block
 constexpr int KL = kThreads / CL;      // 16 k lanes
-constexpr int CT = 4 * CL;
-constexpr int R = 4;                   // word rows per lane (32 values of k)
-constexpr int kGroupWordRows = 16;     // 128 / 8
-constexpr int KLG = kGroupWordRows / R;
-constexpr int GB = KL / KLG;           // groups per block
+constexpr int CT = 4 * CL;             // columns per block
+constexpr int R = 8;                   // word rows per lane (64 values of k)
+constexpr int kBlockK = KL * R * 8;    // 1024 values of k per block
+constexpr int GB = kBlockK / 128;      // 8 quantisation groups per block, two k lanes each
+constexpr float kFix = 1073741824.f;   // 2^30
 
 template <class T> __device__ __forceinline__ float ldf(const T* p, size_t i) { return (float)p[i]; }
+
+__device__ __forceinline__ float ubyte(unsigned int w, int b) {       // byte b of w as a float (v_cvt_f32_ubyte<b>)
+  return (float)((w >> (8 * b)) & 0xffu);
+}
 
 template <class XT, class ST>
 __global__ __launch_bounds__(kThreads) void gemv_gptq_kernel(const XT* __restrict__ x, const unsigned int* __restrict__ qweight,
                                                              const ST* __restrict__ scales, XT* __restrict__ y, int K, int N,
-                                                             int splits, float* __restrict__ partial,
-                                                             unsigned int* __restrict__ tickets) {
-  __shared__ float red[KL][CT];
+                                                             int splits, unsigned long long* __restrict__ slots) {
+  __shared__ __align__(16) float s_x[kBlockK];
+  __shared__ __align__(16) float red[KL][CT];
   __shared__ float xsum[KL];
-  __shared__ unsigned int s_ticket;
   const int tid = threadIdx.x, cl = tid % CL, kl = tid / CL;
   const int tile = blockIdx.x, split = blockIdx.y;
   const int n0 = tile * CT + cl * 4;
   const int wrows = K >> 3;
-  const int r0 = (split * KL + kl) * R;
-  const bool active = (n0 < N) && (r0 < wrows);
+  const int r0 = (split * KL + kl) * R;                   // first word row of this lane
+  // lanes past an edge read a valid patch instead of branching; their x is zero / their columns are never written
+  const int n0c = n0 < N ? n0 : 0;
+
+  // x of the block first: it is small, comes from L2, and nothing can be multiplied without it
+  const int k0 = split * kBlockK + 4 * tid;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s_x[4 * tid + j] = (k0 + j < K) ? ldf(x, (size_t)k0 + j) : 0.f;
 
   u32x4 w[R];
 #pragma unroll
-  for (int i = 0; i < R; ++i)
-    w[i] = (active && r0 + i < wrows)
-               ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(qweight + (size_t)(r0 + i) * N + n0))
-               : u32x4{0, 0, 0, 0};
-  float xv[R][8];
-#pragma unroll
-  for (int i = 0; i < R; ++i)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) xv[i][j] = (r0 + i < wrows) ? ldf(x, (size_t)(r0 + i) * 8 + j) : 0.f;
-
+  for (int i = 0; i < R; ++i) {
+    const int r = r0 + i < wrows ? r0 + i : wrows - 1;    // past the end: any valid row, x is zero there
+    w[i] = *reinterpret_cast<const u32x4*>(qweight + (size_t)r * N + n0c);
+  }
+  // column owners fetch the scales of their column for the eight groups of the block
   const int col = tile * CT + tid;
   const bool owner = (tid < CT) && (col < N);
-  const int g0 = (split * KL * R) / kGroupWordRows, groups = K / 128;
+  const int g0 = split * GB, groups = K >> 7;
   float sc[GB];
 #pragma unroll
   for (int g = 0; g < GB; ++g) sc[g] = (owner && g0 + g < groups) ? ldf(scales, (size_t)(g0 + g) * N + col) : 0.f;
 
+  art_lds_barrier();                                     // LDS only: the weight loads stay in flight
   float acc[4] = {0.f, 0.f, 0.f, 0.f}, xs = 0.f;
 #pragma unroll
   for (int i = 0; i < R; ++i) {
+    const f32x4 xa = *reinterpret_cast<const f32x4*>(&s_x[(kl * R + i) * 8]);
+    const f32x4 xb = *reinterpret_cast<const f32x4*>(&s_x[(kl * R + i) * 8 + 4]);
+    xs += ((xa[0] + xa[1]) + (xa[2] + xa[3])) + ((xb[0] + xb[1]) + (xb[2] + xb[3]));
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      xs += xv[i][j];
-#pragma unroll
-      for (int c = 0; c < 4; ++c) acc[c] = fmaf(xv[i][j], (float)((w[i][c] >> (4 * j)) & 15u), acc[c]);
+    for (int c = 0; c < 4; ++c) {
+      const unsigned int even = w[i][c] & 0x0F0F0F0Fu, odd = (w[i][c] >> 4) & 0x0F0F0F0Fu;   // nibbles 0,2,4,6 | 1,3,5,7
+      float a = acc[c];
+      a = fmaf(xa[0], ubyte(even, 0), a);
+      a = fmaf(xa[1], ubyte(odd, 0), a);
+      a = fmaf(xa[2], ubyte(even, 1), a);
+      a = fmaf(xa[3], ubyte(odd, 1), a);
+      a = fmaf(xb[0], ubyte(even, 2), a);
+      a = fmaf(xb[1], ubyte(odd, 2), a);
+      a = fmaf(xb[2], ubyte(even, 3), a);
+      a = fmaf(xb[3], ubyte(odd, 3), a);
+      acc[c] = a;
     }
   }
   *reinterpret_cast<f32x4*>(&red[kl][cl * 4]) = f32x4{acc[0], acc[1], acc[2], acc[3]};
   if (cl == 0) xsum[kl] = xs;
   __syncthreads();
+  if (!owner) return;
 
   float res = 0.f;
-  if (tid < CT) {
 #pragma unroll
-    for (int g = 0; g < GB; ++g) {
-      float a = 0.f, s = 0.f;
-#pragma unroll
-      for (int q = 0; q < KLG; ++q) {
-        a += red[g * KLG + q][tid];
-        s += xsum[g * KLG + q];
-      }
-      res += sc[g] * (a - 8.f * s);
-    }
+  for (int g = 0; g < GB; ++g) {                         // a group is two k lanes
+    const float a = red[2 * g][tid] + red[2 * g + 1][tid];
+    const float s = xsum[2 * g] + xsum[2 * g + 1];
+    res += sc[g] * (a - 8.f * s);
   }
   if (splits == 1) {
-    if (owner) y[col] = (XT)res;
+    y[col] = (XT)res;
     return;
   }
-  if (owner) __hip_atomic_store(&partial[(size_t)split * N + col], res, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  // The partial sums were written through to device-coherent memory; wait until
-  // they have landed (vmcnt(0)) before this block's ticket can be seen.  A device-scope
-  // release fence would do the same but writes back the whole L2 of the XCD.
-  __atomic_signal_fence(__ATOMIC_SEQ_CST);
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  __syncthreads();
-  if (tid == 0) s_ticket = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __syncthreads();
-  if (s_ticket != (unsigned int)(splits - 1)) return;
-  __atomic_signal_fence(__ATOMIC_SEQ_CST);
-  if (owner) {
-    float r = 0.f;
-    for (int s = 0; s < splits; ++s)
-      r += __hip_atomic_load(&partial[(size_t)s * N + col], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    y[col] = (XT)r;
+  // one returning atomic: [arrival count : 8][2^-30 fixed-point sum : 56]
+  unsigned long long* slot = slots + col;
+  const long long mine = (1LL << 56) + __float2ll_rn(res * kFix);
+  const long long old = (long long)__hip_atomic_fetch_add(slot, (unsigned long long)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (((old + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
+    const long long total = old + mine - ((long long)splits << 56);
+    y[col] = (XT)((float)total * (1.f / kFix));
+    *slot = 0ull;                       // ready for the next launch (stream order makes this visible)
   }
-  if (tid == 0) tickets[tile] = 0u;
 }
 
 template <class XT, class ST>
 int launch(const void* x, const void* qw, const void* sc, void* y, int K, int N, hipStream_t stream) {
-  const int wrows = K / 8;
   const int tiles = (N + CT - 1) / CT;
-  const int splits = (wrows + KL * R - 1) / (KL * R);
+  const int splits = (K + kBlockK - 1) / kBlockK;
+  ART_REQUIRE(splits <= 127, "art_gemv_gptq: K too large (%d)", K);
   art::Workspace& ws = art::workspace();
   ART_REQUIRE(ws.base != nullptr, "art_gemv_gptq: call art_init first");
-  const size_t ticket_bytes = art::kGemvTicketBytes;
-  ART_REQUIRE((size_t)tiles * 4 <= ticket_bytes, "art_gemv_gptq: N too large (%d)", N);
-  ART_REQUIRE(splits == 1 || art::kScratchOffset + (size_t)splits * N * 4 <= ws.bytes, "art_gemv_gptq: workspace too small");
-  unsigned int* tickets = reinterpret_cast<unsigned int*>(ws.base);
-  float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(ws.base) + art::kScratchOffset);
+  ART_REQUIRE(art::kSlotOffset + (size_t)N * 8 <= art::kScratchOffset, "art_gemv_gptq: N too large (%d)", N);
+  unsigned long long* slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(ws.base) + art::kSlotOffset);
   gemv_gptq_kernel<XT, ST><<<dim3(tiles, splits), dim3(kThreads), 0, stream>>>(
-      (const XT*)x, (const unsigned int*)qw, (const ST*)sc, (XT*)y, K, N, splits, partial, tickets);
+      (const XT*)x, (const unsigned int*)qw, (const ST*)sc, (XT*)y, K, N, splits, slots);
   ART_LAUNCH_CHECK();
   return 0;
 }
