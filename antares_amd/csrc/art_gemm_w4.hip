@@ -5,8 +5,9 @@
 // dequant + matmul program of samples/05_llama2_7b_int4.py:135-144 is exported with a batch axis.
 //
 // Design for MI355X:
-//   * the weights are read from HBM exactly once; a block owns 128 columns (one full 128-byte line of
-//     every packed row) and a contiguous range of k groups;
+//   * the weights are read from HBM exactly once; a block of eight waves owns 256 columns (two full
+//     128-byte lines of every packed row, and as many bytes of weights as of x per step) and a contiguous
+//     range of k groups;
 //   * unpacking is fused into the LDS staging: 16 bytes (16 columns x 2 k) become two rows of fp16
 //     (q - z) values - exact small integers - with one shift, four v_bitop3_b32 and four packed
 //     subtractions per word.  The columns of every group of four land in LDS in the order 0,2,1,3,
@@ -18,8 +19,7 @@
 //   * a step is 64 k.  LDS holds two steps: while the matrix cores work on step t, the same waves
 //     unpack step t+1 into the other buffer; one barrier per step, and it waits for LDS only, so the
 //     register stages (a whole group = two steps each, two of them) keep their global loads in flight
-//     across it.  58 KiB of LDS and < 256 registers: two blocks per compute unit, whose phases drift
-//     apart and fill each other's gaps;
+//     across it.  92 KiB of LDS and < 256 registers: one block = two waves per SIMD on every compute unit;
 //   * split-K without atomics (5.6 M float atomics cost 75 us on this chip): each K-split writes its
 //     fp32 tile to the library workspace and a second small kernel adds the splits in a fixed order
 //     and rounds once to fp16 - results do not depend on timing.
@@ -39,7 +39,8 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
-constexpr int BM = 64, BN = 128, GK = 128;     // rows and columns of a block, k of a quantisation group
+constexpr int kThreads = 512;                  // 8 waves: 32 columns each
+constexpr int BM = 64, BN = kThreads / 2, GK = 128;   // rows and columns of a block, k of a quantisation group
 constexpr int SK = 64;                         // k of a step (half a group)
 constexpr int W_LD = BN + 32;                  // halves per weight row in LDS: 320 bytes, so the four k rows
                                                // a transposing read touches fall on disjoint banks
@@ -63,7 +64,7 @@ __device__ __forceinline__ unsigned int and_or(unsigned int w, unsigned int mask
 __device__ __forceinline__ int unpermute(int p) { return (p & ~3) | ((p & 1) << 1) | ((p >> 1) & 1); }
 
 template <int MT>   // MT accumulator tiles of 32 rows: 1 for M <= 32, 2 for M <= 64
-__global__ __launch_bounds__(256, 2) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
+__global__ __launch_bounds__(kThreads, 512 / kThreads) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
                                                              const _Float16* __restrict__ scales,
                                                              const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y,
                                                              float* __restrict__ partial, int M, int K, int N, int splits,
@@ -81,18 +82,20 @@ __global__ __launch_bounds__(256, 2) void gemm_w4a16_kernel(const _Float16* __re
   const int groups = g_end - g_begin;
 
   // ---- global -> register staging, one quantisation group (two steps) per stage
-  // weights of a step: 32 packed rows x 128 bytes = 256 chunks of 16 bytes, one per thread
-  const int cc = tid & 7;                       // 16-column chunk
-  const int pr = tid >> 3;                      // packed row of the step
+  // weights of a step: 32 packed rows x BN bytes = kThreads chunks of 16 bytes, one per thread
+  constexpr int kChunks = BN / 16;              // 16-column chunks per packed row
+  const int cc = tid % kChunks;                 // 16-column chunk
+  const int pr = tid / kChunks;                 // packed row of the step (kThreads / kChunks = 32 of them)
   const bool col_ok = n0 + cc * 16 < N;         // N % 16 == 0: a chunk is inside or outside as a whole
   const int wcol = col_ok ? n0 + cc * 16 : 0;   // columns past N: load valid memory, results are never stored
   const unsigned char* wp = qweight + (size_t)pr * N + wcol;
-  // x of a step: MT*32 rows x 64 k = MT*256 chunks of 16 bytes, MT per thread; rows past M repeat row M-1
-  const _Float16* xp[MT];
-  int xs_off[MT];
+  // x of a step: MT*32 rows x 64 k = MT*256 chunks of 16 bytes, XC per thread; rows past M repeat row M-1
+  constexpr int XC = (MT * 256 + kThreads - 1) / kThreads;     // chunks of x per thread and step
+  const _Float16* xp[XC];
+  int xs_off[XC];
 #pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
+  for (int i = 0; i < XC; ++i) {
+    const int c = tid + kThreads * i, row = c >> 3, kc = c & 7;
     xp[i] = x + (size_t)(row < M ? row : M - 1) * K + kc * 8;
     xs_off[i] = row * X_LD + kc * 8;
   }
@@ -108,7 +111,7 @@ __global__ __launch_bounds__(256, 2) void gemm_w4a16_kernel(const _Float16* __re
 
   // Stages are indexed statically (a run-time index would put the arrays in scratch memory).
   u32x4 wq[2][2];      // [stage][step of the group]
-  u32x4 xr[2][2][MT];
+  u32x4 xr[2][2][XC];
   u32x2 zq[2];
   _Float16 sc16[2];
   auto load_group = [&](int g, auto tag) {
@@ -116,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void gemm_w4a16_kernel(const _Float16* __re
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
-      for (int i = 0; i < MT; ++i) xr[S][h][i] = *reinterpret_cast<const u32x4*>(xp[i] + (size_t)g * GK + h * SK);
+      for (int i = 0; i < XC; ++i) xr[S][h][i] = *reinterpret_cast<const u32x4*>(xp[i] + (size_t)g * GK + h * SK);
       wq[S][h] = *reinterpret_cast<const u32x4*>(wp + ((size_t)g * (GK / 2) + h * (SK / 2)) * N);
     }
     zq[S] = *reinterpret_cast<const u32x2*>(qzeros + (size_t)g * (N / 2) + (wcol >> 1));
@@ -165,7 +168,7 @@ __global__ __launch_bounds__(256, 2) void gemm_w4a16_kernel(const _Float16* __re
     *reinterpret_cast<u32x4*>(row + W_LD) = odd[0];
     *reinterpret_cast<u32x4*>(row + W_LD + 8) = odd[1];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) *reinterpret_cast<u32x4*>(Xs + buf * X_TILE + xs_off[i]) = xr[S][H][i];
+    for (int i = 0; i < XC; ++i) *reinterpret_cast<u32x4*>(Xs + buf * X_TILE + xs_off[i]) = xr[S][H][i];
   };
   // Operand fragments of two k-steps of 16 (kk0, kk0 + 1) of the step in LDS buffer `buf`.
   auto read_frags = [&](h8 (&fa)[2][MT], h8 (&fb)[2], int buf, int kk0) {
@@ -198,7 +201,7 @@ __global__ __launch_bounds__(256, 2) void gemm_w4a16_kernel(const _Float16* __re
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
       __builtin_amdgcn_sched_group_barrier(0x002, 24, 0);       \
     }                                                           \
-    __builtin_amdgcn_sched_group_barrier(0x200, 4 + MT, 0);     \
+    __builtin_amdgcn_sched_group_barrier(0x200, 4 + XC, 0);     \
     __builtin_amdgcn_sched_barrier(0);                          \
   } while (0)
   // Second half: the MFMAs of k-steps 2,3 with the first operand reads of the next step (and the global loads) between them.
@@ -293,13 +296,13 @@ __global__ __launch_bounds__(256) void gemm_w4a16_combine_kernel(const float* __
   *reinterpret_cast<h4*>(y + i * 4) = out;
 }
 
-// Number of K-splits: as many blocks as the chip holds at once (two per compute unit), but at least
+// Number of K-splits: as many blocks as the chip holds at once (one per compute unit), but at least
 // two groups per block, no more partial-tile bytes than weight bytes (every split adds an fp32 copy of
-// the output to the traffic), and no more than the scratch space allows.  Measured optimum at M = 64 on
-// MI355X: 8 splits for 4096x4096 and 11008x4096, 5 for 4096x11008, 2 for 4096x32000.
+// the output to the traffic), and no more than the scratch space allows.  The rule lands on the measured
+// optimum at M = 64 on MI355X: 8 splits for 4096x4096, 5 for 4096x11008, 16 for 11008x4096, 2 for 4096x32000.
 int choose_splits(int rows, int N, int K, size_t scratch_bytes, int compute_units) {
   const int col_tiles = (N + BN - 1) / BN, G = K / GK;
-  int s = 2 * compute_units / col_tiles;
+  int s = (512 / kThreads) * compute_units / col_tiles;      // blocks that are resident at once
   if (s > G / 2) s = G / 2;
   const size_t per_split = (size_t)rows * N * sizeof(float);
   const size_t weight_bytes = (size_t)K * N / 2;
@@ -343,11 +346,11 @@ extern "C" int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const 
     _Float16* ys = (_Float16*)y_dev + (size_t)m0 * N;
     const dim3 grid(col_tiles * splits);
     if (rows <= 32)
-      gemm_w4a16_kernel<1><<<grid, 256, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
+      gemm_w4a16_kernel<1><<<grid, kThreads, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
                                                          col_tiles, mg);
     else
-      gemm_w4a16_kernel<2><<<grid, 256, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
+      gemm_w4a16_kernel<2><<<grid, kThreads, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
                                                          col_tiles, mg);
     ART_LAUNCH_CHECK();
