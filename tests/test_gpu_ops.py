@@ -144,7 +144,7 @@ def test_w4a16_gemv_matches_oracle(autort, M, K, N):
                                    (100, 512, 4096), (200, 4096, 512),
                                    (64, 4096, 4096), (64, 4096, 11008), (64, 11008, 4096), (64, 4096, 32000)])
 def test_w4a16_gemm_matches_oracle(autort, M, K, N):
-    """Batches of more than 8 rows run on the matrix cores (one pass over the weights per 64 rows)."""
+    """Batches of four rows and more run on the matrix cores (one pass over the weights per 64 rows)."""
     from oracle import hot_ops
     note(f'w4a16 gemm M={M} K={K} N={N}')
     p = workloads.w4_problem(K + N + M, M, K, N)
@@ -163,6 +163,27 @@ def test_w4a16_gemm_matches_oracle(autort, M, K, N):
     y1 = f(args[0][m:m + 1].contiguous(), *args[1:])
     assert np.allclose(y1.cpu().numpy().astype(np.float32), want[m:m + 1].astype(np.float32), **FP16_TOL)
     assert np.allclose(y1.float().cpu().numpy(), y[m:m + 1].float().cpu().numpy(), rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize('M,K,N', [(4, 512, 256), (5, 1024, 144), (6, 4096, 512), (7, 384, 1040), (8, 4096, 4096)])
+def test_w4a16_gemv_entry_point_up_to_eight_rows(autort, M, K, N):
+    """`art_gemv_w4a16` takes up to 8 rows (the weights are streamed once per pair of rows); autort.export sends
+    4 rows and more to the matrix-core kernel, so the entry point is called directly here."""
+    from ctypes import c_void_p
+    from antares_amd.runtime import capi
+    from oracle import hot_ops
+    note(f'art_gemv_w4a16 direct M={M} K={K} N={N}')
+    p = workloads.w4_problem(K + N + M, M, K, N)
+    dev = autort.device()
+    capi.init(dev.index or 0)
+    x, q, s_, z = (p[k].to(dev) for k in ('x', 'qweight', 'scales', 'qzeros'))
+    y = torch.empty(M, N, dtype=torch.float16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    capi.check(capi.lib().art_gemv_w4a16(c_void_p(x.data_ptr()), c_void_p(q.data_ptr()), c_void_p(s_.data_ptr()),
+                                         c_void_p(z.data_ptr()), c_void_p(y.data_ptr()), M, K, N, c_void_p(stream)))
+    torch.cuda.synchronize()
+    want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy())
+    assert np.allclose(y.cpu().numpy().astype(np.float32), want.astype(np.float32), **FP16_TOL)
 
 
 def test_w4a16_generic_lowering_agrees(autort):
