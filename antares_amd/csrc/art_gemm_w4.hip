@@ -1,4 +1,4 @@
-// Weight-only int4 GEMM for a batch of rows (prefill, M > 8): the same arithmetic as the GEMV of
+// Weight-only int4 GEMM for a batch of rows (prefill, four rows and more): the same arithmetic as the GEMV of
 // art_gemv_w4.hip,
 //     y[m,n] = sum_g s[g,n] * sum_{k in group g} x[m,k] * (q[k,n] - z[g,n]),      group = 128 k,
 // with the inner sums on the matrix cores.  Replaces the kernel the reference generates when the
