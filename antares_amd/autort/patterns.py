@@ -41,22 +41,32 @@ def _gptq_inputs(xdt: str, sdt: str):
     return [f'input0={xdt}[S:4096]', 'qweight=int32[L:512, N:12288]', f'scales={sdt}[K:32, N:12288]']
 
 
+def _gptq_roles(op):
+    """Which declared tensor is x, qweight, scales and the output (the ABI order is by name; roles go by dtype and
+    rank).  Worked out once per operator."""
+    roles = getattr(op, '_gptq_roles', None)
+    if roles is None:
+        g = op.fused
+        names = {n: g.tensors[n] for n in g.abi_inputs}
+        q_name = next(n for n, t in names.items() if t.dtype == 'int32')
+        x_name = next(n for n, t in names.items() if len(t.shape) == 1)
+        s_name = next(n for n in names if n not in (q_name, x_name))
+        roles = (x_name, q_name, s_name, g.abi_outputs[0], int(names[x_name].dtype == 'float16'),
+                 int(names[s_name].dtype == 'float16'))
+        op._gptq_roles = roles
+    return roles
+
+
 def _gptq_handler(op, bound, env, stream) -> bool:
-    g = op.fused
-    x_name, q_name, s_name = g.abi_inputs[0], g.abi_inputs[1], g.abi_inputs[2]
-    # abi order is sorted by name; find roles by dtype / rank instead
-    names = {n: g.tensors[n] for n in g.abi_inputs}
-    q_name = next(n for n, t in names.items() if t.dtype == 'int32')
-    x_name = next(n for n, t in names.items() if len(t.shape) == 1)
-    s_name = next(n for n in names if n not in (q_name, x_name))
-    out = bound[g.abi_outputs[0]]
+    x_name, q_name, s_name, out_name, x_f16, s_f16 = _gptq_roles(op)
+    out = bound[out_name]
     x, q, s = bound[x_name], bound[q_name], bound[s_name]
     K, N = x.shape[0], q.shape[1]
-    if K % 128 or N % 4 or q.shape[0] * 8 != K or s.shape[0] * 128 != K or q.data_ptr() % 16:
+    qp = q.data_ptr()
+    if K % 128 or N % 4 or q.shape[0] * 8 != K or s.shape[0] * 128 != K or qp % 16:
         return False
-    capi.check(capi.lib().art_gemv_gptq(c_void_p(x.data_ptr()), c_void_p(q.data_ptr()), c_void_p(s.data_ptr()),
-                                       c_void_p(out.data_ptr()), K, N, int(names[x_name].dtype == 'float16'),
-                                       int(names[s_name].dtype == 'float16'), c_void_p(stream)))
+    capi.check(capi.lib().art_gemv_gptq(c_void_p(x.data_ptr()), c_void_p(qp), c_void_p(s.data_ptr()),
+                                       c_void_p(out.data_ptr()), K, N, x_f16, s_f16, c_void_p(stream)))
     return True
 
 

@@ -17,6 +17,7 @@ int4 dequant + GEMV of samples/05_llama2_7b_int4.py:135-139 becomes one kernel.
 from __future__ import annotations
 
 from dataclasses import dataclass, field, replace
+from functools import cached_property
 from typing import Dict, List, Optional, Sequence, Tuple
 
 from .nodes import Dim, Expr, rewrite, walk
@@ -34,13 +35,13 @@ class Graph:
     dims: Dict[str, Optional[int]]               # named run-time dims -> default extent
     source: str = ''
 
-    # -- argument order -----------------------------------------------------
-    @property
+    # -- argument order (computed once: a Graph is not changed after it is built) --------
+    @cached_property
     def inout(self) -> List[str]:
         written = {s.output for s in self.statements}
         return [n for n in self.declared if n in written]
 
-    @property
+    @cached_property
     def used_inputs(self) -> List[str]:
         used = set()
         for s in self.statements:
@@ -48,16 +49,16 @@ class Graph:
         produced = {s.output for s in self.statements}
         return [n for n in self.declared if n in used and n not in produced]
 
-    @property
+    @cached_property
     def abi_inputs(self) -> List[str]:
         return sorted(self.used_inputs)
 
-    @property
+    @cached_property
     def abi_outputs(self) -> List[str]:
         outs = set(self.outputs) | set(self.inout)
         return sorted(outs)
 
-    @property
+    @cached_property
     def dim_names(self) -> List[str]:
         return sorted(self.dims)
 
