@@ -132,16 +132,16 @@ class Rotary:
                 raise ValueError(f'{self.name}: inv_freq is too short')
         _require_cuda(x, freq, out)
         pos_dev, pos = _pos_args(extra, self.name)
-        stride = 0
+        stride, out_rows = 0, 0
         if out.numel() != x.numel():
             # a whole [positions, heads*head_dim] cache: the row is chosen by the device-side position
             if not pos_dev.value or out.numel() % x.numel() != 0:
                 raise ValueError(f'{self.name}: out must match x in size (or be a cache with extra=[position tensor])')
-            stride = x.numel()
+            stride, out_rows = x.numel(), out.numel() // x.numel()
         if out.dtype != x.dtype:
             raise ValueError(f'{self.name}: out must have the dtype of x')
         capi.check(capi.lib().art_rotary(c_void_p(x.data_ptr()), c_void_p(freq.data_ptr()), c_void_p(out.data_ptr()), heads,
-                                        head_dim, int(self.interleaved), pos_dev, pos, stride, _dt(x, 'x'), _dt(freq, 'inv_freq'),
+                                        head_dim, int(self.interleaved), pos_dev, pos, stride, out_rows, _dt(x, 'x'), _dt(freq, 'inv_freq'),
                                         _dt(out, 'out'), c_void_p(current_stream_handle())))
         return out
 
@@ -239,7 +239,7 @@ class AttentionRope:
         capi.check(capi.lib().art_decode_attention_rope(c_void_p(qkv.data_ptr()), c_void_p(inv_freq.data_ptr()),
                                                        c_void_p(key_cache.data_ptr()), c_void_p(val_cache.data_ptr()),
                                                        c_void_p(att_f.data_ptr()), c_void_p(out.data_ptr()), heads, head_dim, pos_dev,
-                                                       c_void_p(current_stream_handle())))
+                                                       key_cache.numel() // (heads * head_dim), c_void_p(current_stream_handle())))
         return out
 
 
@@ -267,7 +267,8 @@ class AttentionRopeSplit:
             raise TypeError('attention_rope_split_f16: extra=[pos] must be a 1-element int32 GPU tensor')
         capi.check(capi.lib().art_decode_attention_rope_split(
             c_void_p(qkv.data_ptr()), c_void_p(inv_freq.data_ptr()), c_void_p(key_cache.data_ptr()), c_void_p(val_cache.data_ptr()),
-            c_void_p(att_f.data_ptr()), c_void_p(partial.data_ptr()), heads, head_dim, pos_dev, parts,
+            c_void_p(att_f.data_ptr()), c_void_p(partial.data_ptr()), heads, head_dim, pos_dev,
+            key_cache.numel() // (heads * head_dim), parts,
             c_void_p(current_stream_handle())))
         return partial
 
@@ -312,7 +313,7 @@ class RopeQkvStore:
             raise TypeError(f'{self.name}: extra=[pos] must be a 1-element int32 GPU tensor')
         capi.check(capi.lib().art_rope_qkv_store(c_void_p(qkv.data_ptr()), c_void_p(inv_freq.data_ptr()), c_void_p(q_out.data_ptr()),
                                                 c_void_p(key_cache.data_ptr()), c_void_p(val_cache.data_ptr()), heads, head_dim,
-                                                pos_dev, _dt(qkv, 'qkv'), _dt(inv_freq, 'inv_freq'), c_void_p(current_stream_handle())))
+                                                pos_dev, key_cache.numel() // (heads * head_dim), _dt(qkv, 'qkv'), _dt(inv_freq, 'inv_freq'), c_void_p(current_stream_handle())))
         return q_out
 
 

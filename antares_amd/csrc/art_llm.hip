@@ -75,9 +75,12 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const XT* __restrict__ x,
 template <class XT, class FT, class OT, bool INTERLEAVED>
 __global__ __launch_bounds__(256) void rotary_kernel(const XT* __restrict__ x, const FT* __restrict__ freq, OT* __restrict__ out,
                                                       int heads, int half, const int* __restrict__ pos_dev, int pos_host,
-                                                      long long out_row_stride) {
+                                                      long long out_row_stride, int out_rows) {
   const int pos = pos_dev ? *pos_dev : pos_host;
-  out += (size_t)pos * out_row_stride;                // out is a [positions, heads*head_dim] cache when the stride is set
+  // out is a [out_rows, heads*head_dim] cache when the stride is set; a position past its end writes nothing
+  // (a recorded graph replayed too often must not run off the cache)
+  if (out_row_stride > 0 && (pos < 0 || pos >= out_rows)) return;
+  out += (size_t)pos * out_row_stride;
   const int i = blockIdx.x * 256 + threadIdx.x;       // pair index over heads * half
   if (i >= heads * half) return;
   const int h = i / half, j = i % half;
@@ -159,13 +162,28 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
   // parts > 1: `parts` blocks share a head, each attends over a contiguous range of the cached positions and
   // leaves its unnormalised state in partial[head][part][kAttPartialStride] = { acc[128], max, sum, -, - };
   // whoever consumes the result merges them (the o-projection does it while it loads x).
-  constexpr int D = 128, U = 4;
+  constexpr int D = 128, U = 4;                          // len_host: the length, or the rows of the cache when len_dev is given
   __shared__ float s_m[kAttWaves], s_l[kAttWaves];
   __shared__ float s_acc[kAttWaves][D];
   __shared__ float s_q[D];
   __shared__ float s_k[D], s_v[D];
   const int S = len_dev ? (*len_dev + 1) : len_host;     // device form carries the position, length = pos + 1
   const int h = blockIdx.x / parts, part = blockIdx.x % parts, tid = threadIdx.x;
+  if (len_dev && (S < 1 || S > len_host)) {
+    // The position read on the device is past the end of the cache (len_host rows): touch no cache row and
+    // hand on NaN, which every consumer propagates, instead of running off the allocation.
+    if (tid < D) {
+      const float nan = __builtin_nanf("");
+      if (parts == 1) {
+        st(out, (size_t)h * D + tid, nan);
+      } else {
+        float* dst = partial + ((size_t)h * parts + part) * kAttPartialStride;
+        dst[tid] = nan;
+        if (tid == 0) { dst[D] = 0.f; dst[D + 1] = nan; }
+      }
+    }
+    return;
+  }
   const int sub = tid & 7, group = tid >> 3;
   const float scale = att_f[0];
   const size_t row = (size_t)heads * D;
@@ -318,8 +336,9 @@ namespace {
 template <class T, class FT>
 __global__ __launch_bounds__(256) void rope_qkv_store_kernel(const T* __restrict__ qkv, const FT* __restrict__ freq, T* __restrict__ q_out,
                                                               T* __restrict__ key_cache, T* __restrict__ val_cache, int heads, int half,
-                                                              const int* __restrict__ pos_dev) {
+                                                              const int* __restrict__ pos_dev, int max_positions) {
   const int pos = *pos_dev;
+  if (pos < 0 || pos >= max_positions) return;        // past the end of the caches: write nothing
   const int dim = heads * half * 2;
   const int pairs = heads * half;
   const int i = blockIdx.x * 256 + threadIdx.x;
@@ -370,17 +389,17 @@ extern "C" int art_rmsnorm(const void* x_dev, const void* vsum_dev, const void* 
 }
 
 extern "C" int art_rotary(const void* x_dev, const void* freq_dev, void* out_dev, int heads, int head_dim, int interleaved,
-                          const void* pos_dev, int pos, long long out_row_stride, int x_dtype, int freq_dtype, int out_dtype,
-                          void* stream) {
+                          const void* pos_dev, int pos, long long out_row_stride, int out_rows, int x_dtype, int freq_dtype,
+                          int out_dtype, void* stream) {
   ART_REQUIRE(x_dev && freq_dev && out_dev && heads >= 1 && head_dim >= 2 && head_dim % 2 == 0, "art_rotary: bad arguments");
   ART_REQUIRE(ART_DT_OK(x_dtype) && ART_DT_OK(freq_dtype) && ART_DT_OK(out_dtype), "art_rotary: dtype codes are 0 (f32) / 1 (f16)");
   ART_REQUIRE(x_dtype == out_dtype, "art_rotary: input and output must have the same dtype");
-  ART_REQUIRE(out_row_stride >= 0, "art_rotary: negative row stride");
+  ART_REQUIRE(out_row_stride >= 0 && (out_row_stride == 0 || out_rows >= 1), "art_rotary: a cache output needs its row stride and row count");
   hipStream_t st = (hipStream_t)stream;
   const int half = head_dim / 2, pairs = heads * half;
   const dim3 grid((pairs + 255) / 256), block(256);
   const int* pd = (const int*)pos_dev;
-#define ART_ROT(XT, FT, IL) rotary_kernel<XT, FT, XT, IL><<<grid, block, 0, st>>>((const XT*)x_dev, (const FT*)freq_dev, (XT*)out_dev, heads, half, pd, pos, out_row_stride)
+#define ART_ROT(XT, FT, IL) rotary_kernel<XT, FT, XT, IL><<<grid, block, 0, st>>>((const XT*)x_dev, (const FT*)freq_dev, (XT*)out_dev, heads, half, pd, pos, out_row_stride, out_rows)
   if (interleaved) {
     if (x_dtype == 0) { if (freq_dtype == 0) ART_ROT(float, float, true); else ART_ROT(float, _Float16, true); }
     else { if (freq_dtype == 0) ART_ROT(_Float16, float, true); else ART_ROT(_Float16, _Float16, true); }
@@ -398,7 +417,7 @@ extern "C" int art_decode_attention(const void* q_dev, const void* k_dev, const 
                                     int out_dtype, void* stream) {
   ART_REQUIRE(q_dev && k_dev && v_dev && att_f_dev && out_dev, "art_decode_attention: null pointer");
   ART_REQUIRE(head_dim == 128, "art_decode_attention: head_dim must be 128 (got %d)", head_dim);
-  ART_REQUIRE(heads >= 1 && (pos_dev || seq_len >= 1), "art_decode_attention: bad shape");
+  ART_REQUIRE(heads >= 1 && seq_len >= 1, "art_decode_attention: bad shape (seq_len is the length, or the rows of the cache when the position is read on the device)");
   ART_REQUIRE(ART_DT_OK(q_dtype) && ART_DT_OK(kv_dtype) && ART_DT_OK(out_dtype), "art_decode_attention: dtype codes are 0 (f32) / 1 (f16)");
   ART_REQUIRE(q_dtype == out_dtype, "art_decode_attention: q and out must have the same dtype");
   ART_REQUIRE(((uintptr_t)k_dev % 16) == 0 && ((uintptr_t)v_dev % 16) == 0, "art_decode_attention: k and v must be 16-byte aligned");
@@ -414,15 +433,17 @@ extern "C" int art_decode_attention(const void* q_dev, const void* k_dev, const 
 }
 
 extern "C" int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, void* q_out_dev, void* key_cache_dev, void* val_cache_dev,
-                                  int heads, int head_dim, const void* pos_dev, int dtype, int freq_dtype, void* stream) {
+                                  int heads, int head_dim, const void* pos_dev, int max_positions, int dtype, int freq_dtype,
+                                  void* stream) {
   ART_REQUIRE(qkv_dev && freq_dev && q_out_dev && key_cache_dev && val_cache_dev && pos_dev, "art_rope_qkv_store: null pointer");
+  ART_REQUIRE(max_positions >= 1, "art_rope_qkv_store: the caches have no rows");
   ART_REQUIRE(heads >= 1 && head_dim >= 2 && head_dim % 2 == 0, "art_rope_qkv_store: bad shape");
   ART_REQUIRE(ART_DT_OK(dtype) && ART_DT_OK(freq_dtype), "art_rope_qkv_store: dtype codes are 0 (f32) / 1 (f16)");
   const int half = head_dim / 2, dim = heads * head_dim;
   const dim3 grid((2 * heads * half + dim + 255) / 256), block(256);
   hipStream_t st = (hipStream_t)stream;
   const int* pd = (const int*)pos_dev;
-#define ART_RQS(T, FT) rope_qkv_store_kernel<T, FT><<<grid, block, 0, st>>>((const T*)qkv_dev, (const FT*)freq_dev, (T*)q_out_dev, (T*)key_cache_dev, (T*)val_cache_dev, heads, half, pd)
+#define ART_RQS(T, FT) rope_qkv_store_kernel<T, FT><<<grid, block, 0, st>>>((const T*)qkv_dev, (const FT*)freq_dev, (T*)q_out_dev, (T*)key_cache_dev, (T*)val_cache_dev, heads, half, pd, max_positions)
   if (dtype == 0) { if (freq_dtype == 0) ART_RQS(float, float); else ART_RQS(float, _Float16); }
   else { if (freq_dtype == 0) ART_RQS(_Float16, float); else ART_RQS(_Float16, _Float16); }
 #undef ART_RQS
@@ -432,23 +453,24 @@ extern "C" int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, voi
 
 extern "C" int art_decode_attention_rope(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev, void* val_cache_dev,
                                          const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev,
-                                         void* stream) {
+                                         int max_positions, void* stream) {
   return art_decode_attention_rope_split(qkv_dev, inv_freq_dev, key_cache_dev, val_cache_dev, att_f_dev, out_dev, heads, head_dim,
-                                         pos_dev, 1, stream);
+                                         pos_dev, max_positions, 1, stream);
 }
 
 extern "C" int art_decode_attention_rope_split(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev,
                                                void* val_cache_dev, const void* att_f_dev, void* out_dev, int heads, int head_dim,
-                                               const void* pos_dev, int parts, void* stream) {
+                                               const void* pos_dev, int max_positions, int parts, void* stream) {
   ART_REQUIRE(qkv_dev && inv_freq_dev && key_cache_dev && val_cache_dev && att_f_dev && out_dev && pos_dev,
               "art_decode_attention_rope: null pointer");
   ART_REQUIRE(head_dim == 128 && heads >= 1, "art_decode_attention_rope: head_dim must be 128 (got %d)", head_dim);
   ART_REQUIRE(parts >= 1 && parts <= 16, "art_decode_attention_rope: parts must be in 1..16 (got %d)", parts);
+  ART_REQUIRE(max_positions >= 1, "art_decode_attention_rope: the caches have no rows");
   ART_REQUIRE(((uintptr_t)key_cache_dev % 16) == 0 && ((uintptr_t)val_cache_dev % 16) == 0 && ((uintptr_t)out_dev % 16) == 0,
               "art_decode_attention_rope: caches and output must be 16-byte aligned");
   attention_kernel<_Float16, _Float16, _Float16, true><<<dim3(heads * parts), dim3(kAttThreads), 0, (hipStream_t)stream>>>(
       (const _Float16*)qkv_dev, (_Float16*)key_cache_dev, (_Float16*)val_cache_dev, (const float*)att_f_dev,
-      parts == 1 ? (_Float16*)out_dev : nullptr, heads, (const int*)pos_dev, 0, (const _Float16*)inv_freq_dev,
+      parts == 1 ? (_Float16*)out_dev : nullptr, heads, (const int*)pos_dev, max_positions, (const _Float16*)inv_freq_dev,
       parts == 1 ? nullptr : (float*)out_dev, parts);
   ART_LAUNCH_CHECK();
   return 0;

@@ -164,25 +164,31 @@ int art_partition_even_first_i32(const void* in_dev, void* out_dev, long long n,
  *   flat vector: (x[2j], x[2j+1]) rotated by pos * freq[j], freq having one entry
  *   per pair of the whole vector.  pos is read from pos_dev (int32 on the device)
  *   when pos_dev != NULL, else taken from `pos`.  With out_row_stride > 0 the result
- *   is written at out + pos * out_row_stride elements (a row of a key cache).
+ *   is written at out + pos * out_row_stride elements (a row of a key cache of out_rows rows;
+ *   a position outside 0..out_rows-1 writes nothing).
  * art_decode_attention: one query per head against a cache of seq_len positions:
  *     a[h,s] = att_f[0] * sum_m q[h,m] k[s,h,m];  p = softmax_s(a);  out[h,m] = sum_s p[h,s] v[s,h,m]
  *   q, out: [heads, 128]; k, v: [seq_len, heads, 128] (dense).  When pos_dev != NULL
- *   the length is *pos_dev + 1 and seq_len is ignored. */
+ *   the length is *pos_dev + 1 and seq_len is the number of rows k and v have: a length
+ *   beyond it reads nothing and returns NaN. */
 int art_rmsnorm(const void* x_dev, const void* vsum_dev, const void* w_dev, void* out_dev, int rows, int n, float inv_n,
                 float eps, int x_dtype, int w_dtype, int out_dtype, void* stream);
 int art_rotary(const void* x_dev, const void* freq_dev, void* out_dev, int heads, int head_dim, int interleaved,
-               const void* pos_dev, int pos, long long out_row_stride, int x_dtype, int freq_dtype, int out_dtype,
-               void* stream);
+               const void* pos_dev, int pos, long long out_row_stride, int out_rows, int x_dtype, int freq_dtype,
+               int out_dtype, void* stream);
 /* One token's q | k | v (3 * heads * head_dim values): q rotated into q_out, k rotated into row
- * *pos_dev of key_cache, v copied into row *pos_dev of val_cache (caches: [positions, heads*head_dim]).
- * One launch for lines :155-158 and the v part of :151-152 of samples/05_llama2_7b_int4.py. */
+ * *pos_dev of key_cache, v copied into row *pos_dev of val_cache (caches: [max_positions, heads*head_dim];
+ * a position outside 0..max_positions-1 writes nothing).  One launch for lines :155-158 and the v part of :151-152 of samples/05_llama2_7b_int4.py. */
 int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, void* q_out_dev, void* key_cache_dev, void* val_cache_dev,
-                       int heads, int head_dim, const void* pos_dev, int dtype, int freq_dtype, void* stream);
+                       int heads, int head_dim, const void* pos_dev, int max_positions, int dtype, int freq_dtype,
+                       void* stream);
 /* art_rope_qkv_store and art_decode_attention in one launch (fp16): block h rotates its head's q and k,
- * writes k and v into cache row *pos_dev and attends over rows 0..*pos_dev. */
+ * writes k and v into cache row *pos_dev and attends over rows 0..*pos_dev.  The caches have max_positions rows:
+ * a position outside 0..max_positions-1 (a recorded graph replayed once too often) touches no cache row and
+ * returns NaN. */
 int art_decode_attention_rope(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev, void* val_cache_dev,
-                              const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev, void* stream);
+                              const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev,
+                              int max_positions, void* stream);
 /* art_decode_attention_rope spread over `parts` blocks per head (1..8), each attending over a contiguous share of
  * the cached positions.  With parts == 1 out_dev receives the fp16 result as above.  With parts > 1 out_dev is a
  * float buffer [heads][parts][132] that receives, per (head, part), 128 unnormalised sums, the running maximum and
@@ -192,7 +198,7 @@ int art_decode_attention_rope(const void* qkv_dev, const void* inv_freq_dev, voi
  * attention (samples/05_llama2_7b_int4.py:165-168) needs no extra launch. */
 int art_decode_attention_rope_split(const void* qkv_dev, const void* inv_freq_dev, void* key_cache_dev, void* val_cache_dev,
                                     const void* att_f_dev, void* out_dev, int heads, int head_dim, const void* pos_dev,
-                                    int parts, void* stream);
+                                    int max_positions, int parts, void* stream);
 /* y = fp16(product of the merged attention output with the int4 matrix) [+ residual]; partial_dev as written by
  * art_decode_attention_rope_split with the same `parts` (2..8), K = heads * 128. */
 int art_gemv_w4a16_attn(const void* partial_dev, int parts, const void* qweight_dev, const void* scales_dev,

@@ -200,3 +200,40 @@ def test_split_attention_merged_by_the_projection(parts, pos):
     merged = (acc * wgt[:, :, None]).sum(1) / (sm * wgt).sum(1)[:, None]
     assert torch.allclose(merged.float(), att.float(), rtol=2e-3, atol=2e-3)
     assert torch.allclose(y2.float(), y1.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_position_past_the_cache_touches_nothing(autort):
+    """A position read on the device that lies past the last cache row (a recorded graph replayed once too often)
+    must not run off the allocation: the cache-writing operators write nothing, the attention returns NaN."""
+    note('device-side position == rows of the cache')
+    dev = autort.device()
+    H, D, ROWS = 4, 128, 6
+    g = torch.Generator().manual_seed(3)
+    backing_k = torch.randn(ROWS + 2, H * D, generator=g).half().to(dev)     # two guard rows behind the cache
+    backing_v = torch.randn(ROWS + 2, H * D, generator=g).half().to(dev)
+    key_cache, val_cache = backing_k[:ROWS], backing_v[:ROWS]
+    before_k, before_v = backing_k.clone(), backing_v.clone()
+    qkv = torch.randn(3 * H * D, generator=g).half().to(dev)
+    inv = torch.rand(D, generator=g).half().to(dev)
+    att_f = torch.tensor([0.1], dtype=torch.float32, device=dev)
+    pos = torch.tensor([ROWS], dtype=torch.int32, device=dev)
+
+    out = torch.zeros(H, D, dtype=torch.float16, device=dev)
+    autort.ops.attention_rope_f16(qkv, inv, key_cache, val_cache, att_f, out, extra=[pos])
+    assert torch.isnan(out).all()
+    partial = torch.zeros(H, 4, 132, dtype=torch.float32, device=dev)
+    autort.ops.attention_rope_split_f16(qkv, inv, key_cache, val_cache, att_f, partial, extra=[pos])
+    assert torch.isnan(partial[:, :, :128]).all() and torch.isnan(partial[:, :, 129]).all()
+    q_out = torch.zeros(H, D, dtype=torch.float16, device=dev)
+    autort.ops.rope_qkv_store_f16(qkv, inv, q_out, key_cache, val_cache, extra=[pos])
+    autort.ops.rotary_f16(qkv[:H * D].view(H, 2, -1), inv, key_cache, extra=[pos])
+    out2 = torch.zeros(H, D, dtype=torch.float16, device=dev)
+    autort.ops.attention_f16(q_out, key_cache.view(ROWS, H, D), val_cache.view(ROWS, H, D), att_f, out2, extra=[pos])
+    assert torch.isnan(out2).all()
+    torch.cuda.synchronize()
+    assert torch.equal(backing_k, before_k) and torch.equal(backing_v, before_v)
+    # the last valid position still works
+    pos.fill_(ROWS - 1)
+    autort.ops.attention_rope_f16(qkv, inv, key_cache, val_cache, att_f, out, extra=[pos])
+    assert torch.isfinite(out).all()
+    assert torch.equal(backing_k[ROWS:], before_k[ROWS:]) and torch.equal(backing_v[ROWS:], before_v[ROWS:])
