@@ -538,7 +538,8 @@ __global__ __launch_bounds__(kGreedyThreads) void greedy_next_kernel(const _Floa
     for (int w = 1; w < kGreedyThreads / 64; ++w)
       if (s_val[w] > b || (s_val[w] == b && s_idx[w] < bi)) { b = s_val[w]; bi = s_idx[w]; }
     if (bi == 0x7fffffff) bi = 0;                 // every logit was NaN or -inf
-    const int t = (next_pos < prompt_len) ? prompt[next_pos] : bi;
+    int t = (next_pos < prompt_len) ? prompt[next_pos] : bi;
+    t = t < 0 ? 0 : (t >= vocab ? vocab - 1 : t);            // a prompt id outside the vocabulary must not index past the table
     s_token = t;
     *token = t;
     *pos = next_pos;
