@@ -121,7 +121,7 @@ def _gemm_f16_handler(op, bound, env, stream) -> bool:
     a, b, c = bound['a'], bound['b'], bound['c']
     M, K = a.shape
     N = b.shape[1]
-    if M % 256 or N % 256 or K % 64 or a.data_ptr() % 16 or b.data_ptr() % 16 or c.data_ptr() % 16:
+    if N % 8 or K % 64 or a.data_ptr() % 16 or b.data_ptr() % 16 or c.data_ptr() % 16:
         return False
     capi.check(capi.lib().art_gemm_f16(c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()), M, N, K,
                                       c_void_p(stream)))

@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int MT = M / BM, NT = N / BN;
+  const int MT = (M + BM - 1) / BM, NT = (N + BN - 1) / BN;      // edge tiles are clamped on the way in and cut on the way out
   int tile = xcd_tile(blockIdx.x, gridDim.x), tm, tn;
   if ((MT % 4 == 0) && (NT % 8 == 0)) {   // 4 x 8 super-tiles, row-major inside and outside
     const int super = tile >> 5, in = tile & 31, sn_count = NT >> 3;
@@ -69,8 +69,6 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
     tm = tile / NT;
     tn = tile % NT;
   }
-  const _Float16* Ag = A + (size_t)tm * BM * K;
-  const _Float16* Bg = B + (size_t)tn * BN;
 
   // global -> register staging: 4 chunks of 16 bytes per thread for each operand and stage.  The
   // per-thread part of every address is computed once; a tile only adds a wave-uniform offset.
@@ -80,8 +78,10 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int c = tid + 256 * i;
-    pa[i] = Ag + (size_t)(c >> 2) * K + (c & 3) * 8;
-    pb[i] = Bg + (size_t)(c >> 5) * N + (c & 31) * 8;
+    // rows past M and columns past N repeat the last valid ones: their products are never stored
+    const int arow = tm * BM + (c >> 2), bcol = tn * BN + (c & 31) * 8;
+    pa[i] = A + (size_t)(arow < M ? arow : M - 1) * K + (c & 3) * 8;
+    pb[i] = B + (size_t)(c >> 5) * N + (bcol < N ? bcol : N - 8);
   }
   const size_t b_step = (size_t)BK * N;
   auto load_tiles = [&](int kt, auto tag) {
@@ -207,12 +207,13 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
         cs[row * C_LD + col] = (_Float16)acc[i][j][r];
       }
   __syncthreads();
-  _Float16* Cg = C + (size_t)tm * BM * N + (size_t)tn * BN;
 #pragma unroll
   for (int i = 0; i < 32; ++i) {
     const int c = tid + 256 * i;               // 256 rows x 32 chunks of 8 halves
     const int row = c >> 5, ch = c & 31;
-    *reinterpret_cast<u32x4*>(Cg + (size_t)row * N + ch * 8) = *reinterpret_cast<const u32x4*>(cs + row * C_LD + ch * 8);
+    const int grow = tm * BM + row, gcol = tn * BN + ch * 8;
+    if (grow < M && gcol < N)
+      *reinterpret_cast<u32x4*>(C + (size_t)grow * N + gcol) = *reinterpret_cast<const u32x4*>(cs + row * C_LD + ch * 8);
   }
 }
 
@@ -220,8 +221,8 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
 
 extern "C" int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream) {
   ART_REQUIRE(a_dev && b_dev && c_dev, "art_gemm_f16: null pointer");
-  ART_REQUIRE(M > 0 && N > 0 && K > 0 && M % BM == 0 && N % BN == 0 && K % 64 == 0,
-              "art_gemm_f16: M and N must be multiples of 256 and K of 64 (M=%d N=%d K=%d)", M, N, K);
+  ART_REQUIRE(M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 64 == 0,
+              "art_gemm_f16: N must be a multiple of 8 and K of 64 (M=%d N=%d K=%d)", M, N, K);
   ART_REQUIRE(((uintptr_t)a_dev % 16) == 0 && ((uintptr_t)b_dev % 16) == 0 && ((uintptr_t)c_dev % 16) == 0,
               "art_gemm_f16: operands must be 16-byte aligned");
   static bool configured = false;
@@ -230,7 +231,7 @@ extern "C" int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, i
                                 (int)kLdsBytes));
     configured = true;
   }
-  const int blocks = (M / BM) * (N / BN);
+  const int blocks = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   gemm_f16_kernel<<<dim3(blocks), dim3(256), kLdsBytes, (hipStream_t)stream>>>((const _Float16*)a_dev, (const _Float16*)b_dev,
                                                                                 (_Float16*)c_dev, M, N, K);
   ART_LAUNCH_CHECK();

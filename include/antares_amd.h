@@ -137,7 +137,7 @@ int art_gemv_gptq(const void* x_dev, const void* qweight_dev, const void* scales
                   int K, int N, int x_f16, int scales_f16, void* stream);
 
 /* fp16 GEMM on the matrix cores: C[M,N] = A[M,K] @ B[K,N], all row-major, fp32
- * accumulation, fp16 output.  M % 256 == 0, N % 256 == 0, K % 64 == 0.
+ * accumulation, fp16 output.  Any M; N % 8 == 0, K % 64 == 0 (tiles of 256 x 256; edge tiles are clamped).
  * Replaces the kernel the reference generates for `C[N,M] +=! A[N,K] * B[K,M]`
  * (AntaresIR.md:115; tiled schedule backends/c-rocm/schedule/standard/algo_tiling.py:35-98). */
 int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream);

@@ -36,7 +36,9 @@ def test_small_against_loop_nest_oracle(gemm):
     assert np.allclose(got.astype(np.float32), want.astype(np.float32), **FP16_TOL)
 
 
-@pytest.mark.parametrize('M,N,K', [(256, 256, 64), (256, 512, 128), (512, 256, 192), (1024, 2048, 1024), (4096, 4096, 4096)])
+@pytest.mark.parametrize('M,N,K', [(256, 256, 64), (256, 512, 128), (512, 256, 192), (1024, 2048, 1024), (4096, 4096, 4096),
+                                   # edge tiles: any M, N % 8 == 0
+                                   (1, 256, 64), (100, 264, 128), (257, 248, 64), (300, 1000, 192), (64, 4096, 4096), (777, 8, 64)])
 def test_against_float64_product(gemm, M, N, K):
     autort, op = gemm
     print(f'[case] gemm {M}x{N}x{K}', flush=True)
@@ -57,7 +59,8 @@ def test_against_float64_product(gemm, M, N, K):
         assert torch.equal(f(bb.to(dev), eye.to(dev)).cpu(), bb)
 
 
-def test_shapes_outside_the_tile_grid_use_the_generic_lowering(gemm):
+def test_shapes_the_kernel_does_not_take_use_the_generic_lowering(gemm):
+    """K % 64 != 0 (or N % 8 != 0) is left to the generic reduce lowering."""
     autort, op = gemm
     print('[case] gemm 96x80x40 (generic lowering)', flush=True)
     g = torch.Generator().manual_seed(5)
