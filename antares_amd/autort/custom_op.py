@@ -10,21 +10,26 @@ the kernels and fills ``output_infos`` / ``output_names`` / ``kernel_sources``;
 calling the module takes the inputs in ``input_orders`` order, allocates the
 outputs and returns one tensor or a tuple.  Where the reference shells out to
 the ``antares`` service and a pybind module (main_ops.cc:17-54), this one lowers
-in-process and launches through the C ABI.
+in-process and launches through the C ABI.  ``kernel_sources`` is the kernel
+container the reference would have received from the service, and ``custom_key``
+the number ``inject`` gave it: ``forward(op.custom_key, inputs + outputs)`` of
+``antares_amd.autort.execution_module`` runs that container as the pybind module
+does; calling the operator itself takes the faster route through ``autort.export``
+(hand-written kernels where the program is a known pattern).
 """
 from __future__ import annotations
 
-import itertools
 from typing import Dict, List, Sequence, Tuple, Union
 
 import torch
 
+from ..lower.evaluator_emit import emit_evaluator_module
+from .execution_module import inject
 from .op import ExportedOp
 
 _DTYPE_NAME = {torch.float64: 'float64', torch.float32: 'float32', torch.float16: 'float16', torch.int64: 'int64',
                torch.int32: 'int32', torch.int16: 'int16', torch.int8: 'int8', torch.uint8: 'uint8'}
 _DTYPE_TORCH = {v: k for k, v in _DTYPE_NAME.items()}
-_keys = itertools.count(1)
 
 
 class CustomOp(torch.nn.Module):
@@ -67,8 +72,8 @@ class CustomOp(torch.nn.Module):
         env = g.bind_dims({})
         self.output_infos = [(n, _DTYPE_TORCH[g.tensors[n].dtype], [int(d) for d in g.shape_of(n, env)]) for n in g.outputs]
         self.output_names = [x[0] for x in self.output_infos]
-        self.kernel_sources = op.source
-        self.custom_key = next(_keys)
+        self.kernel_sources = emit_evaluator_module(op.fused)
+        self.custom_key = inject(self.kernel_sources)
         self._op = op
         return self
 
