@@ -142,6 +142,19 @@ int art_module_load(const void* image, size_t size, art_module** out) {
   return 0;
 }
 
+int art_module_load_file(const char* path, art_module** out) {
+  ART_REQUIRE(path && out, "art_module_load_file: null argument");
+  FILE* f = fopen(path, "rb");
+  if (!f) return art::fail("art_module_load_file: cannot open %s", path);
+  std::vector<char> image;
+  char buf[65536];
+  size_t n;
+  while ((n = fread(buf, 1, sizeof(buf), f)) > 0) image.insert(image.end(), buf, buf + n);
+  fclose(f);
+  ART_REQUIRE(!image.empty(), "art_module_load_file: %s is empty", path);
+  return art_module_load(image.data(), image.size(), out);
+}
+
 int art_module_unload(art_module* module) {
   ART_REQUIRE(module != nullptr, "art_module_unload: null module");
   ART_HIP(hipModuleUnload(module->handle));

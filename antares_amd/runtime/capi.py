@@ -34,6 +34,7 @@ _SIGNATURES = {
     'art_module_compile': (c_int, [c_char_p, c_char_p, POINTER(c_void_p), POINTER(c_size_t)]),
     'art_blob_free': (None, [c_void_p]),
     'art_module_load': (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
+    'art_module_load_file': (c_int, [c_char_p, POINTER(c_void_p)]),
     'art_module_unload': (c_int, [c_void_p]),
     'art_get_function': (c_int, [c_void_p, c_char_p, POINTER(c_void_p)]),
     'art_launch': (c_int, [c_void_p, c_uint, c_uint, c_uint, c_uint, c_uint, c_uint, c_uint, c_void_p,

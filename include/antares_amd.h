@@ -65,6 +65,8 @@ const char* art_compile_log(void);
 
 /* Load a code object; replaces ab::moduleLoad (backend.hpp:161-170). */
 int art_module_load(const void* image, size_t size, art_module** out);
+/* The same from a code-object file (what `hipcc --genco` or art_module_compile wrote). */
+int art_module_load_file(const char* path, art_module** out);
 int art_module_unload(art_module* module);
 
 /* Look a kernel up by name; replaces ab::moduleGetFunction (backend.hpp:172-197). */

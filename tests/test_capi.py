@@ -48,6 +48,11 @@ def test_bad_arguments_return_errors(lib):
     assert l.art_gemv_w4a16(None, None, None, None, None, 1, 4096, 4096, None) != 0
     assert b'null pointer' in l.art_last_error()
     assert l.art_module_load(None, 0, None) != 0
+    assert l.art_module_load_file(b'/nonexistent/kernel.hsaco', None) != 0
+    import ctypes
+    h = ctypes.c_void_p()
+    assert l.art_module_load_file(b'/nonexistent/kernel.hsaco', ctypes.byref(h)) != 0
+    assert b'cannot open' in l.art_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch, lib):

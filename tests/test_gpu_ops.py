@@ -258,3 +258,21 @@ def test_generic_matmul_and_scatter(autort):
     h(hist, idx.to(dev), upd.to(dev))
     want = torch.zeros(16, dtype=torch.int64).index_add_(0, idx.long(), upd.long())
     assert hist.cpu().long().tolist() == want.tolist()
+
+
+def test_code_object_file_loads_and_runs(autort, tmp_path):
+    """art_module_load_file: a code object written to disk (what `hipcc --genco` leaves) is loaded and launched."""
+    import ctypes
+    from antares_amd.runtime import capi
+    note('art_module_load_file')
+    capi.init(0)
+    image = capi.compile_hip('extern "C" __global__ void twice(float* a, int n) { int i = blockIdx.x * 64 + threadIdx.x; if (i < n) a[i] *= 2.f; }')
+    path = tmp_path / 'twice.hsaco'
+    path.write_bytes(image)
+    h, f = ctypes.c_void_p(), ctypes.c_void_p()
+    capi.check(capi.lib().art_module_load_file(str(path).encode(), ctypes.byref(h)))
+    capi.check(capi.lib().art_get_function(h, b'twice', ctypes.byref(f)))
+    a = torch.arange(100, dtype=torch.float32, device=autort.device())
+    capi.launch(f, (2, 1, 1), (64, 1, 1), torch.cuda.current_stream().cuda_stream, [a.data_ptr(), 100])
+    torch.cuda.synchronize()
+    assert torch.equal(a.cpu(), torch.arange(100, dtype=torch.float32) * 2)
