@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kThreads) void gemv_gptq_kernel(const XT* __restric
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int r = r0 + i < wrows ? r0 + i : wrows - 1;    // past the end: any valid row, x is zero there
-    w[i] = *reinterpret_cast<const u32x4*>(qweight + (size_t)r * N + n0c);
+    w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(qweight + (size_t)r * N + n0c));   // streamed once
   }
   // column owners fetch the scales of their column for the eight groups of the block
   const int col = tile * CT + tid;
