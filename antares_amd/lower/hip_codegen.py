@@ -294,9 +294,14 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
                     body.append(f'  typedef {HIP_TYPE[tensors[n].dtype]} __vec_{n} __attribute__((ext_vector_type({V})));')
                 body.append(f'  const long long __nvec = __total / {V};')
                 body.append('  for (long long __v = __tid; __v < __nvec; __v += __nthr) {')
+                # a tensor no other statement of the program touches is streamed: non-temporal accesses measured
+                # 4520 against 4110 GB/s on the 4 096 000-element sigmoid
+                def streamed(n):
+                    return sum(1 for s_ in graph.statements if n in s_.reads or n == s_.output) == 1
                 for n in names:
                     if n != st.output or n in reads:
-                        body.append(f'    const __vec_{n} __in_{n} = ((const __vec_{n}*){n})[__v];')
+                        src_ = f'((const __vec_{n}*){n})[__v]'
+                        body.append(f'    const __vec_{n} __in_{n} = ' + (f'__builtin_nontemporal_load(&{src_});' if streamed(n) else f'{src_};'))
                 body.append(f'    __vec_{st.output} __out;')
                 vem = ExprEmitter(tensors, load_override=lambda n: f'__in_{n.name}[__e]')
                 body.append('    #pragma unroll')
@@ -305,7 +310,8 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
                     body.append(f'      const int {st.data_axes[0][0]} = (int)(__v * {V} + __e); (void){st.data_axes[0][0]};')
                 body.append(f'      __out[__e] = ({oct_})({vem.expr(root)});')
                 body.append('    }')
-                body.append(f'    ((__vec_{st.output}*){st.output})[__v] = __out;')
+                dst_ = f'((__vec_{st.output}*){st.output})[__v]'
+                body.append(f'    __builtin_nontemporal_store(__out, &{dst_});' if streamed(st.output) else f'    {dst_} = __out;')
                 body.append('  }')
                 body.append(f'  for (long long __i = __nvec * {V} + __tid; __i < __total; __i += __nthr) {{')
                 body += _decompose('__i', st.data_axes, '    ')
