@@ -14,7 +14,7 @@
 //            total; then, tile by tile, it ranks the even values with a
 //            wavefront prefix + a 4-wave prefix through LDS, compacts evens
 //            and odds of the tile in LDS and writes both runs with fully
-//            coalesced stores:
+//            coalesced 16-byte non-temporal stores:
 //              even -> out[evens_before + rank]
 //              odd  -> out[total_even + odds_before + rank]
 //
@@ -37,9 +37,13 @@ __device__ __forceinline__ int even_count4(i32x4 v) {
 }
 
 // Loads vector `j` of this thread (elements 4*(j*256+tid) .. +3 of the tile); elements past n read as odd (1).
+template <bool LAST_USE = false>
 __device__ __forceinline__ i32x4 load_vec(const int* __restrict__ in, long long base, int j, long long n) {
   const long long e0 = base + 4LL * (j * kThreads + threadIdx.x);
-  if (e0 + 3 < n) return *reinterpret_cast<const i32x4*>(in + e0);
+  if (e0 + 3 < n) {
+    if (LAST_USE) return __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(in + e0));   // the scatter pass is the last reader
+    return *reinterpret_cast<const i32x4*>(in + e0);
+  }
   i32x4 v = {1, 1, 1, 1};
   if (e0 + 0 < n) v.x = in[e0 + 0];
   if (e0 + 1 < n) v.y = in[e0 + 1];
@@ -83,7 +87,7 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
   const long long span_base = (long long)b * tiles_per_block * kTile;
   i32x4 v[kVecPerThread];
 #pragma unroll
-  for (int j = 0; j < kVecPerThread; ++j) v[j] = load_vec(in, span_base, j, n);
+  for (int j = 0; j < kVecPerThread; ++j) v[j] = load_vec<true>(in, span_base, j, n);
 
   // evens before this block and in total (64-bit: n may exceed 2^31 / 2)
   unsigned long long before_sum = 0, total_sum = 0;
@@ -110,7 +114,7 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
     const bool more = (s + 1 < tiles_per_block) && (base + kTile < n);
     if (more) {
 #pragma unroll
-      for (int j = 0; j < kVecPerThread; ++j) vn[j] = load_vec(in, base + kTile, j, n);
+      for (int j = 0; j < kVecPerThread; ++j) vn[j] = load_vec<true>(in, base + kTile, j, n);
     }
     const long long valid = (n - base < kTile) ? (n - base) : kTile;      // elements of this tile that exist
     unsigned int cnt[kVecPerThread], incl[kVecPerThread];
@@ -157,8 +161,22 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
     art_lds_barrier();
     const long long odd_base = total_even + (base - even_before);
     const unsigned int tile_odd = (unsigned int)valid - tile_even;     // padding was counted as odd and sits last
-    for (unsigned int i = tid; i < tile_even; i += kThreads) out[even_before + i] = s_items[i];
-    for (unsigned int i = tid; i < tile_odd; i += kThreads) out[odd_base + i] = s_items[tile_even + i];
+    // Both runs leave as 16-byte non-temporal stores (written once, read by nobody here): up to three elements
+    // bring the destination to a 16-byte boundary, whole vectors follow, up to three elements finish the run.
+    auto flush_run = [&](long long dst0, unsigned int src0, unsigned int count) {
+      const unsigned int to_boundary = (4u - (unsigned int)((reinterpret_cast<uintptr_t>(out + dst0) >> 2) & 3)) & 3u;
+      const unsigned int head = to_boundary < count ? to_boundary : count;
+      const unsigned int vecs = (count - head) >> 2, tail = (count - head) & 3;
+      if (tid < head) __builtin_nontemporal_store(s_items[src0 + tid], &out[dst0 + tid]);
+      for (unsigned int q = tid; q < vecs; q += kThreads) {
+        const unsigned int s = src0 + head + 4 * q;
+        const i32x4 pack = {s_items[s], s_items[s + 1], s_items[s + 2], s_items[s + 3]};
+        __builtin_nontemporal_store(pack, reinterpret_cast<i32x4*>(out + dst0 + head + 4 * (long long)q));
+      }
+      if (tid < tail) __builtin_nontemporal_store(s_items[src0 + head + 4 * vecs + tid], &out[dst0 + head + 4 * (long long)vecs + tid]);
+    };
+    flush_run(even_before, 0, tile_even);
+    flush_run(odd_base, tile_even, tile_odd);
     even_before += tile_even;
     if (more) {
 #pragma unroll
@@ -175,6 +193,7 @@ extern "C" int art_partition_even_first_i32(const void* in_dev, void* out_dev, l
   if (n == 0) return 0;
   ART_REQUIRE(in_dev && out_dev && in_dev != out_dev, "art_partition_even_first_i32: null or aliased pointers");
   ART_REQUIRE(((uintptr_t)in_dev % 16) == 0, "art_partition_even_first_i32: input must be 16-byte aligned");
+  ART_REQUIRE(((uintptr_t)out_dev % 4) == 0, "art_partition_even_first_i32: output must be 4-byte aligned");
   art::Workspace& ws = art::workspace();
   ART_REQUIRE(ws.base != nullptr, "art_partition_even_first_i32: call art_init first");
   const long long tiles = (n + kTile - 1) / kTile;

@@ -102,6 +102,16 @@ def test_partition_empty_and_degenerate(autort):
     ev = torch.arange(0, 20000, 2, dtype=torch.int32, device=dev)
     assert torch.equal(autort.ops.partition_even_first_i32(ev), ev)
     assert torch.equal(autort.ops.partition_even_first_i32(ev + 1), ev + 1)
+    # the output may start anywhere on a 4-byte boundary (its 16-byte stores find their own alignment) and nothing
+    # outside it is written
+    for shift in (1, 2, 3):
+        x = workloads.partition_input(shift, 10_007).to(dev)
+        backing = torch.full((10_007 + 8,), -7, dtype=torch.int32, device=dev)
+        out = backing[shift:shift + 10_007]
+        autort.ops.partition_even_first_i32(x, out)
+        xc = x.cpu()
+        assert torch.equal(out.cpu(), torch.cat([xc[xc % 2 == 0], xc[xc % 2 == 1]]))
+        assert (backing[:shift] == -7).all() and (backing[shift + 10_007:] == -7).all()
 
 
 def test_partition_full_size_properties(autort):
