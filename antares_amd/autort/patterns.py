@@ -95,8 +95,9 @@ def _w4a16_handler(op, bound, env, stream) -> bool:
     if K % 128 or N % 16 or q.shape[0] * 2 != K or s.shape[0] * 128 != K or z.shape[1] * 2 != N \
             or q.data_ptr() % 16 or x.data_ptr() % 16 or z.data_ptr() % 8 or y.data_ptr() % 8:
         return False
-    # the vector-unit kernel streams the weights once per pair of rows (7.6 / 10.7 / 16.1 / 19.5 us for 1..4 rows
-    # of 4096 x 11008), the matrix-core kernel once per 64 rows (16 us for 8 rows): four rows and more go there
+    # the vector-unit kernel streams the weights once per four rows (7.5 / 11.1 / 13.0 / 15.3 us for 1..4 rows of
+    # 4096 x 11008, 22 us for five), the matrix-core kernel once per 64 rows (16 us for 4..32 rows): four rows and
+    # more go there
     entry = capi.lib().art_gemv_w4a16 if M <= 3 else capi.lib().art_gemm_w4a16
     capi.check(entry(c_void_p(x.data_ptr()), c_void_p(q.data_ptr()), c_void_p(s.data_ptr()),
                                         c_void_p(z.data_ptr()), c_void_p(y.data_ptr()), M, K, N, c_void_p(stream)))

@@ -401,11 +401,13 @@ extern "C" int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const 
   ART_REQUIRE(M >= 1 && M <= 8, "art_gemv_w4a16: M must be in 1..8 (got %d); larger batches go through art_gemm_w4a16", M);
   hipStream_t st = (hipStream_t)stream;
   int m = 0;
-  while (m < M) {       // rows of x are handled two or one at a time
-    const int step = (M - m >= 2) ? 2 : 1;
+  while (m < M) {       // rows of x are handled up to four at a time
+    const int step = (M - m >= 4) ? 4 : (M - m);
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m * N;
-    int rc = step == 2 ? launch<2>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st)
+    int rc = step == 4 ? launch<4>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st)
+           : step == 3 ? launch<3>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st)
+           : step == 2 ? launch<2>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st)
                        : launch<1>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st);
     if (rc) return rc;
     m += step;
