@@ -72,7 +72,7 @@ class CustomOp(torch.nn.Module):
         env = g.bind_dims({})
         self.output_infos = [(n, _DTYPE_TORCH[g.tensors[n].dtype], [int(d) for d in g.shape_of(n, env)]) for n in g.outputs]
         self.output_names = [x[0] for x in self.output_infos]
-        self.kernel_sources = emit_evaluator_module(op.fused)
+        self.kernel_sources = emit_evaluator_module(op.lowered)
         self.custom_key = inject(self.kernel_sources)
         self._op = op
         return self

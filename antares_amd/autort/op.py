@@ -18,7 +18,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..ir import Graph, fuse_elementwise, parse_program
+from ..ir import Graph, fuse_elementwise, parse_program, split_wide_reductions
 from ..lower import lower_graph
 from ..runtime import capi
 
@@ -82,7 +82,11 @@ class ExportedOp:
         self.inout = list(self.graph.inout)
         # outputs the caller does not pass among the declared tensors
         self.fresh_outputs = [o for o in self.graph.outputs if o not in self.declared]
-        self.source, self.plans = lower_graph(self.fused, prefix='autort_' + _ident(self.name))
+        # what the generic lowering compiles: wide reductions with few outputs become two statements (statically
+        # sized ones here; programs with named dimensions get a variant per set of values at call time)
+        self.lowered: Graph = split_wide_reductions(self.fused)
+        self.source, self.plans = lower_graph(self.lowered, prefix='autort_' + _ident(self.name))
+        self._variants: Dict[tuple, dict] = {}
         self._module: Optional[capi.Module] = None
         self._image: Optional[bytes] = None
         from . import patterns
@@ -177,13 +181,31 @@ class ExportedOp:
         if not t.is_contiguous():
             raise ValueError(f'tensor `{name}` must be contiguous (views are fine if they are dense)')
 
+    def _variant(self, env: Dict[str, int]) -> dict:
+        """Graph, plans and module for these values of the named dimensions: the default ones, unless a reduction
+        of the program is worth slicing at these sizes (split_wide_reductions), which needs its own kernels."""
+        key = tuple(env[d] for d in self.fused.dim_names)
+        v = self._variants.get(key)
+        if v is None:
+            g = split_wide_reductions(self.lowered, env) if self.fused.dims else self.lowered
+            if g is self.lowered:
+                v = {'graph': self.lowered, 'plans': self.plans, 'module': None, 'source': None}
+            else:
+                source, plans = lower_graph(g, prefix='autort_' + _ident(self.name) + '_s' + '_'.join(str(k) for k in key))
+                v = {'graph': g, 'plans': plans, 'module': None, 'source': source}
+            if len(self._variants) < 64:
+                self._variants[key] = v
+        if v['module'] is None:
+            v['module'] = self._load() if v['source'] is None else capi.Module(compile_cached(v['source']))
+        return v
+
     def _run_generic(self, bound: Dict[str, torch.Tensor], env: Dict[str, int], dev, stream: int):
-        module = self._load()
-        g = self.fused
+        variant = self._variant(env)
+        module, g, plans_ = variant['module'], variant['graph'], variant['plans']
         dims = [env[d] for d in g.dim_names]
         trials = self.config.get('tune')
         trials = trials if isinstance(trials, int) and trials > 0 else 0
-        for plan in self.plans:
+        for plan in plans_:
             for n in plan.args:
                 if n not in bound:         # intermediate (reduce result) of a multi-kernel program
                     bound[n] = torch.empty(g.shape_of(n, env), dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)

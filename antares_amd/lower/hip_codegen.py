@@ -255,7 +255,24 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
     reads = [r for r in st.reads]
     args = sorted(set(reads) - {st.output}) + [st.output]
     written = [st.output]
-    em = ExprEmitter(tensors)
+
+    def one_touch(n: Expr) -> Optional[str]:
+        """A load that reads every element of its tensor exactly once in the whole program - indexed by all axes of
+        the statement, each once, and no other statement or load touches the tensor - carries the non-temporal
+        hint (an evict-first stream: measured +10 % on the 4 096 000-element sigmoid)."""
+        axes = [ax for ax, _ in st.data_axes + st.reduce_axes]
+        if n.name == st.output or any(a.kind != 'axis' for a in n.args):
+            return None
+        if sorted(a.name for a in n.args) != sorted(axes):
+            return None
+        if sum(1 for s_ in graph.statements if n.name in s_.reads or n.name == s_.output) != 1:
+            return None
+        if sum(1 for m in walk(st.root) if m.kind == 'load' and m.name == n.name) != 1:
+            return None
+        return f'__builtin_nontemporal_load(&{n.name}[{plain.offset(n.name, [plain.expr(a) for a in n.args])}])'
+
+    plain = ExprEmitter(tensors)
+    em = ExprEmitter(tensors, load_override=one_touch)
     total = ' * '.join(f'(long long)__ext_{ax}' for ax, _ in st.data_axes) or '1LL'
     oct_ = HIP_TYPE[st.out_dtype]
     src: List[str] = []
@@ -350,6 +367,7 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
             b.append(f'  for (long long __o = {out_var}; __o < __total; __o += {out_step}) {{')
             b += _decompose('__o', st.data_axes, '    ')
             b.append(f'    {act} __acc = {ident};')
+            b.append('    #pragma unroll 4')
             b.append(f'    for (long long __k = {lane}; __k < __red; __k += {nlanes}) {{')
             b += [l.replace('__r', '__q') for l in _decompose('__k', st.reduce_axes, '      ')]
             b.append(f'      __acc = {op}(__acc, ({act})({em.expr(root)}));')
@@ -377,11 +395,11 @@ def _reduce_axis_contiguous(st, tensors) -> Optional[bool]:
     score = 0
     for n in walk(st.root):
         if n.kind == 'load' and n.args:
-            last = n.args[-1]
+            names = {m.name for m in walk(n.args[-1]) if m.kind == 'axis'}     # `S * chunk + C` walks memory along C
             w = len(n.args)
-            if last.kind == 'axis' and last.name in raxes:
+            if names & raxes:
                 score += w
-            elif last.kind == 'axis' and last.name in daxes:
+            elif names & daxes:
                 score -= w
     if score == 0:
         return None

@@ -286,3 +286,41 @@ def test_code_object_file_loads_and_runs(autort, tmp_path):
     capi.launch(f, (2, 1, 1), (64, 1, 1), torch.cuda.current_stream().cuda_stream, [a.data_ptr(), 100])
     torch.cuda.synchronize()
     assert torch.equal(a.cpu(), torch.arange(100, dtype=torch.float32) * 2)
+
+
+@pytest.mark.parametrize('ir,inputs,shapes', [
+    ('output0[] +=! input0[N]', ['input0=float32[N:1048576]'], [(1048576,), (1000003,), (262144,)]),
+    ('output0[C] +=! input0[N, C]', ['input0=float32[N:2048, C:512]'], [(2048, 512), (4096, 96)]),
+    ('output0[N] >=! input0[N, C]', ['input0=float32[N:8, C:65536]'], [(8, 65536), (3, 40000)]),
+    ('output0[N] <=! input0[N, C]', ['input0=float32[8, 32768]'], [(8, 32768)]),
+    ('output0[N, M] +=! input0[N, K] * input1[K, M]', ['input0=float32[N:4, K:8192]', 'input1=float32[K:8192, M:16]'], [(4, 8192, 16)]),
+    ('output0[] +=! input0[N]', ['input0=int32[N:2097152]'], [(2097152,)]),
+])
+def test_wide_reductions_are_sliced_and_still_right(autort, ir, inputs, shapes):
+    """Reductions with too few outputs to fill the chip run as two statements (slices, then the slices); programs with
+    named dimensions get kernels per set of values, and sizes that do not divide fall back to the one-statement form."""
+    note(f'wide reduction {ir}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='wide_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    g = torch.Generator().manual_seed(11)
+    for shape in shapes:
+        if 'input1' in ir:
+            n, k, m = shape
+            a, b = torch.randn(n, k, generator=g), torch.randn(k, m, generator=g)
+            got = op(a.to(dev), b.to(dev)).cpu()
+            assert torch.allclose(got, (a.double() @ b.double()).float(), rtol=1e-4, atol=1e-3)
+            continue
+        if 'int32' in inputs[0]:
+            x = torch.randint(-1000, 1000, shape, generator=g, dtype=torch.int32)
+            assert int(op(x.to(dev)).cpu()) == int(x.sum())
+            continue
+        x = torch.randn(shape, generator=g)
+        got = op(x.to(dev)).cpu()
+        if '>=!' in ir:
+            assert torch.equal(got, x.max(dim=1).values)
+        elif '<=!' in ir:
+            assert torch.equal(got, x.min(dim=1).values)
+        elif ir.startswith('output0[C]'):
+            assert torch.allclose(got, x.double().sum(0).float(), rtol=1e-4, atol=1e-3)
+        else:
+            assert abs(float(got) - float(x.double().sum())) < 0.05
