@@ -133,6 +133,22 @@ class KernelPlan:
     vec: int = 1                   # elements per lane in the vector variant
     vec_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for it
     reduce_contiguous: Optional[bool] = None   # True: a reduce axis is fastest in the biggest operand
+    tile_axes: Optional[Tuple[str, str]] = None   # permutation copies: last axis of the load, last axis of the store
+
+    def _tiles(self, env: Dict[str, int]) -> int:
+        """64 x 64 tiles of the transposing variant, 0 when it does not apply or an axis is too short to pay."""
+        if self.tile_axes is None or 'tile' not in self.variants:
+            return 0
+        n = 1
+        for ax, e in self.data_axes:
+            v = e if isinstance(e, int) else env[e]
+            if ax in self.tile_axes:
+                if v < 16:
+                    return 0
+                n *= (v + 63) // 64
+            else:
+                n *= v
+        return n
 
     def choose(self, env: Dict[str, int], pointers: Dict[str, int]) -> Tuple[str, int, int]:
         """-> (kernel symbol, grid.x, block.x) for these extents and addresses."""
@@ -148,6 +164,9 @@ class KernelPlan:
             if 'vec' in self.variants and all(pointers[t] % 16 == 0 for t in self.vec_tensors) and total >= self.vec:
                 work = (total + self.vec - 1) // self.vec
                 return self.variants['vec'], min((work + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
+            tiles = self._tiles(env)
+            if tiles:
+                return self.variants['tile'], min(tiles, MAX_GRID), BLOCK
             return self.variants['scalar'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
         if self.kind == 'scatter':
             return self.variants['scalar'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
@@ -174,6 +193,8 @@ class KernelPlan:
         if self.kind == 'map':
             if 'vec' in self.variants and all(pointers[t] % 16 == 0 for t in self.vec_tensors) and total >= self.vec:
                 tags.append(('vec', (total + self.vec - 1) // self.vec))
+            if self._tiles(env):
+                tags.append(('tile', self._tiles(env) * BLOCK))
             tags.append(('scalar', total))
         elif self.kind == 'scatter':
             tags.append(('scalar', total))
@@ -221,6 +242,27 @@ def _root_and_cond(st, em: ExprEmitter):
         cond = rel.join(f'({em.expr(c)})' for c in root.conds)
         root = root.args[0]
     return root, cond
+
+
+def _transpose_axes(st, tensors):
+    """(A, B) when the statement is a permutation copy (possibly with elementwise work on top): one load, indexed
+    by all data axes, each once and bare, whose last axis A differs from the last axis B of the store.  Reading
+    walks memory along A, writing along B; a tile in LDS turns one into the other."""
+    axes = [a for a, _ in st.data_axes]
+    if st.scatter or st.reduce_axes or len(axes) < 2 or [i.name for i in st.out_index if i.kind == 'axis'] != axes:
+        return None
+    if st.root.kind == 'when' and len(st.root.args) == 1:
+        return None
+    loads = [n for n in walk(st.root) if n.kind == 'load']
+    if len(loads) != 1 or loads[0].name == st.output:
+        return None
+    idx = loads[0].args
+    if any(a.kind != 'axis' for a in idx) or sorted(a.name for a in idx) != sorted(axes):
+        return None
+    if sum(1 for n in walk(st.root) if n.kind == 'axis') != len(idx):       # a bare axis used as a value
+        return None
+    a_ax, b_ax = idx[-1].name, axes[-1]
+    return None if a_ax == b_ax else (a_ax, b_ax)
 
 
 def _is_flat_map(st, tensors) -> bool:
@@ -337,6 +379,35 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
                 src.append('\n'.join(body))
                 variants['vec'] = sym
                 plan.vec, plan.vec_tensors = V, names
+        tr = _transpose_axes(st, tensors)
+        if tr is not None:
+            a_ax, b_ax = tr
+            others = [(ax, e) for ax, e in st.data_axes if ax not in (a_ax, b_ax)]
+            sym = name + '_x'
+            body = [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st)
+            body += [f'  __shared__ {oct_} __tile[64][65];',
+                     '  const int __tx = threadIdx.x & 63, __ty = threadIdx.x >> 6;',
+                     f'  const long long __ta = ((long long)__ext_{a_ax} + 63) / 64, __tb = ((long long)__ext_{b_ax} + 63) / 64;',
+                     '  const long long __batch = ' + (' * '.join(f'(long long)__ext_{ax}' for ax, _ in others) or '1LL') + ';',
+                     '  for (long long __t = blockIdx.x; __t < __ta * __tb * __batch; __t += gridDim.x) {',
+                     '    const long long __ia = __t % __ta, __ib = (__t / __ta) % __tb;',
+                     '    long long __r = __t / (__ta * __tb); (void)__r;']
+            for ax, _ in reversed(others):
+                body.append(f'    const int {ax} = (int)(__r % __ext_{ax}); __r /= __ext_{ax};')
+            body += ['    for (int __row = __ty; __row < 64; __row += 4) {       // read along the input\'s last axis',
+                     f'      const int {a_ax} = (int)(__ia * 64 + __tx), {b_ax} = (int)(__ib * 64 + __row);',
+                     f'      if ({a_ax} < __ext_{a_ax} && {b_ax} < __ext_{b_ax}) __tile[__row][__tx] = ({oct_})({plain.expr(root)});',
+                     '    }',
+                     '    __syncthreads();',
+                     '    for (int __row = __ty; __row < 64; __row += 4) {       // write along the output\'s last axis',
+                     f'      const int {a_ax} = (int)(__ia * 64 + __row), {b_ax} = (int)(__ib * 64 + __tx);',
+                     f'      if ({a_ax} < __ext_{a_ax} && {b_ax} < __ext_{b_ax}) {dst} = __tile[__tx][__row];',
+                     '    }',
+                     '    __syncthreads();',
+                     '  }', '}']
+            src.append('\n'.join(body))
+            variants['tile'] = sym
+            plan.tile_axes = (a_ax, b_ax)
 
     elif plan.kind == 'scatter':
         sym = name

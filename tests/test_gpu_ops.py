@@ -324,3 +324,26 @@ def test_wide_reductions_are_sliced_and_still_right(autort, ir, inputs, shapes):
             assert torch.allclose(got, x.double().sum(0).float(), rtol=1e-4, atol=1e-3)
         else:
             assert abs(float(got) - float(x.double().sum())) < 0.05
+
+
+@pytest.mark.parametrize('ir,spec,shape,perm', [
+    ('output0[C, N] = input0[N, C]', 'input0=float32[N:1000, C:777]', (1000, 777), (1, 0)),
+    ('output0[N, H, W, C] = input0[N, C, H, W]', 'input0=float16[N:3, C:70, H:5, W:129]', (3, 70, 5, 129), (0, 2, 3, 1)),
+    ('output0[B, C, N] = input0[N, B, C] * 2', 'input0=float32[N:65, B:2, C:64]', (65, 2, 64), (1, 2, 0)),
+    ('output0[C, N] = input0[N, C]', 'input0=int32[N:16, C:4096]', (16, 4096), (1, 0)),
+])
+def test_permutation_copies_go_through_lds_tiles(autort, ir, spec, shape, perm):
+    """A copy whose store walks memory along another axis than its load is lowered to 64 x 64 tiles through LDS."""
+    note(f'tiled permutation {ir} {shape}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=[spec], name='perm_' + str(abs(hash((ir, spec))) % 10 ** 8))
+    assert 'tile' in op.plans[0].variants
+    g = torch.Generator().manual_seed(4)
+    if 'int32' in spec:
+        x = torch.randint(-10 ** 6, 10 ** 6, shape, generator=g, dtype=torch.int32)
+    else:
+        x = torch.randn(shape, generator=g).to(torch.float16 if 'float16' in spec else torch.float32)
+    want = x.permute(*perm).contiguous()
+    if '* 2' in ir:
+        want = want * 2
+    assert torch.equal(op(x.to(dev)).cpu(), want)
