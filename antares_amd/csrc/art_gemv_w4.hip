@@ -356,7 +356,7 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     const long long old = (long long)__hip_atomic_fetch_add(slot, (unsigned long long)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (((old + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
       const long long total = old + mine - ((long long)splits << 56);
- _Float16 o = (_Float16)((float)total * (1.f / kFix));
+      _Float16 o = (_Float16)((float)total * (1.f / kFix));
       if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)fused.residual[col]);
       y[(size_t)m * N + col] = o;
       *slot = 0ull;                     // ready for the next launch (stream order makes this visible)
