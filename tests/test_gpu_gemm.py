@@ -68,3 +68,27 @@ def test_shapes_the_kernel_does_not_take_use_the_generic_lowering(gemm):
     b = (torch.randn(40, 80, generator=g) * 0.1).half()
     got = op(a.to(autort.device()), b.to(autort.device())).cpu().numpy()
     assert np.allclose(got.astype(np.float32), oracle_gemm(a.numpy(), b.numpy()).astype(np.float32), **FP16_TOL)
+
+
+def test_8192_cubed_through_a_random_projection(gemm):
+    """The larger benchmark size, checked by a property that needs O(n^2) work on the host:
+    (A B) v = A (B v) for a random v, in float64 from the fp16 operands and the fp16 result."""
+    autort, op = gemm
+    n = 8192
+    print(f'[case] gemm {n}^3 projection', flush=True)
+    a, b = workloads.gemm_inputs(3, n)
+    dev = autort.device()
+    c = op(a.to(dev), b.to(dev)).cpu()
+    g = torch.Generator().manual_seed(9)
+    for _ in range(2):
+        v = torch.randn(n, generator=g, dtype=torch.float64)
+        want = a.double() @ (b.double() @ v)
+        got = c.double() @ v
+        # every element of C carries a relative rounding error of 2^-11; over a row of n random terms they add up to
+        # about sqrt(n) * 2^-11 * |c| * |v| - three times that is the bound
+        bound = 3 * (n ** 0.5) * 2.0 ** -11 * c.double().abs().mean() * v.abs().mean() * 1.3
+        assert (got - want).abs().max() < bound, ((got - want).abs().max(), bound)
+    # and the rows and columns are where they belong: two single-row / single-column spot checks in float64
+    i, j = 1234, 4321
+    assert abs(float(c[i, j]) - float(a[i].double() @ b[:, j].double())) < 1e-2 * max(1.0, abs(float(c[i, j])))
+    assert abs(float(c[n - 1, 0]) - float(a[n - 1].double() @ b[:, 0].double())) < 1e-2 * max(1.0, abs(float(c[n - 1, 0])))
