@@ -214,10 +214,13 @@ def fuse_elementwise(graph: Graph) -> Graph:
 
 def _divisor_near(extent: int, target: int) -> int:
     """The divisor of `extent` closest to `target` within a factor of two of it, or 0."""
-    best = 0
-    for d in range(max(2, target // 2), min(extent, target * 2) + 1):
-        if extent % d == 0 and (best == 0 or abs(d - target) < abs(best - target)):
-            best = d
+    best, d = 0, 1
+    while d * d <= extent:
+        if extent % d == 0:
+            for c in (d, extent // d):
+                if max(2, target // 2) <= c <= target * 2 and (best == 0 or abs(c - target) < abs(best - target)):
+                    best = c
+        d += 1
     return best
 
 
