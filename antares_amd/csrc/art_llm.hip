@@ -104,35 +104,31 @@ __global__ __launch_bounds__(256) void rotary_kernel(const XT* __restrict__ x, c
 // att[h,s] = (sum_m q[h,m] k[s,h,m]) * att_f ; p = softmax_s(att) ; out[h,m] = sum_s p[h,s] v[s,h,m]
 // One block of 512 threads per head.  Eight lanes share a position (16 dims = 32 bytes of fp16 each), so
 // a wavefront reads eight 256-byte rows per step; every 8-lane group keeps an online-softmax state (max,
-// sum, 16 partial outputs) for the positions it visits and has four positions in flight, 256 positions
-// (128 KiB) per block - a compute unit needs that much outstanding to stream at its full rate.  The
+// sum, 16 partial outputs) for the positions it visits and has four fp16 (two fp32) positions in flight,
+// 128 KiB per block - a compute unit needs that much outstanding to stream at its full rate.  The
 // eight groups of a wavefront are merged with lane exchanges, the eight wavefronts through LDS.
-template <class T> struct Row16;   // 16 consecutive elements as floats
+
+// 16 consecutive elements of a cache row, kept as loaded (fp16 rows stay packed: half the registers of a
+// converted copy, which is what lets four positions per group be in flight without spilling) and converted where
+// they are used.
+template <class T> struct Row16;
 template <> struct Row16<_Float16> {
-  static __device__ __forceinline__ void load(const _Float16* p, float (&f)[16]) {
-    const u32x4 a = *reinterpret_cast<const u32x4*>(p), b = *reinterpret_cast<const u32x4*>(p + 8);
-    const unsigned int wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-      const h2 v = __builtin_bit_cast(h2, wds[i]);
-      f[2 * i] = (float)v.x;
-      f[2 * i + 1] = (float)v.y;
-    }
+  typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+  struct Raw { h8 lo, hi; };
+  static __device__ __forceinline__ void load(const _Float16* p, Raw& r) {
+    r.lo = *reinterpret_cast<const h8*>(p);
+    r.hi = *reinterpret_cast<const h8*>(p + 8);
   }
+  static __device__ __forceinline__ float at(const Raw& r, int i) { return i < 8 ? (float)r.lo[i] : (float)r.hi[i - 8]; }
 };
 template <> struct Row16<float> {
-  static __device__ __forceinline__ void load(const float* p, float (&f)[16]) {
-    typedef float f32x4 __attribute__((ext_vector_type(4)));
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  struct Raw { f32x4 q[4]; };
+  static __device__ __forceinline__ void load(const float* p, Raw& r) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const f32x4 a = *reinterpret_cast<const f32x4*>(p + 4 * i);
-      f[4 * i] = a[0];
-      f[4 * i + 1] = a[1];
-      f[4 * i + 2] = a[2];
-      f[4 * i + 3] = a[3];
-    }
+    for (int i = 0; i < 4; ++i) r.q[i] = *reinterpret_cast<const f32x4*>(p + 4 * i);
   }
+  static __device__ __forceinline__ float at(const Raw& r, int i) { return r.q[i >> 2][i & 3]; }
 };
 
 constexpr int kAttThreads = 512;
@@ -162,7 +158,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
   // parts > 1: `parts` blocks share a head, each attends over a contiguous range of the cached positions and
   // leaves its unnormalised state in partial[head][part][kAttPartialStride] = { acc[128], max, sum, -, - };
   // whoever consumes the result merges them (the o-projection does it while it loads x).
-  constexpr int D = 128, U = 4;                          // len_host: the length, or the rows of the cache when len_dev is given
+  constexpr int D = 128, U = 8 / sizeof(KT);              // len_host: the length, or the rows of the cache when len_dev is given
   __shared__ float s_m[kAttWaves], s_l[kAttWaves];
   __shared__ float s_acc[kAttWaves][D];
   __shared__ float s_q[D];
@@ -208,7 +204,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
   }
   // U positions per group are requested before the first is used, and the first round is requested
   // before the rotary phase, which does not depend on it
-  float kf[U][16], vf[U][16];
+  typename Row16<KT>::Raw kf[U], vf[U];
   auto request = [&](int s0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -264,12 +260,12 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
     d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xf, 0xf, false));
     return d;
   };
-  auto absorb = [&](float d, const float (&vrow)[16]) {   // one position into this group's online softmax
+  auto absorb = [&](float d, auto value) {                // one position into this group's online softmax
     const float mn = fmaxf(m, d);
     const float corr = __expf(m - mn), p = __expf(d - mn);
     l = l * corr + p;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * vrow[i]);
+    for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * value(i));
     m = mn;
   };
   for (int s0 = s_start; s0 < Sc; s0 += kAttGroups * U) {
@@ -278,9 +274,9 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
     for (int u = 0; u < U; ++u) {
       float d = 0.f;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kf[u][i], d);
+      for (int i = 0; i < 16; ++i) d = fmaf(qf[i], Row16<KT>::at(kf[u], i), d);
       d = group_sum(d);
-      if (s0 + u * kAttGroups < Sc) absorb(d, vf[u]);
+      if (s0 + u * kAttGroups < Sc) absorb(d, [&](int i) { return Row16<KT>::at(vf[u], i); });
     }
   }
   if (newest_here) {                                      // the newest position, from LDS, joins group 0
@@ -294,7 +290,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
 #pragma unroll
     for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kn[i], d);
     d = group_sum(d);
-    if (group == 0) absorb(d, vn);
+    if (group == 0) absorb(d, [&](int i) { return vn[i]; });
   }
   att_merge_lane(m, l, acc, 8);       // the eight groups of a wavefront: lanes that differ in bits 3..5
   att_merge_lane(m, l, acc, 16);
