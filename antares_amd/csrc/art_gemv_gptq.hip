@@ -15,8 +15,8 @@
 //     v_cvt_f32_ubyte0..3 turns each byte into a float, one FMA per weight: 2.4 VALU operations per weight;
 //   * the k lanes of a block meet in LDS; the owner of a column applies scale and the fixed zero point 8 once
 //     per (group, column): s * (acc - 8 * sum(x));
-//   * the K-splits of a column meet in one returning 64-bit atomic: a 2^-30 fixed-point partial sum with an
-//     arrival count in the top byte.  Integer addition is associative, so the result does not depend on the
+//   * the K-splits of a column meet in one returning 64-bit atomic: a fixed-point partial sum (steps of 2^-22) with an
+//     arrival count in the top byte and a count of non-finite partial sums in the bottom one.  Integer addition is associative, so the result does not depend on the
 //     arrival order; the block that sees count == splits - 1 holds the total, writes y and clears the slot.
 #include "art_common.h"
 
@@ -33,6 +33,19 @@ constexpr int R = 8;                   // word rows per lane (64 values of k)
 constexpr int kBlockK = KL * R * 8;    // 1024 values of k per block
 constexpr int GB = kBlockK / 128;      // 8 quantisation groups per block, two k lanes each
 constexpr float kFix = 1073741824.f;   // 2^30
+
+// A partial sum on its way through the 64-bit slot: a multiple of 256 in units of 2^-30 (so 2^-22 is the step), which
+// leaves the low byte free to count the partial sums that are not finite or too large for the field (2^24 / splits
+// keeps the sum of all of them below 2^55, clear of the arrival count above it).  Such a partial sum contributes 1:
+// it can neither run into the count - which would leave the slot dirty for every later launch - nor get lost: a
+// total with a non-zero low byte is written out as NaN.
+__device__ __forceinline__ long long to_fixed(float r, int splits) {
+  const float limit = 16777216.f / (float)splits;
+  return fabsf(r) < limit ? __float2ll_rn(r * (kFix / 256.f)) * 256 : 1LL;     // NaN fails the comparison too
+}
+__device__ __forceinline__ float from_fixed(long long total) {
+  return (total & 255) ? __builtin_nanf("") : (float)total * (1.f / kFix);
+}
 
 template <class T> __device__ __forceinline__ float ldf(const T* p, size_t i) { return (float)p[i]; }
 
@@ -112,13 +125,13 @@ __global__ __launch_bounds__(kThreads) void gemv_gptq_kernel(const XT* __restric
     y[col] = (XT)res;
     return;
   }
-  // one returning atomic: [arrival count : 8][2^-30 fixed-point sum : 56]
+  // one returning atomic: [arrival count : 8][fixed-point sum : 56]
   unsigned long long* slot = slots + col;
-  const long long mine = (1LL << 56) + __float2ll_rn(res * kFix);
+  const long long mine = (1LL << 56) + to_fixed(res, splits);
   const long long old = (long long)__hip_atomic_fetch_add(slot, (unsigned long long)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (((old + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
     const long long total = old + mine - ((long long)splits << 56);
-    y[col] = (XT)((float)total * (1.f / kFix));
+    y[col] = (XT)from_fixed(total);
     *slot = 0ull;                       // ready for the next launch (stream order makes this visible)
   }
 }

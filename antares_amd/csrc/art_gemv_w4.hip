@@ -28,8 +28,9 @@
 //   * the k lanes of a block meet in LDS (16 KiB), the owner of a column applies
 //     scale and zero point;
 //   * the K-splits of a column meet in ONE returning 64-bit atomic per block:
-//     the partial sum travels as a 2^-30 fixed-point integer with an arrival
-//     count in the top byte.  Integer addition is associative, so the result
+//     the partial sum travels as a fixed-point integer (steps of 2^-22) with an
+//     arrival count in the top byte and a count of non-finite partial sums in the
+//     bottom one.  Integer addition is associative, so the result
 //     does not depend on arrival order (deterministic), and the block whose
 //     atomic returns count == splits-1 holds the complete sum in registers: it
 //     writes y and resets the slot.  One round trip, no fence, no re-read.
@@ -79,6 +80,19 @@ constexpr int KL = kThreads / CL;      // 32 k lanes per block, 8 per wavefront 
 constexpr int CT = 16 * CL;            // 128 columns per block
 constexpr int kRowsPerBlock = KL * R;  // 256 packed rows = 512 values of k
 constexpr float kFix = 1073741824.f;   // 2^30
+
+// A partial sum on its way through the 64-bit slot: a multiple of 256 in units of 2^-30 (so 2^-22 is the step), which
+// leaves the low byte free to count the partial sums that are not finite or too large for the field (2^24 / splits
+// keeps the sum of all of them below 2^55, clear of the arrival count above it).  Such a partial sum contributes 1:
+// it can neither run into the count - which would leave the slot dirty for every later launch - nor get lost: a
+// total with a non-zero low byte is written out as NaN.
+__device__ __forceinline__ long long to_fixed(float r, int splits) {
+  const float limit = 16777216.f / (float)splits;
+  return fabsf(r) < limit ? __float2ll_rn(r * (kFix / 256.f)) * 256 : 1LL;     // NaN fails the comparison too
+}
+__device__ __forceinline__ float from_fixed(long long total) {
+  return (total & 255) ? __builtin_nanf("") : (float)total * (1.f / kFix);
+}
 
 // Sum over the 8 k lanes of a wavefront (lanes that share lane % 8); all lanes get the sum.
 __device__ __forceinline__ float sum_k_lanes_of_wave(float v) {
@@ -350,13 +364,13 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
       y[(size_t)m * N + col] = o;
       continue;
     }
-    // one returning atomic: [arrival count : 8][2^-30 fixed-point sum : 56]
+    // one returning atomic: [arrival count : 8][fixed-point sum : 56]
     unsigned long long* slot = slots + (size_t)m * N + col;
-    const long long mine = (1LL << 56) + __float2ll_rn(r * kFix);
+    const long long mine = (1LL << 56) + to_fixed(r, splits);
     const long long old = (long long)__hip_atomic_fetch_add(slot, (unsigned long long)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (((old + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
       const long long total = old + mine - ((long long)splits << 56);
-      _Float16 o = (_Float16)((float)total * (1.f / kFix));
+      _Float16 o = (_Float16)from_fixed(total);
       if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)fused.residual[col]);
       y[(size_t)m * N + col] = o;
       *slot = 0ull;                     // ready for the next launch (stream order makes this visible)

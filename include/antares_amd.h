@@ -107,6 +107,9 @@ int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* strea
  * x: fp16 [M,K]; qweight: uint8 [K/2,N], low nibble = even k; scales: fp16
  * [K/128,N]; qzeros: uint8 [K/128,N/2], low nibble = even n; y: fp16 [M,N].
  * fp32 accumulation.  M <= 8 here (decode); K % 128 == 0, N % 16 == 0.
+ * The sums over the K/512 slices of k meet as fixed-point numbers (steps of
+ * 2^-22): a slice whose sum is NaN, infinite or beyond 2^24 / (K/512) in
+ * magnitude turns y[m,n] into NaN (its exact value would be far outside fp16).
  * Replaces the kernel the reference generates from the dequant+GEMV program
  * of samples/05_llama2_7b_int4.py:135-144 (antares/default_codegen.py:13). */
 int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
@@ -134,7 +137,9 @@ int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, const void*
 /* The reference's own weight format (samples/05_llama2_7b_int4.py:135-139):
  * qweight int32 [K/8,N], eight nibbles per word along K (least significant
  * first), zero point fixed at 8, scales fp32 or fp16 [K/128,N], x and y fp32
- * or fp16 (x_f16 / scales_f16 select).  M = 1. */
+ * or fp16 (x_f16 / scales_f16 select).  M = 1.  The sums over the K/1024
+ * slices of k meet as fixed-point numbers (steps of 2^-22): a slice whose sum
+ * is NaN, infinite or beyond 2^24 / (K/1024) in magnitude turns y[n] into NaN. */
 int art_gemv_gptq(const void* x_dev, const void* qweight_dev, const void* scales_dev, void* y_dev,
                   int K, int N, int x_f16, int scales_f16, void* stream);
 

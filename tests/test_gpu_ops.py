@@ -196,6 +196,50 @@ def test_w4a16_gemv_entry_point_up_to_eight_rows(autort, M, K, N):
     assert np.allclose(y.cpu().numpy().astype(np.float32), want.astype(np.float32), **FP16_TOL)
 
 
+@pytest.mark.parametrize('poison', [float('nan'), float('inf'), 60000.0])
+def test_gemv_with_non_finite_rows_stays_clean(autort, poison):
+    """A NaN, an infinity or values that overflow the sum in x must come out as non-finite results (the reference's
+    float sums propagate them) and must not leave anything behind in the split-K slots: the same operator called
+    on ordinary data right afterwards gives the ordinary answer."""
+    from antares_amd.autort import patterns
+    from oracle import hot_ops
+    note(f'w4a16 / gptq gemv with x poisoned by {poison}')
+    dev = autort.device()
+    K, N = 4096, 1024
+    p = workloads.w4_problem(77, 1, K, N)
+    f = w4_op(autort)
+    args = [p[k].to(dev) for k in ('x', 'qweight', 'scales', 'qzeros')]
+    good = f(*args)
+    bad_x = args[0].clone()
+    if poison == 60000.0:
+        bad_x[:] = poison                        # finite, but every partial sum is far outside fp16
+    else:
+        bad_x[0, 1000] = poison
+    bad = f(bad_x, *args[1:])
+    if poison != 60000.0:
+        assert not torch.isfinite(bad).any()
+    again = f(*args)
+    assert torch.equal(again, good)
+    want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy())
+    assert np.allclose(again.cpu().numpy().astype(np.float32), want.astype(np.float32), **FP16_TOL)
+    # the sample's own program (fp32, GPTQ words)
+    g = torch.Generator().manual_seed(5)
+    q = torch.randint(0, 16, (K, N), generator=g)
+    s = torch.rand(K // 128, N, generator=g) * 0.019 + 0.001
+    x = torch.randn(K, generator=g)
+    h = autort.export(ir=patterns.GPTQ_GEMV_IR, inputs=patterns._gptq_inputs('float32', 'float32'))
+    qw = workloads.pack_gptq(q).to(dev)
+    good = h(x.to(dev), qw, s.to(dev)).clone()
+    bad_x = x.clone()
+    if poison == 60000.0:
+        bad_x[:] = 1e30                          # the sums are beyond what a split-K slot carries: reported as NaN
+    else:
+        bad_x[17] = poison
+    bad = h(bad_x.to(dev), qw, s.to(dev))
+    assert not torch.isfinite(bad).any()
+    assert torch.equal(h(x.to(dev), qw, s.to(dev)), good)
+
+
 def test_w4a16_generic_lowering_agrees(autort):
     """The same program through the generic reduce lowering (no hand kernel)."""
     from oracle import hot_ops
