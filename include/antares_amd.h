@@ -10,6 +10,14 @@
  * the library owns loaded modules for the life of the process and one internal
  * workspace per device that is allocated by art_init().
  *
+ * The kernels that split K or work in two passes (art_gemv_w4a16*, art_gemv_gptq,
+ * art_gemm_w4a16, art_partition_even_first_i32) keep their partial results in
+ * that workspace, so on one device two of their launches must not be in flight
+ * at the same time: enqueue them on one stream, or order the streams with
+ * events.  The reference has the same single-caller contract (static state, no
+ * locks: frameworks/pytorch/main_ops.cc:14-15).  Launches leave the workspace
+ * clean, also when their inputs hold NaN or infinities.
+ *
  * The first group replaces the reference's header-only `namespace ab` device
  * runtime and its ExecutionModule; the second group are typed entry points for
  * the hand-written kernels that replace generated code on the hot path.
