@@ -11,8 +11,8 @@ tensors that only live between two kernels; frameworks/pytorch/main_ops.cc:17-54
 
 This module is that pair on the C ABI of this library: containers come from
 `antares_amd.lower.evaluator_emit.emit_evaluator_module` (or from a file written by it), kernels are compiled
-in-process for gfx950 and launched on torch's current stream.  Launch extents given by `$` keys (run-time sized
-grids) are not produced by this build's emitter and are rejected here.
+in-process for gfx950 and launched on torch's current stream.  Launch extents given by `$` keys (grids sized at
+launch time from the integer arguments) follow the reference's rule; this build's own emitter does not write them.
 """
 from __future__ import annotations
 
@@ -74,12 +74,20 @@ class ExecutionModule:
                 self.local_tensors[n] = (dt, shape)
             threads: Dict[str, int] = {}
             for key, val in re.findall(r'// \[thread_extent\] (\S+) = (-?\d+)', piece):
-                if key.startswith('$'):
-                    raise NotImplementedError('run-time sized launch extents (`$` keys) are not supported')
                 if threads.get(key, 0) > 0 and threads[key] != int(val):
                     raise ValueError(f'Multiple `{key}` extents conflict in values: {threads[key]} v.s. {val}')
                 threads[key] = int(val)
-            self.kernels.append({'name': name, 'in': [p[0] for p in ins], 'out': [p[0] for p in outs], 'threads': threads})
+            # Run-time sized grid (backends/c-rocm/include/backend.hpp:184-194, 204-215): `$` is the position of the
+            # first integer argument that sizes it, `$$` a constant factor, `$i` the elements a block takes of the
+            # i-th such argument (negative: that argument does not count).
+            dynamic = None
+            if threads.get('$', 0):
+                divisors = []
+                while threads.get(f'${len(divisors)}', 0):
+                    divisors.append(threads[f'${len(divisors)}'])
+                dynamic = (threads['$'], threads.get('$$', 1), divisors)
+            self.kernels.append({'name': name, 'in': [p[0] for p in ins], 'out': [p[0] for p in outs], 'threads': threads,
+                                 'dynamic': dynamic})
         if not self.kernels:
             raise ValueError('the container holds no kernel')
         self._image = compile_cached(source)
@@ -118,10 +126,20 @@ class ExecutionModule:
                     dt, shape = self.local_tensors[n]
                     memory[n] = torch.empty(shape, dtype=TORCH_DTYPE[dt], device=dev)
             th = k['threads']
+            args = [memory[n].data_ptr() for n in k['in'] + k['out']] + self.dim_values
+            grid_x = th.get('blockIdx.x', 1)
+            if k['dynamic'] is not None:
+                first, grid_x, divisors = k['dynamic']
+                if first + len(divisors) > len(args) or first < len(k['in']) + len(k['out']):
+                    raise ValueError(f'kernel `{k["name"]}`: `$ = {first}` does not point at its integer arguments')
+                for i, d in enumerate(divisors):
+                    if d > 0:
+                        grid_x *= (args[first + i] + d - 1) // d
+                if grid_x == 0:
+                    continue                        # nothing to do at these sizes (backend.hpp:214)
             capi.launch(module.function(k['name']),
-                        (th.get('blockIdx.x', 1), th.get('blockIdx.y', 1), th.get('blockIdx.z', 1)),
-                        (th.get('threadIdx.x', 1), th.get('threadIdx.y', 1), th.get('threadIdx.z', 1)), stream,
-                        [memory[n].data_ptr() for n in k['in'] + k['out']] + self.dim_values)
+                        (grid_x, th.get('blockIdx.y', 1), th.get('blockIdx.z', 1)),
+                        (th.get('threadIdx.x', 1), th.get('threadIdx.y', 1), th.get('threadIdx.z', 1)), stream, args)
 
 
 _sources: List[str] = []

@@ -31,10 +31,50 @@ def test_container_is_parsed_like_the_reference_does():
     assert [k['out'] for k in m.kernels] == [['temp0'], ['temp1'], ['output0']]
     assert all(k['threads']['threadIdx.x'] == 256 and k['threads']['blockIdx.x'] >= 1 for k in m.kernels)
     assert m.local_tensors['temp1'] == ('float32', [8])
-    with pytest.raises(NotImplementedError):
-        ExecutionModule(text.replace('// [thread_extent] blockIdx.x = ', '// [thread_extent] $ = 1\n// [thread_extent] blockIdx.x = ', 1))
+    assert all(k['dynamic'] is None for k in m.kernels)
     with pytest.raises(ValueError):
         ExecutionModule('// no globals here\n')
+
+
+DYNAMIC_GRID = '''// GLOBALS: a:float32[1000] -> b:float32[1000]
+// BACKEND: c-mi355x (default)
+// VAMAP: N:%d
+// ---------------------------------------------------------------------------
+// LOCAL: scale_k -- a:float32[1000] -> b:float32[1000]
+
+extern "C" __global__ __launch_bounds__(128) void scale_k(float* __restrict__ a, float* __restrict__ b, int N) {
+  // [thread_extent] threadIdx.x = 128
+  // [thread_extent] $ = 2
+  // [thread_extent] $$ = 1
+  // [thread_extent] $0 = 128
+  const int i = blockIdx.x * 128 + threadIdx.x;
+  if (i < N) b[i] = a[i] * 3.0f + (float)gridDim.x;
+}
+'''
+
+
+def test_grid_sized_at_launch_is_parsed():
+    """`$` keys (backends/c-rocm/include/backend.hpp:184-194): first integer argument, constant factor, per-argument block sizes."""
+    m = ExecutionModule(DYNAMIC_GRID % 1000)
+    assert m.dim_values == [1000] and m.kernels[0]['dynamic'] == (2, 1, [128])
+    assert m.kernels[0]['threads']['threadIdx.x'] == 128
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('n', [1000, 129, 1, 0])
+def test_grid_sized_at_launch_runs(n):
+    """gridDim.x = $$ * ceil(N / $0) is worked out from the integer argument at launch; 0 blocks: nothing is launched."""
+    import autort
+    print(f'[case] run-time sized grid N={n}', flush=True)
+    dev = autort.device()
+    a = torch.arange(1000, dtype=torch.float32, device=dev)
+    b = torch.full((1000,), -1.0, device=dev)
+    ExecutionModule(DYNAMIC_GRID % n).compute([a, b])
+    want = torch.full((1000,), -1.0)
+    want[:n] = torch.arange(n, dtype=torch.float32) * 3 + (n + 127) // 128
+    assert torch.equal(b.cpu(), want)
+    with pytest.raises(ValueError):
+        ExecutionModule(DYNAMIC_GRID.replace('$ = 2', '$ = 1') % n).compute([a, b])
 
 
 def test_keys_count_up_and_unknown_keys_fail():
