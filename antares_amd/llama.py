@@ -124,6 +124,7 @@ class LlamaInt4Decoder:
         self.hb = torch.empty(cfg.ffn, **f16)
         self.logits = torch.empty(cfg.vocab, **f16)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self._prefill_cache: Dict[int, Dict[str, object]] = {}      # prompt length -> operators of `prefill`
         self._ops()
 
     def _ops(self):
@@ -193,6 +194,93 @@ class LlamaInt4Decoder:
             self.add(self.x, self.proj)
         ops.rmsnorm_f16(self.x, None, self.w['final_norm'], self.xb, extra=[1.0 / d, cfg.rms_eps])
         self._linear(self.xb, self.w['lm_head'], self.logits)
+        return self.logits
+
+    # -- whole-prompt ingestion ------------------------------------------------
+    def _prefill_ops(self, T: int):
+        """Operators of `prefill` for a prompt of T tokens: einstein_v2 programs at static sizes (compiled once per
+        T and kept in the code-object cache) around the batched int4 projections."""
+        ops = self._prefill_cache.get(T)
+        if ops is not None:
+            return ops
+        cfg, a = self.cfg, self.autort
+        d, H, D, F, V = cfg.dim, cfg.n_heads, cfg.head_dim, cfg.ffn, cfg.vocab
+        J = D // 2
+        f32 = '.to(`float32`)'
+        ang = f'(T{f32} * freq[J]{f32})'
+        rope = (f'(src[T, {{base}} + H * {D} + P * {J} + J]{f32} * {ang}.call(`cos`) + (P * 2 - 1){f32} * '
+                f'src[T, {{base}} + H * {D} + (1 - P) * {J} + J]{f32} * {ang}.call(`sin`)).to(`float16`) where H in {H}, P in 2, J in {J}')
+        scale = repr(1.0 / math.sqrt(D))
+        ops = {
+            'embed': a.export(ir='emb[T, D] = table[tok[T], D]', inputs=[f'table=float16[{V}, {d}]', f'tok=int32[{T}]'],
+                              name=f'prefill_embed_{T}'),
+            'rms': a.export(ir=f'ss[T] +=! x[T, D]{f32} * x[T, D]{f32}; '
+                               f'out[T, D] = (x[T, D]{f32} * (ss[T] * {1.0 / d!r} + {cfg.rms_eps!r}).call(`rsqrt`) * w[D]{f32}).to(`float16`)',
+                            inputs=[f'x=float16[{T}, {d}]', f'w=float16[{d}]'], name=f'prefill_rmsnorm_{T}'),
+            'rope_q': a.export(ir='qr[T, H, P, J] = ' + rope.format(base=0), inputs=[f'src=float16[{T}, {3 * d}]', f'freq=float16[{D}]'],
+                               name=f'prefill_rope_q_{T}'),
+            'rope_k': a.export(ir='kr[T, H, P, J] = ' + rope.format(base=d), inputs=[f'src=float16[{T}, {3 * d}]', f'freq=float16[{D}]'],
+                               name=f'prefill_rope_k_{T}'),
+            'copy_v': a.export(ir=f'vc[T, D] = src[T, {2 * d} + D] where D in {d}', inputs=[f'src=float16[{T}, {3 * d}]'],
+                               name=f'prefill_copy_v_{T}'),
+            'scores': a.export(ir=f'sc[H, T, S] +=! qr[T, H, D]{f32} * kc[S, H, D]{f32}',
+                               inputs=[f'qr=float16[{T}, {H}, {D}]', f'kc=float16[{T}, {H}, {D}]'], name=f'prefill_scores_{T}'),
+            'softmax_v': a.export(
+                ir=f'mx[H, T] >=! (sc[H, T, S] * {scale}).when([S <= T], -3.0e38); '
+                   f'ex[H, T, S] = (sc[H, T, S] * {scale} - mx[H, T]).call(`exp`).when([S <= T], 0.0); '
+                   f'den[H, T] +=! ex[H, T, S]; '
+                   f'av[T, H, D] +=! ex[H, T, S] * vc[S, H, D]{f32}; '
+                   f'att[T, H, D] = (av[T, H, D] / den[H, T]).to(`float16`)',
+                inputs=[f'sc=float32[{H}, {T}, {T}]', f'vc=float16[{T}, {H}, {D}]'], name=f'prefill_softmax_v_{T}'),
+            'silu_mul': a.export(
+                ir=f'hid[T, N] = (gu[T, N]{f32} / (1.0 + (0.0 - gu[T, N]{f32}).call(`exp`)) * gu[T, {F} + N]{f32}).to(`float16`) where N in {F}',
+                inputs=[f'gu=float16[{T}, {2 * F}]'], name=f'prefill_silu_mul_{T}'),
+        }
+        self._prefill_cache[T] = ops
+        return ops
+
+    def prefill(self, tokens: torch.Tensor) -> torch.Tensor:
+        """Ingests a whole prompt (int32 [T] on the device, T >= 4, positions 0..T-1) in one pass: the projections
+        run as batched int4 GEMMs on the matrix cores (`gemv_w4a16` with T rows), attention is causal over the
+        prompt, keys and values land in cache rows 0..T-1.  Leaves the step state at the last prompt position
+        (self.pos = T - 1, self.x = its hidden state, self.logits = its logits), so `advance()` and the recorded
+        decode step continue from there.  Same operators and roundings as the one-token step, applied to T rows."""
+        cfg = self.cfg
+        T = int(tokens.numel())
+        d, H, D, F = cfg.dim, cfg.n_heads, cfg.head_dim, cfg.ffn
+        if not 4 <= T <= cfg.max_seq:
+            raise ValueError(f'prefill takes 4..{cfg.max_seq} tokens, got {T}')
+        ops = self._prefill_ops(T)
+        f16 = dict(dtype=torch.float16, device=self.dev)
+        x = ops['embed'](self.w['embed'], tokens.view(T))
+        qkv, proj = torch.empty(T, 3 * d, **f16), torch.empty(T, d, **f16)
+        gu = torch.empty(T, 2 * F, **f16)
+
+        def linear(inp, lin, out):
+            self.gemv(inp, lin['qweight'], lin['scales'], lin['qzeros'], out=out)
+
+        for l, lw in enumerate(self.w['layers']):
+            xb = ops['rms'](x, lw['att_norm'])
+            linear(xb, lw['qkv'], qkv)
+            kc, vc = self.key_cache[l][:T], self.val_cache[l][:T]
+            qr = ops['rope_q'](qkv, self.inv_freq)
+            ops['rope_k'](qkv, self.inv_freq, out=kc.view(T, H, 2, D // 2))
+            ops['copy_v'](qkv, out=vc)
+            sc = ops['scores'](qr.view(T, H, D), kc.view(T, H, D))
+            att = ops['softmax_v'](sc, vc.view(T, H, D))
+            linear(att.view(T, d), lw['o'], proj)
+            self.add(x.view(-1), proj.view(-1))
+            xb = ops['rms'](x, lw['ffn_norm'])
+            linear(xb, lw['gate_up'], gu)
+            hid = ops['silu_mul'](gu)
+            linear(hid, lw['down'], proj)
+            self.add(x.view(-1), proj.view(-1))
+        self.x.copy_(x[T - 1])
+        self.pos.fill_(T - 1)
+        self.token.copy_(tokens.view(T)[T - 1:T])
+        h = self.w['lm_head']
+        self.autort.ops.gemv_w4a16_fused(self.x, h['qweight'], h['scales'], h['qzeros'], self.logits,
+                                         norm_weight=self.w['final_norm'], eps=cfg.rms_eps)
         return self.logits
 
     def advance(self, prompt: Optional[torch.Tensor] = None):
