@@ -203,7 +203,13 @@ class LlamaInt4Decoder:
         ops = self._prefill_cache.get(T)
         if ops is not None:
             return ops
-        cfg, a = self.cfg, self.autort
+        from .autort.op import ExportedOp
+
+        class _Programs:            # same operators as autort.export makes, but neither listed in autort.ops nor written
+            @staticmethod          # to module files: there is one set per prompt length
+            def export(ir, inputs, name):
+                return ExportedOp(ir, list(inputs), name=name)
+        cfg, a = self.cfg, _Programs
         d, H, D, F, V = cfg.dim, cfg.n_heads, cfg.head_dim, cfg.ffn, cfg.vocab
         J = D // 2
         f32 = '.to(`float32`)'
