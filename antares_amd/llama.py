@@ -205,11 +205,11 @@ class LlamaInt4Decoder:
             return ops
         from .autort.op import ExportedOp
 
-        class _Programs:            # same operators as autort.export makes, but neither listed in autort.ops nor written
-            @staticmethod          # to module files: there is one set per prompt length
-            def export(ir, inputs, name):
-                return ExportedOp(ir, list(inputs), name=name)
-        cfg, a = self.cfg, _Programs
+        def program(ir, inputs, name):
+            # the operator autort.export would make, but neither listed in autort.ops nor written to a module file:
+            # there is one set of these per prompt length
+            return ExportedOp(ir, list(inputs), name=name)
+        cfg = self.cfg
         d, H, D, F, V = cfg.dim, cfg.n_heads, cfg.head_dim, cfg.ffn, cfg.vocab
         J = D // 2
         f32 = '.to(`float32`)'
@@ -218,27 +218,27 @@ class LlamaInt4Decoder:
                 f'src[T, {{base}} + H * {D} + (1 - P) * {J} + J]{f32} * {ang}.call(`sin`)).to(`float16`) where H in {H}, P in 2, J in {J}')
         scale = repr(1.0 / math.sqrt(D))
         ops = {
-            'embed': a.export(ir='emb[T, D] = table[tok[T], D]', inputs=[f'table=float16[{V}, {d}]', f'tok=int32[{T}]'],
+            'embed': program(ir='emb[T, D] = table[tok[T], D]', inputs=[f'table=float16[{V}, {d}]', f'tok=int32[{T}]'],
                               name=f'prefill_embed_{T}'),
-            'rms': a.export(ir=f'ss[T] +=! x[T, D]{f32} * x[T, D]{f32}; '
+            'rms': program(ir=f'ss[T] +=! x[T, D]{f32} * x[T, D]{f32}; '
                                f'out[T, D] = (x[T, D]{f32} * (ss[T] * {1.0 / d!r} + {cfg.rms_eps!r}).call(`rsqrt`) * w[D]{f32}).to(`float16`)',
                             inputs=[f'x=float16[{T}, {d}]', f'w=float16[{d}]'], name=f'prefill_rmsnorm_{T}'),
-            'rope_q': a.export(ir='qr[T, H, P, J] = ' + rope.format(base=0), inputs=[f'src=float16[{T}, {3 * d}]', f'freq=float16[{D}]'],
+            'rope_q': program(ir='qr[T, H, P, J] = ' + rope.format(base=0), inputs=[f'src=float16[{T}, {3 * d}]', f'freq=float16[{D}]'],
                                name=f'prefill_rope_q_{T}'),
-            'rope_k': a.export(ir='kr[T, H, P, J] = ' + rope.format(base=d), inputs=[f'src=float16[{T}, {3 * d}]', f'freq=float16[{D}]'],
+            'rope_k': program(ir='kr[T, H, P, J] = ' + rope.format(base=d), inputs=[f'src=float16[{T}, {3 * d}]', f'freq=float16[{D}]'],
                                name=f'prefill_rope_k_{T}'),
-            'copy_v': a.export(ir=f'vc[T, D] = src[T, {2 * d} + D] where D in {d}', inputs=[f'src=float16[{T}, {3 * d}]'],
+            'copy_v': program(ir=f'vc[T, D] = src[T, {2 * d} + D] where D in {d}', inputs=[f'src=float16[{T}, {3 * d}]'],
                                name=f'prefill_copy_v_{T}'),
-            'scores': a.export(ir=f'sc[H, T, S] +=! qr[T, H, D]{f32} * kc[S, H, D]{f32}',
+            'scores': program(ir=f'sc[H, T, S] +=! qr[T, H, D]{f32} * kc[S, H, D]{f32}',
                                inputs=[f'qr=float16[{T}, {H}, {D}]', f'kc=float16[{T}, {H}, {D}]'], name=f'prefill_scores_{T}'),
-            'softmax_v': a.export(
+            'softmax_v': program(
                 ir=f'mx[H, T] >=! (sc[H, T, S] * {scale}).when([S <= T], -3.0e38); '
                    f'ex[H, T, S] = (sc[H, T, S] * {scale} - mx[H, T]).call(`exp`).when([S <= T], 0.0); '
                    f'den[H, T] +=! ex[H, T, S]; '
                    f'av[T, H, D] +=! ex[H, T, S] * vc[S, H, D]{f32}; '
                    f'att[T, H, D] = (av[T, H, D] / den[H, T]).to(`float16`)',
                 inputs=[f'sc=float32[{H}, {T}, {T}]', f'vc=float16[{T}, {H}, {D}]'], name=f'prefill_softmax_v_{T}'),
-            'silu_mul': a.export(
+            'silu_mul': program(
                 ir=f'hid[T, N] = (gu[T, N]{f32} / (1.0 + (0.0 - gu[T, N]{f32}).call(`exp`)) * gu[T, {F} + N]{f32}).to(`float16`) where N in {F}',
                 inputs=[f'gu=float16[{T}, {2 * F}]'], name=f'prefill_silu_mul_{T}'),
         }
