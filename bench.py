@@ -51,10 +51,13 @@ def parse_args():
     return ap.parse_args()
 
 
-def time_graph(torch, capi, fn, steps, warmup):
+def time_graph(torch, capi, fn, steps, warmup, warm_ms=0.0):
     """Records ``fn`` (which enqueues kernels on the current stream) in a HIP
     graph, replays it warmup + steps times, returns mean seconds per replay of
-    the timed ones, measured with events on the replay stream."""
+    the timed ones, measured with events on the replay stream.  ``warm_ms`` > 0
+    keeps replaying until that much time has gone by: a kernel that loads the
+    matrix cores for a millisecond at a time only settles at its sustained
+    clock after some tens of milliseconds."""
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         fn()                                   # first call: compiles / loads modules, outside capture
@@ -65,6 +68,11 @@ def time_graph(torch, capi, fn, steps, warmup):
         for _ in range(warmup):
             graph.replay()
         stream.synchronize()
+        t_end = time.perf_counter() + warm_ms * 1e-3
+        while warm_ms > 0 and time.perf_counter() < t_end:
+            for _ in range(4):
+                graph.replay()
+            stream.synchronize()
         torch.cuda.synchronize()
         start, stop = capi.Event(), capi.Event()
         start.record(stream.cuda_stream)
@@ -104,7 +112,7 @@ def bench_gemm_f16(torch, autort, capi, workloads, steps, warmup, seed, n):
     op = autort.export(ir=patterns.GEMM_F16_IR, inputs=patterns.GEMM_F16_INPUTS, name='gemm_f16')
     a, b = (t.to(dev) for t in workloads.gemm_inputs(seed, n))
     c = torch.empty(n, n, dtype=torch.float16, device=dev)
-    sec = time_graph(torch, capi, lambda: op(a, b, out=c), steps, warmup)
+    sec = time_graph(torch, capi, lambda: op(a, b, out=c), steps, warmup, warm_ms=40.0)
     tflops = 2.0 * n * n * n / sec / 1e12
     return {'workload': f'fp16 GEMM M=N=K={n} (fp32 accumulate)', 'us_per_launch': sec * 1e6, 'tflops': tflops,
             'roofline_bound': 'mfma', 'roofline_frac': tflops / MFMA_F16_PEAK_TFLOPS}
