@@ -45,7 +45,7 @@ def parse_args():
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-extra', action='store_true', help='headline workload only')
     ap.add_argument('--no-decode', action='store_true', help='skip the 32-layer decode leg')
-    ap.add_argument('--decode-cpu-steps', type=int, default=2, help='decode steps timed on the CPU oracle (0 = skip)')
+    ap.add_argument('--decode-cpu-steps', type=int, default=4, help='decode steps timed on the CPU oracle (0 = skip)')
     ap.add_argument('--att-parts', type=int, default=8, help='blocks per head of the decode attention (1 = unsplit)')
     ap.add_argument('--seed', type=int, default=0)
     return ap.parse_args()
@@ -245,6 +245,58 @@ def cpu_baseline_gemv(workloads, K, N, M, seed, budget_s=15.0):
                       f'{t["seconds"] * 1e3:.1f} ms per run'}
 
 
+def cpu_time_program(ir, inputs, tensors, budget_s):
+    """Seconds per run of an einstein_v2 program on the CPU oracle (rank-striding thread pool, reference's flags)."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    return CpuModule(parse_program(ir, inputs), nranks=256).time(budget_s=budget_s, **tensors)
+
+
+def cpu_baseline_extras(workloads, seed):
+    """CPU oracle beside the other configurations, each on a bounded sample: workload name -> cpu_baseline object."""
+    import numpy as np
+    from antares_amd.autort import patterns
+    from oracle import hot_ops
+    out = {}
+    # int4 GEMM, M = 64: the same program as the headline with 64 rows of x
+    K, N, M, n_sample = 4096, 11008, 64, 2752          # a quarter of the columns: the loop nest costs the same per column
+    p = workloads.w4_problem(seed, M, K, n_sample)
+    t = cpu_time_program(patterns.W4A16_IR, patterns.W4A16_INPUTS,
+                         dict(x=p['x'].numpy(), qweight=p['qweight'].numpy().view('int8'), scales=p['scales'].numpy(),
+                              qzeros=p['qzeros'].numpy().view('int8')), budget_s=2.0)
+    by = workloads.w4_bytes(M, K, n_sample)
+    out[f'int4 g128 GEMM M={M} K={K} N={N}'] = {
+        'value': round(by / t['seconds'] / 1e9, 4), 'unit': 'GB/s', 'cores': t['threads'], 'kind': 'port',
+        'sample': f'{t["runs"]} timed run(s) of the same GEMM on {n_sample} of the {N} columns, {t["seconds"] * 1e3:.0f} ms per run'}
+    # fp16 GEMM: a 1024^3 corner of the 4096^3 problem (the loop nest does 2 flop per step whatever the size)
+    n = 1024
+    a, b = workloads.gemm_inputs(seed, n)
+    t = cpu_time_program(patterns.GEMM_F16_IR, patterns.GEMM_F16_INPUTS, dict(a=a.numpy(), b=b.numpy()), budget_s=4.0)
+    out['fp16 GEMM M=N=K=4096 (fp32 accumulate)'] = {
+        'value': round(2.0 * n ** 3 / t['seconds'] / 1e12, 5), 'unit': 'TFLOP/s', 'cores': t['threads'], 'kind': 'port',
+        'sample': f'{t["runs"]} timed run(s) of the same program at M=N=K={n}, {t["seconds"] * 1e3:.0f} ms per run'}
+    # sigmoid at full size
+    n = 4_096_000
+    x = workloads.sigmoid_input(seed, n)
+    t = cpu_time_program('sigmoid_f32[N] = 1 - 1 / (1 + data[N].call(strs.exp))', ['data=float32[N:4096000]'], dict(data=x.numpy()),
+                         budget_s=2.0)
+    out[f'sigmoid f32 N={n}'] = {'value': round(8 * n / t['seconds'] / 1e9, 3), 'unit': 'GB/s', 'cores': t['threads'], 'kind': 'port',
+                                 'sample': f'{t["runs"]} timed run(s) at full size, {t["seconds"] * 1e3:.2f} ms per run'}
+    # partition at full size: the plain-C restatement of the sample's three steps, one thread
+    n = 16_777_216
+    v = workloads.partition_input(seed, n).numpy()
+    hot_ops.sort_even_first_i32(v)
+    t0 = time.perf_counter()
+    runs = 3
+    for _ in range(runs):
+        hot_ops.sort_even_first_i32(v)
+    sec = (time.perf_counter() - t0) / runs
+    out[f'stable even-first partition int32 N={n}'] = {
+        'value': round(8 * n / sec / 1e9, 3), 'unit': 'GB/s', 'cores': 1, 'kind': 'port',
+        'sample': f'{runs} timed run(s) at full size after 1 warm-up, {sec * 1e3:.1f} ms per run'}
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -288,6 +340,11 @@ def main():
         for fn in (bench_sigmoid, bench_partition):
             r = fn(torch, autort, capi, workloads, args.steps, args.warmup, args.seed)
             extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
+        if not args.no_cpu:
+            cpu = cpu_baseline_extras(workloads, args.seed)
+            for e in extra:
+                if e['workload'] in cpu:
+                    e['cpu_baseline'] = cpu[e['workload']]
         result['extra'] = extra
     if not args.no_decode:
         result['decode'] = bench_decode(torch, autort, capi, args.seed, cpu_steps=0 if args.no_cpu else args.decode_cpu_steps,
