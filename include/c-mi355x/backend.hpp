@@ -81,43 +81,51 @@ namespace ab {
     return m;
   }
 
+  // What the evaluator keeps per kernel is opaque to it (it only hands the vector back to launchKernel), so the
+  // launch description is one record behind the first element.
+  struct KernelLaunch {
+    art_func* fn = nullptr;
+    unsigned grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
+    int first_sizing_arg = 0;                    // `$`: position of the first integer argument that sizes the grid (0: fixed grid)
+    long grid_factor = 1;                        // `$$`
+    std::vector<long> elements_per_block;        // `$0`, `$1`, ...: negative = that argument does not count
+  };
+
   inline std::vector<void*> moduleGetFunction(const void* hModule, const std::string& fname,
                                               const std::unordered_map<std::string, int>& threads) {   // backend.hpp:172
-    auto query = [&](const std::string& axis, long defval = 1) -> void* {
-      auto it = threads.find(axis);
-      return (void*)(it == threads.end() ? defval : (long)it->second);
+    auto extent = [&threads](const std::string& key, long fallback) {
+      const auto it = threads.find(key);
+      return it == threads.end() ? fallback : (long)it->second;
     };
-    art_func* f = nullptr;
-    ART_OK(art_get_function((art_module*)hModule, fname.c_str(), &f));
-    std::vector<void*> fdata = {f, query("blockIdx.x"), query("blockIdx.y"), query("blockIdx.z"),
-                                query("threadIdx.x"), query("threadIdx.y"), query("threadIdx.z")};
-    if (void* first = query("$", 0)) {                                   // dynamic grid: $$ * prod(ceil(arg_i / $i))
-      fdata.push_back(first);
-      fdata.push_back(query("$$", 1));
-      for (int i = 0;; ++i) {
-        void* item = query("$" + std::to_string(i), 0);
-        if (!item) break;
-        fdata.push_back(item);
-      }
+    KernelLaunch* k = new KernelLaunch;          // lives as long as the module: the reference never unloads either
+    ART_OK(art_get_function((art_module*)hModule, fname.c_str(), &k->fn));
+    static const char* const axes[3] = {"x", "y", "z"};
+    for (int a = 0; a < 3; ++a) {
+      k->grid[a] = (unsigned)extent(std::string("blockIdx.") + axes[a], 1);
+      k->block[a] = (unsigned)extent(std::string("threadIdx.") + axes[a], 1);
     }
-    return fdata;
+    k->first_sizing_arg = (int)extent("$", 0);
+    if (k->first_sizing_arg) {                   // grid.x = $$ * prod(ceil(argument_i / $i)), worked out at launch
+      k->grid_factor = extent("$$", 1);
+      for (long per; (per = extent("$" + std::to_string(k->elements_per_block.size()), 0)) != 0;) k->elements_per_block.push_back(per);
+    }
+    return {k};
   }
 
   inline void launchKernel(std::vector<void*>& hFunc, const std::vector<void*>& krnl_args, void* stream) {   // backend.hpp:199
-    if (hFunc.size() > 7) {
-      long blocks = (long)hFunc[8];
-      for (size_t i = 9; i < hFunc.size(); ++i) {
-        const long val = (long)hFunc[i];
-        if (val < 0) continue;
-        const int arg = (int)(long)krnl_args[i - 9 + (long)hFunc[7]];
-        blocks *= (arg + val - 1) / val;
+    const KernelLaunch& k = *(const KernelLaunch*)hFunc[0];
+    unsigned grid_x = k.grid[0];
+    if (k.first_sizing_arg) {
+      long blocks = k.grid_factor;
+      for (size_t i = 0; i < k.elements_per_block.size(); ++i) {
+        const long per = k.elements_per_block[i];
+        if (per > 0) blocks *= ((long)(int)(long)krnl_args[k.first_sizing_arg + i] + per - 1) / per;
       }
-      hFunc[1] = (void*)blocks;
-      if (!blocks) return;
+      if (blocks == 0) return;                   // nothing to do at these sizes
+      grid_x = (unsigned)blocks;
     }
     // one 64-bit slot per argument, exactly what the evaluator hands over (execute_module.hpp:340-352)
-    ART_OK(art_launch((art_func*)hFunc[0], (unsigned)(long)hFunc[1], (unsigned)(long)hFunc[2], (unsigned)(long)hFunc[3],
-                      (unsigned)(long)hFunc[4], (unsigned)(long)hFunc[5], (unsigned)(long)hFunc[6], 0, stream,
+    ART_OK(art_launch(k.fn, grid_x, k.grid[1], k.grid[2], k.block[0], k.block[1], k.block[2], 0, stream,
                       (const uint64_t*)krnl_args.data(), (int)krnl_args.size()));
   }
 
