@@ -5,6 +5,11 @@ Restates the forward pass of samples/05_llama2_7b_int4.py:146-177 for the
 benchmark configuration (packed int4 linears with zero points, fp16 everything
 else) out of the oracle's own operators (hot_ops.c).  Every operator output is
 rounded to fp16, as each GPU operator rounds its output.
+
+Pinned by tests/test_oracle.py::test_decode_oracle_against_independent_float64_restatement:
+ten positions against a torch float64 forward pass written from the sample's text
+with library routines only (dense matmul, silu, softmax, rotate_half), logits,
+greedy tokens and cache rows.
 """
 from __future__ import annotations
 

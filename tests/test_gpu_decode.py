@@ -124,3 +124,57 @@ def test_prefill_of_a_whole_prompt_matches_the_oracle_token_by_token(T):
     assert np.allclose(got2, want2, **LOGIT_TOL), np.abs(got2 - want2).max()
     with pytest.raises(ValueError):
         dec.prefill(prompt[:3].to(dec.dev))
+
+
+@pytest.mark.parametrize('graph', [False, True])
+def test_full_width_decode_matches_the_oracle(graph):
+    """The benchmark model's widths (dim 4096, 32 heads, ffn 11008, vocab 32000, cache of 384 rows, attention over
+    8 blocks per head) on two layers, with the caches pre-filled so that positions 0, 1, 200 and 383 run with their
+    real lengths: logits, the device's greedy token and the cache rows against the oracle, eager and as a replayed graph."""
+    from antares_amd.llama import LlamaConfig, LlamaInt4Decoder, random_weights
+    from oracle.llama_ref import LlamaRef
+    cfg = LlamaConfig(n_layers=2)
+    assert (cfg.dim, cfg.n_heads, cfg.ffn, cfg.vocab, cfg.max_seq) == (4096, 32, 11008, 32000, 384)
+    w = random_weights(cfg, seed=9)
+    # the oracle's projections on its thread pool (bit-identical to the plain-C loop, 2 s instead of 14 s per step)
+    from antares_amd.autort import patterns
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    mod = CpuModule(parse_program(patterns.W4A16_IR, patterns.W4A16_INPUTS), nranks=256, fast_math=False)
+
+    def linear(x, lin):
+        return mod(x=np.ascontiguousarray(x), qweight=lin['qweight'].numpy().view('int8'), scales=lin['scales'].numpy(),
+                   qzeros=lin['qzeros'].numpy().view('int8'))['y']
+    ref = LlamaRef(cfg, w, linear=linear)
+    dec = LlamaInt4Decoder(cfg, w, fused=True, att_parts=8)
+    g = torch.Generator().manual_seed(17)
+    keys = (torch.randn(cfg.n_layers, cfg.max_seq, cfg.dim, generator=g) * 0.5).half()
+    vals = (torch.randn(cfg.n_layers, cfg.max_seq, cfg.dim, generator=g) * 0.5).half()
+    ref.key_cache[:], ref.val_cache[:] = keys.numpy(), vals.numpy()
+    dec.key_cache.copy_(keys)
+    dec.val_cache.copy_(vals)
+    if graph:
+        kc, vc = dec.key_cache.clone(), dec.val_cache.clone()
+        dec.reset(0, 0)
+        dec.capture(greedy=True)
+        dec.key_cache.copy_(kc)           # the recording ran the step once at position 0
+        dec.val_cache.copy_(vc)
+    for pos, token in [(0, 11), (1, 31999), (200, 4242), (383, 0)]:
+        print(f'[case] full width graph={graph} pos={pos}', flush=True)
+        want = ref.forward(token, pos).astype(np.float32)
+        dec.reset(token, pos)
+        if graph:
+            dec.graph.replay()
+            torch.cuda.synchronize()
+            got = dec.logits.float().cpu().numpy()
+        else:
+            got = dec.step().float().cpu().numpy()
+        assert np.allclose(got, want, **LOGIT_TOL), (pos, np.abs(got - want).max())
+        if graph:
+            top2 = np.sort(want)[-2:]
+            assert int(dec.pos.item()) == pos + 1
+            if top2[1] - top2[0] > 0.1:
+                assert int(dec.token.item()) == int(np.argmax(want))
+        for l in range(cfg.n_layers):
+            assert np.allclose(dec.key_cache[l, pos].float().cpu().numpy(), ref.key_cache[l, pos].astype(np.float32), rtol=2e-2, atol=2e-2)
+            assert np.allclose(dec.val_cache[l, pos].float().cpu().numpy(), ref.val_cache[l, pos].astype(np.float32), rtol=2e-2, atol=2e-2)

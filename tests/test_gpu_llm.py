@@ -237,3 +237,56 @@ def test_position_past_the_cache_touches_nothing(autort):
     autort.ops.attention_rope_f16(qkv, inv, key_cache, val_cache, att_f, out, extra=[pos])
     assert torch.isfinite(out).all()
     assert torch.equal(backing_k[ROWS:], before_k[ROWS:]) and torch.equal(backing_v[ROWS:], before_v[ROWS:])
+
+
+@pytest.mark.usefixtures('oracle_built')
+@pytest.mark.parametrize('parts', [1, 4, 8])
+@pytest.mark.parametrize('pos', [0, 31, 130, 255, 256, 257, 383])
+def test_fused_decode_attention_against_the_oracle(parts, pos):
+    """The kernels the decode step runs - attention_rope_f16 (parts == 1) and attention_rope_split_f16 merged by
+    gemv_w4a16_attn - against the oracle's rotary + attention (+ int4 projection) at the full head count, at
+    positions on both sides of every 256-position round of the kernel, including the cache rows they write."""
+    import autort
+    from antares_amd import workloads
+    from oracle import hot_ops
+    dev = autort.device()
+    H, D, S = 32, 128, 384
+    g = torch.Generator().manual_seed(1000 * parts + pos)
+    note(f'fused attention vs oracle parts={parts} pos={pos}')
+    qkv = torch.randn(3 * H * D, generator=g).half()
+    inv = (1.0 / (10000 ** (torch.arange(0, D, 2).float() / D))).half()
+    inv_freq = torch.cat([inv, inv])
+    kc = (torch.randn(S, H * D, generator=g) * 0.5).half()
+    vc = torch.randn(S, H * D, generator=g).half()
+    att_f = 1 / math.sqrt(D)
+    # oracle: rotate q and k, put k and v into row `pos`, attend over rows 0..pos
+    q, k, v = qkv[:H * D].numpy(), qkv[H * D:2 * H * D].numpy(), qkv[2 * H * D:].numpy()
+    q_rot = hot_ops.rotary(q.reshape(H, 2, D // 2), inv_freq.numpy(), pos)
+    k_rot = hot_ops.rotary(k.reshape(H, 2, D // 2), inv_freq.numpy(), pos)
+    kc_want, vc_want = kc.numpy().copy(), vc.numpy().copy()
+    kc_want[pos], vc_want[pos] = k_rot.reshape(-1), v
+    att_want = hot_ops.attention(q_rot, kc_want[:pos + 1].reshape(pos + 1, H, D), vc_want[:pos + 1].reshape(pos + 1, H, D), att_f)
+
+    kd, vd = kc.to(dev), vc.to(dev)
+    att_f_t = torch.tensor([att_f], dtype=torch.float32, device=dev)
+    pos_t = torch.tensor([pos], dtype=torch.int32, device=dev)
+    if parts == 1:
+        att = torch.empty(H, D, dtype=torch.float16, device=dev)
+        autort.ops.attention_rope_f16(qkv.to(dev), inv_freq.to(dev), kd, vd, att_f_t, att, extra=[pos_t])
+        assert np.allclose(att.float().cpu().numpy(), att_want.astype(np.float32), **FP16_TOL)
+    else:
+        p = workloads.w4_problem(11, 1, H * D, 4096)
+        res = torch.randn(4096, generator=g).half()
+        partial = torch.full((H, parts, 132), float('nan'), dtype=torch.float32, device=dev)
+        autort.ops.attention_rope_split_f16(qkv.to(dev), inv_freq.to(dev), kd, vd, att_f_t, partial, extra=[pos_t])
+        y = torch.empty(4096, dtype=torch.float16, device=dev)
+        autort.ops.gemv_w4a16_attn(partial, p['qweight'].to(dev), p['scales'].to(dev), p['qzeros'].to(dev), y, residual=res.to(dev))
+        proj = hot_ops.gemm_w4a16(att_want.reshape(1, -1), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy()).reshape(-1)
+        y_want = (proj.astype(np.float32) + res.numpy().astype(np.float32)).astype(np.float16)
+        assert np.allclose(y.float().cpu().numpy(), y_want.astype(np.float32), **FP16_TOL)
+    # cache: row `pos` rewritten, every other row untouched (bit for bit)
+    kg, vg = kd.cpu().numpy(), vd.cpu().numpy()
+    assert np.allclose(kg[pos].astype(np.float32), kc_want[pos].astype(np.float32), **FP16_TOL)
+    assert np.array_equal(vg[pos], vc_want[pos])
+    keep = np.arange(S) != pos
+    assert np.array_equal(kg[keep], kc.numpy()[keep]) and np.array_equal(vg[keep], vc.numpy()[keep])

@@ -2,6 +2,8 @@
 a dropped term / wrong nibble order / transposed operand would break, and the
 agreement of its two independent halves (plain-C hot_ops vs the loop nests
 emitted from the IR)."""
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -264,3 +266,130 @@ def test_attention_closed_forms():
     # q = 0 -> uniform weights -> mean of v ; S = 1 -> v[0]
     assert np.allclose(hot_ops.attention(np.zeros_like(q), k, v, f), v.mean(0), rtol=1e-5, atol=1e-5)
     assert np.allclose(hot_ops.attention(q, k[:1], v[:1], f), v[0], rtol=1e-6, atol=1e-6)
+
+
+# ---------------------------------------------------------------- decode step
+def _dense_f64(lin):
+    """Packed int4 linear -> dense float64 [K, N] with plain torch indexing (no oracle code)."""
+    qw, s, qz = lin['qweight'], lin['scales'].double(), lin['qzeros']
+    K, N = qw.shape[0] * 2, qw.shape[1]
+    q = torch.empty(K, N, dtype=torch.float64)
+    q[0::2] = (qw & 15).double()
+    q[1::2] = (qw >> 4).double()
+    z = torch.empty(K // 128, N, dtype=torch.float64)
+    z[:, 0::2] = (qz & 15).double()
+    z[:, 1::2] = (qz >> 4).double()
+    return (q - z.repeat_interleave(128, 0)) * s.repeat_interleave(128, 0)
+
+
+class TorchDecodeF64:
+    """The forward pass of samples/05_llama2_7b_int4.py:146-177 written from the sample's text with torch float64
+    tensors and library routines (dense matmul, torch.nn.functional.silu, torch.softmax, the Hugging Face
+    x*cos + rotate_half(x)*sin), sharing no code with oracle/llama_ref.py or oracle/hot_ops.c."""
+
+    def __init__(self, cfg, w):
+        self.cfg = cfg
+        self.embed = w['embed'].double()
+        self.final_norm = w['final_norm'].double()
+        self.lm_head = _dense_f64(w['lm_head'])
+        self.layers = [{'att_norm': lw['att_norm'].double(), 'ffn_norm': lw['ffn_norm'].double(),
+                        'qkv': _dense_f64(lw['qkv']), 'o': _dense_f64(lw['o']),
+                        'gate_up': _dense_f64(lw['gate_up']), 'down': _dense_f64(lw['down'])} for lw in w['layers']]
+        D = cfg.head_dim
+        inv = (1.0 / (cfg.rope_base ** (torch.arange(0, D, 2).float() / D))).to(torch.float16)     # sample :125
+        self.inv_freq = torch.cat([inv, inv]).double()                                             # sample :126
+        self.keys = torch.zeros(cfg.n_layers, cfg.max_seq, cfg.n_heads, D, dtype=torch.float64)
+        self.vals = torch.zeros_like(self.keys)
+
+    def norm(self, x, w):                                         # sample :128-131
+        return x * torch.rsqrt((x * x).mean() + self.cfg.rms_eps) * w
+
+    def rope(self, x, pos):                                       # [H, D]
+        half = x.shape[-1] // 2
+        ang = pos * self.inv_freq
+        rotate_half = torch.cat([-x[:, half:], x[:, :half]], dim=-1)
+        return x * torch.cos(ang) + rotate_half * torch.sin(ang)
+
+    def forward(self, token, pos):
+        cfg = self.cfg
+        d, H, D = cfg.dim, cfg.n_heads, cfg.head_dim
+        x = self.embed[token]                                      # :147
+        for l, lw in enumerate(self.layers):
+            xb = self.norm(x, lw['att_norm'])                      # :150
+            q, k, v = (xb @ lw['qkv']).split(d)                    # :151-153, columns q | k | v in this build
+            self.keys[l, pos] = self.rope(k.view(H, D), pos)       # :158
+            self.vals[l, pos] = v.view(H, D)
+            q = self.rope(q.view(H, D), pos)                       # :157
+            ks, vs = self.keys[l, :pos + 1], self.vals[l, :pos + 1]                      # :162-163
+            att = torch.softmax(torch.einsum('hd,shd->hs', q, ks) / math.sqrt(D), dim=-1)   # samples/03_llama_tiny.py:94-99
+            xb = torch.einsum('hs,shd->hd', att, vs).reshape(d)    # :165
+            x = x + xb @ lw['o']                                   # :167-168
+            xb = self.norm(x, lw['ffn_norm'])                      # :169
+            gate, up = (xb @ lw['gate_up']).split(cfg.ffn)         # f1 = gate_proj, f3 = up_proj
+            x = x + (torch.nn.functional.silu(gate) * up) @ lw['down']                   # :171-173
+        return self.norm(x, self.final_norm) @ self.lm_head        # :175-176
+
+
+def test_decode_oracle_against_independent_float64_restatement():
+    """LlamaRef.forward (the checker of the decode parity tests) against TorchDecodeF64 over 10 positions of a
+    prompt-then-greedy run.  A swapped gate/up, a residual in the wrong place, a missing final norm, a wrong
+    rotary pairing or cache row would each move the logits by O(1)."""
+    from antares_amd.llama import LlamaConfig, random_weights
+    from oracle.llama_ref import LlamaRef
+    cfg = LlamaConfig(n_layers=2, dim=512, n_heads=4, ffn=1024, vocab=1024, max_seq=32)
+    w = random_weights(cfg, seed=3)
+    ref, ind = LlamaRef(cfg, w), TorchDecodeF64(cfg, w)
+    prompt = [5, 77, 901]
+    token = prompt[0]
+    worst = 0.0
+    for pos in range(10):
+        got = ref.forward(token, pos).astype(np.float64)
+        want = ind.forward(token, pos).numpy()
+        assert want.std() > 0.3                                     # the logits are not degenerate
+        worst = max(worst, np.abs(got - want).max())
+        # the oracle rounds every operator output to fp16; the restatement rounds nothing
+        assert np.allclose(got, want, rtol=2e-2, atol=2e-2), (pos, np.abs(got - want).max())
+        top2 = np.sort(want)[-2:]
+        if top2[1] - top2[0] > 0.05:
+            assert int(np.argmax(got)) == int(np.argmax(want)), pos
+        token = prompt[pos + 1] if pos + 1 < len(prompt) else int(np.argmax(want))
+        for l in range(cfg.n_layers):                               # the cache rows both sides wrote at this position
+            assert np.allclose(ref.key_cache[l, pos].astype(np.float64), ind.keys[l, pos].reshape(-1).numpy(), rtol=2e-2, atol=2e-2)
+            assert np.allclose(ref.val_cache[l, pos].astype(np.float64), ind.vals[l, pos].reshape(-1).numpy(), rtol=2e-2, atol=2e-2)
+    assert worst < 2e-2
+
+
+def test_decode_oracle_restatement_detects_plausible_mistakes():
+    """The check above has teeth: each of these mis-readings of the sample moves the logits far outside its tolerance."""
+    from antares_amd.llama import LlamaConfig, random_weights
+    cfg = LlamaConfig(n_layers=2, dim=512, n_heads=4, ffn=1024, vocab=1024, max_seq=32)
+    w = random_weights(cfg, seed=3)
+    good = TorchDecodeF64(cfg, w)
+    base = [good.forward(t, p).numpy() for p, t in enumerate([5, 77, 901])]
+
+    class SwappedGate(TorchDecodeF64):
+        def forward(self, token, pos):
+            for lw in self.layers:
+                gu = lw['gate_up']
+                lw['gate_up'] = torch.cat([gu[:, self.cfg.ffn:], gu[:, :self.cfg.ffn]], dim=1)
+            try:
+                return super().forward(token, pos)
+            finally:
+                for lw in self.layers:
+                    gu = lw['gate_up']
+                    lw['gate_up'] = torch.cat([gu[:, self.cfg.ffn:], gu[:, :self.cfg.ffn]], dim=1)
+
+    class NoFinalNorm(TorchDecodeF64):
+        def norm(self, x, w):
+            return x if w is self.final_norm else super().norm(x, w)
+
+    class InterleavedRope(TorchDecodeF64):
+        def rope(self, x, pos):
+            H, D = x.shape
+            z = torch.view_as_complex(x.reshape(H, D // 2, 2).contiguous()) * torch.polar(torch.ones(D // 2, dtype=torch.float64), pos * self.inv_freq[:D // 2])
+            return torch.view_as_real(z).reshape(H, D)
+
+    for cls in (SwappedGate, NoFinalNorm, InterleavedRope):
+        bad = cls(cfg, w)
+        outs = [bad.forward(t, p).numpy() for p, t in enumerate([5, 77, 901])]
+        assert max(np.abs(a - b).max() for a, b in zip(outs, base)) > 0.1, cls.__name__
