@@ -90,7 +90,9 @@ class ExportedOp:
         self._module: Optional[capi.Module] = None
         self._image: Optional[bytes] = None
         from . import patterns
-        self.fast_path = patterns.match(self.fused)
+        hit = patterns.match(self.fused)
+        # hand-written kernel for this program, if any, and which of the caller's tensors plays which part in it
+        self.fast_path, self.fast_roles = hit if hit is not None else (None, {})
         # per-call bookkeeping that does not depend on the call
         self._wanted_dtype = {}
         for n in list(self.declared) + list(self.fresh_outputs):

@@ -2,29 +2,42 @@
 
 A program is recognised by the canonical text of its fused statements (tensor
 and axis names replaced by order of appearance), so the user's spelling of
-names does not matter.  A handler returns True when it ran the operator, or
-False to leave it to the generic lowering (shapes it does not cover).
+names does not matter.  The part each of the caller's tensors plays is taken
+from that same order: ``match`` returns the handler together with a map from
+the registered program's tensor names (the handler's vocabulary: ``x``,
+``qweight`` ...) to the caller's names.  A handler returns True when it ran the
+operator, or False to leave it to the generic lowering (shapes it does not
+cover).
 """
 from __future__ import annotations
 
-from typing import Callable, Dict, Optional
+from typing import Callable, Dict, Optional, Tuple
 
 from ctypes import c_void_p
+
+import torch
 
 from ..ir import Graph, fuse_elementwise, parse_program
 from ..runtime import capi
 
-_TABLE: Dict[str, Callable] = {}
+_TABLE: Dict[str, Tuple[Callable, list]] = {}      # canonical key -> (handler, the registered program's tensor order)
 
 
 def register(ir: str, inputs, handler: Callable):
-    key = fuse_elementwise(parse_program(ir, inputs)).canonical_key()
-    _TABLE[key] = handler
+    g = fuse_elementwise(parse_program(ir, inputs))
+    key = g.canonical_key()
+    _TABLE[key] = (handler, g.canonical_tensor_order())
     return key
 
 
-def match(fused: Graph) -> Optional[Callable]:
-    return _TABLE.get(fused.canonical_key())
+def match(fused: Graph) -> Optional[Tuple[Callable, Dict[str, str]]]:
+    """(handler, roles) for a recognised program, else None.  ``roles`` maps the registered program's tensor names
+    to the names the caller's program uses for the tensors in the same places."""
+    hit = _TABLE.get(fused.canonical_key())
+    if hit is None:
+        return None
+    handler, registered = hit
+    return handler, dict(zip(registered, fused.canonical_tensor_order()))
 
 
 # ---------------------------------------------------------------------------
@@ -41,26 +54,10 @@ def _gptq_inputs(xdt: str, sdt: str):
     return [f'input0={xdt}[S:4096]', 'qweight=int32[L:512, N:12288]', f'scales={sdt}[K:32, N:12288]']
 
 
-def _gptq_roles(op):
-    """Which declared tensor is x, qweight, scales and the output (the ABI order is by name; roles go by dtype and
-    rank).  Worked out once per operator."""
-    roles = getattr(op, '_gptq_roles', None)
-    if roles is None:
-        g = op.fused
-        names = {n: g.tensors[n] for n in g.abi_inputs}
-        q_name = next(n for n, t in names.items() if t.dtype == 'int32')
-        x_name = next(n for n, t in names.items() if len(t.shape) == 1)
-        s_name = next(n for n in names if n not in (q_name, x_name))
-        roles = (x_name, q_name, s_name, g.abi_outputs[0], int(names[x_name].dtype == 'float16'),
-                 int(names[s_name].dtype == 'float16'))
-        op._gptq_roles = roles
-    return roles
-
-
 def _gptq_handler(op, bound, env, stream) -> bool:
-    x_name, q_name, s_name, out_name, x_f16, s_f16 = _gptq_roles(op)
-    out = bound[out_name]
-    x, q, s = bound[x_name], bound[q_name], bound[s_name]
+    r = op.fast_roles
+    x, q, s, out = bound[r['input0']], bound[r['qweight']], bound[r['scales']], bound[r['my_result']]
+    x_f16, s_f16 = int(x.dtype == torch.float16), int(s.dtype == torch.float16)
     K, N = x.shape[0], q.shape[1]
     qp = q.data_ptr()
     if K % 128 or N % 4 or q.shape[0] * 8 != K or s.shape[0] * 128 != K or qp % 16:
@@ -89,7 +86,8 @@ W4A16_INPUTS = ['x=float16[M:1, K:4096]', 'qweight=int8[KH:2048, N:11008]', 'sca
 
 
 def _w4a16_handler(op, bound, env, stream) -> bool:
-    x, q, s, z, y = bound['x'], bound['qweight'], bound['scales'], bound['qzeros'], bound['y']
+    r = op.fast_roles
+    x, q, s, z, y = bound[r['x']], bound[r['qweight']], bound[r['scales']], bound[r['qzeros']], bound[r['y']]
     M, K = x.shape
     N = q.shape[1]
     if K % 128 or N % 16 or q.shape[0] * 2 != K or s.shape[0] * 128 != K or z.shape[1] * 2 != N \
@@ -119,7 +117,8 @@ GEMM_F16_INPUTS = ['a=float16[M:4096, K:4096]', 'b=float16[K:4096, N:4096]']
 
 
 def _gemm_f16_handler(op, bound, env, stream) -> bool:
-    a, b, c = bound['a'], bound['b'], bound['c']
+    r = op.fast_roles
+    a, b, c = bound[r['a']], bound[r['b']], bound[r['c']]
     M, K = a.shape
     N = b.shape[1]
     if N % 8 or K % 64 or a.data_ptr() % 16 or b.data_ptr() % 16 or c.data_ptr() % 16:

@@ -15,9 +15,13 @@
 //     v_cvt_f32_ubyte0..3 turns each byte into a float, one FMA per weight: 2.4 VALU operations per weight;
 //   * the k lanes of a block meet in LDS; the owner of a column applies scale and the fixed zero point 8 once
 //     per (group, column): s * (acc - 8 * sum(x));
-//   * the K-splits of a column meet in one returning 64-bit atomic: a fixed-point partial sum (steps of 2^-22) with an
-//     arrival count in the top byte and a count of non-finite partial sums in the bottom one.  Integer addition is associative, so the result does not depend on the
-//     arrival order; the block that sees count == splits - 1 holds the total, writes y and clears the slot.
+//   * the K-splits of a column meet in returning 64-bit atomics: a fixed-point partial sum with an arrival count in
+//     the top byte and a count of non-finite partial sums in the bottom one.  Integer addition is associative, so
+//     the result does not depend on the arrival order; the block that sees count == splits - 1 holds the total,
+//     writes y and clears the slot.  One slot (steps of 2^-22) is all an fp16 result needs.  An fp32 result gets a
+//     second slot for what the first one rounds away (first slot in steps of 2^-8 up to 2^39 / splits, second in steps of 2^-58): both atomics of a block are issued together,
+//     and the block that completes the first slot usually completes the second as well (else it re-reads it until
+//     the adds that are still in flight have landed), so the sum of the partial sums is exact wherever fp32 is.
 #include "art_common.h"
 
 namespace {
@@ -46,6 +50,22 @@ __device__ __forceinline__ long long to_fixed(float r, int splits) {
 __device__ __forceinline__ float from_fixed(long long total) {
   return (total & 255) ? __builtin_nanf("") : (float)total * (1.f / kFix);
 }
+
+// fp32 results take two slots.  First slot: multiples of 256 in units of 2^-16 (steps of 2^-8, low byte = count of
+// rejected partial sums as above), |r| < 2^39 / splits.  Second slot: what the first rounds away, in units of 2^-58
+// (|r * 2^8| below 2^23 has a fraction, anything larger is an integer already).  Together: every partial sum with
+// 2^-34 <= |r| < 2^39 / splits travels exactly, smaller ones to within 2^-59.
+__device__ __forceinline__ long long to_fixed_wide(float r, int splits) {
+  const float limit = 549755813888.f / (float)splits;
+  return fabsf(r) < limit ? __float2ll_rn(r * 256.f) * 256 : 1LL;
+}
+__device__ __forceinline__ long long to_fixed_rest(float r, int splits) {
+  const float limit = 549755813888.f / (float)splits;
+  if (!(fabsf(r) < limit)) return 0LL;
+  const float t = r * 256.f;                                  // exact
+  return __float2ll_rn((t - rintf(t)) * 1125899906842624.f);  // (t - rint t) is exact, |.| <= 0.5; times 2^50
+}
+constexpr int kMaxSpin = 1 << 22;
 
 template <class T> __device__ __forceinline__ float ldf(const T* p, size_t i) { return (float)p[i]; }
 
@@ -125,13 +145,31 @@ __global__ __launch_bounds__(kThreads) void gemv_gptq_kernel(const XT* __restric
     y[col] = (XT)res;
     return;
   }
-  // one returning atomic: [arrival count : 8][fixed-point sum : 56]
+  // returning atomics: [arrival count : 8][fixed-point sum : 56]
+  constexpr bool exact = sizeof(XT) == 4;              // fp32 result: second slot for the rounded-away part
   unsigned long long* slot = slots + col;
-  const long long mine = (1LL << 56) + to_fixed(res, splits);
+  unsigned long long* slot_lo = slots + N + col;
+  const long long mine = (1LL << 56) + (exact ? to_fixed_wide(res, splits) : to_fixed(res, splits));
+  const long long mine_lo = (1LL << 56) + to_fixed_rest(res, splits);
+  long long old_lo = 0;
+  if (exact) old_lo = (long long)__hip_atomic_fetch_add(slot_lo, (unsigned long long)mine_lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const long long old = (long long)__hip_atomic_fetch_add(slot, (unsigned long long)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (((old + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
     const long long total = old + mine - ((long long)splits << 56);
-    y[col] = (XT)from_fixed(total);
+    if (!exact) {
+      y[col] = (XT)from_fixed(total);
+    } else {
+      // every other block issued its add to the second slot before (or with) the one this block has just seen
+      // land in the first: the count there reaches `splits` within a memory round trip.  The wait is bounded.
+      long long lo = old_lo + mine_lo;
+      for (int spin = 0; ((lo + (1LL << 55)) >> 56) != (long long)splits && spin < kMaxSpin; ++spin)
+        lo = (long long)__hip_atomic_load(slot_lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool complete = ((lo + (1LL << 55)) >> 56) == (long long)splits;
+      lo -= (long long)splits << 56;
+      const double v = (double)(total >> 8) * (1.0 / 256.0) + (double)lo * (1.0 / 288230376151711744.0);     // 2^-8, 2^-58
+      y[col] = (XT)(((total & 255) || !complete) ? __builtin_nanf("") : (float)v);
+      *slot_lo = 0ull;
+    }
     *slot = 0ull;                       // ready for the next launch (stream order makes this visible)
   }
 }
@@ -143,7 +181,7 @@ int launch(const void* x, const void* qw, const void* sc, void* y, int K, int N,
   ART_REQUIRE(splits <= 127, "art_gemv_gptq: K too large (%d)", K);
   art::Workspace& ws = art::workspace();
   ART_REQUIRE(ws.base != nullptr, "art_gemv_gptq: call art_init first");
-  ART_REQUIRE(art::kSlotOffset + (size_t)N * 8 <= art::kScratchOffset, "art_gemv_gptq: N too large (%d)", N);
+  ART_REQUIRE(art::kSlotOffset + (size_t)N * 16 <= art::kScratchOffset, "art_gemv_gptq: N too large (%d)", N);
   unsigned long long* slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(ws.base) + art::kSlotOffset);
   gemv_gptq_kernel<XT, ST><<<dim3(tiles, splits), dim3(kThreads), 0, stream>>>(
       (const XT*)x, (const unsigned int*)qw, (const ST*)sc, (XT*)y, K, N, splits, slots);

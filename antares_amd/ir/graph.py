@@ -65,6 +65,12 @@ class Graph:
     def canonical_key(self) -> str:
         return canonical(self.statements, {k: v.dtype for k, v in self.tensors.items()})
 
+    def canonical_tensor_order(self) -> List[str]:
+        """Tensor names in the order in which canonical_key numbers them."""
+        order: List[str] = []
+        canonical(self.statements, {k: v.dtype for k, v in self.tensors.items()}, order)
+        return order
+
     def to_ir(self) -> str:
         return '; '.join(statement_to_ir(s) for s in self.statements)
 

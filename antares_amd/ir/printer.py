@@ -51,10 +51,12 @@ def statement_to_ir(st, tensor_name=lambda n: n, axis_name=lambda n: n) -> str:
     return f'{tensor_name(st.output)}[{lhs}] {op} {to_ir(st.root, tensor_name, axis_name)}'
 
 
-def canonical(statements, dtypes) -> str:
+def canonical(statements, dtypes, tensor_order=None) -> str:
     """Spelling-independent key: tensors become $t0,$t1.. (with dtype), axes
     $X0,$X1.. in order of first appearance; extents are left out so one key
-    covers every shape."""
+    covers every shape.  ``tensor_order`` (a list) receives the tensors' own names
+    in that order: $tN of one program and $tN of another with the same key play
+    the same part."""
     tmap, amap = {}, {}
 
     def tname(n):
@@ -67,4 +69,7 @@ def canonical(statements, dtypes) -> str:
             amap[n] = f'$X{len(amap)}'
         return amap[n]
 
-    return ' ; '.join(statement_to_ir(st, tname, aname) for st in statements)
+    key = ' ; '.join(statement_to_ir(st, tname, aname) for st in statements)
+    if tensor_order is not None:
+        tensor_order.extend(tmap)              # dicts keep insertion order
+    return key

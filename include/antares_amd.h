@@ -146,8 +146,12 @@ int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, const void*
  * qweight int32 [K/8,N], eight nibbles per word along K (least significant
  * first), zero point fixed at 8, scales fp32 or fp16 [K/128,N], x and y fp32
  * or fp16 (x_f16 / scales_f16 select).  M = 1.  The sums over the K/1024
- * slices of k meet as fixed-point numbers (steps of 2^-22): a slice whose sum
- * is NaN, infinite or beyond 2^24 / (K/1024) in magnitude turns y[n] into NaN. */
+ * slices of k meet as fixed-point numbers, so y does not depend on the order in
+ * which they arrive.  fp16 y: steps of 2^-22; a slice whose sum is NaN, infinite
+ * or beyond 2^24 / (K/1024) in magnitude turns y[n] into NaN.  fp32 y: two
+ * fixed-point words per column, exact for slice sums between 2^-34 and
+ * 2^39 / (K/1024) in magnitude (smaller ones to within 2^-59, larger ones or
+ * non-finite ones turn y[n] into NaN). */
 int art_gemv_gptq(const void* x_dev, const void* qweight_dev, const void* scales_dev, void* y_dev,
                   int K, int N, int x_f16, int scales_f16, void* stream);
 

@@ -135,3 +135,72 @@ def test_sample_decode_step_as_the_sample_writes_it(oracle_built):
             got = forward(token, pos).float().cpu().numpy().reshape(-1)
             assert np.allclose(got, want, rtol=2e-4, atol=2e-4), (pos, np.abs(got - want).max())
             token = int(np.argmax(want))
+
+
+def test_programs_spelled_with_other_names_run_on_the_hand_kernels(oracle_built):
+    """The same three programs with tensor names other than the registered ones: the hand-written kernel must be
+    selected and fed the right operands (a rectangular, non-symmetric case so that a swapped operand cannot pass)."""
+    import autort
+    from antares_amd import workloads
+    from antares_amd.autort import patterns
+    from oracle import hot_ops
+    dev = autort.device()
+    print('[case] fp16 GEMM as input0/input1/output0', flush=True)
+    f = autort.export(ir='''
+        mid[M, N] +=! input0[M, K].to(`float32`) * input1[K, N].to(`float32`)
+        output0[M, N] = mid[M, N].to(`float16`)
+    ''', inputs=['input0=float16[M:4096, K:4096]', 'input1=float16[K:4096, N:4096]'], name='gemm_f16_renamed')
+    assert f.fast_path is not None
+    g = torch.Generator().manual_seed(2)
+    a = (torch.randn(96, 128, generator=g) * 0.1).half()
+    b = (torch.randn(128, 72, generator=g) * 0.1).half()
+    got = f(a.to(dev), b.to(dev)).cpu()
+    assert torch.allclose(got.float(), (a.double() @ b.double()).float(), rtol=1e-2, atol=1e-2)
+
+    print('[case] int4 GEMV as lhs/qw/sc/qz', flush=True)
+    ir = (patterns.W4A16_IR.replace('qweight', 'qw').replace('scales', 'sc').replace('qzeros', 'qz')
+          .replace('x[', 'lhs[').replace('y[', 'out[').replace('acc[', 'tmp['))
+    h = autort.export(ir=ir, inputs=['lhs=float16[M:1, K:4096]', 'qw=int8[KH:2048, N:11008]', 'sc=float16[G:32, N:11008]',
+                                     'qz=int8[G:32, NH:5504]'], name='gemv_w4a16_renamed')
+    assert h.fast_path is not None
+    p = workloads.w4_problem(21, 1, 1024, 272)
+    y = h(p['x'].to(dev), p['qweight'].to(dev), p['scales'].to(dev), p['qzeros'].to(dev)).cpu().numpy()
+    want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy())
+    assert np.allclose(y.astype(np.float32), want.astype(np.float32), rtol=1e-2, atol=1e-2)
+
+    print('[case] GPTQ GEMV as vec/packed/sc', flush=True)
+    ir = SAMPLE_IR.replace('input0', 'vec').replace('qweight', 'packed').replace('scales', 'sc').replace('my_result', 'res')
+    k = autort.export(ir=ir, inputs=['vec=float32[S:4096]', 'packed=int32[L:512, N:12288]', 'sc=float32[K:32, N:12288]'],
+                      name='gemv_gptq_renamed')
+    assert k.fast_path is not None
+    lin = gptq_linear(g, 2048, 192)
+    x = torch.randn(2048, generator=g)
+    y = k(x.to(dev), lin['qweight'].to(dev), lin['scales'].to(dev)).cpu().numpy()
+    want = hot_ops.gemv_gptq_f32(x.numpy(), lin['qweight'].numpy(), lin['scales'].numpy())
+    assert np.allclose(y, want, rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize('K,N', [(2048, 192), (4096, 4096), (11008, 512)])
+def test_gptq_fp32_results_keep_fp32_precision_at_any_magnitude(oracle_built, K, N):
+    """The K-splits of an fp32 result meet exactly: outputs around 1e-7 are as accurate relative to their size as
+    outputs around 1, outputs around 1e6 do not turn into NaN, and a second call gives the same bits."""
+    import autort
+    from oracle import hot_ops
+    dev = autort.device()
+    f = autort.export(ir=SAMPLE_IR, inputs=["input0=float32[S:4096]", "qweight=int32[L:512, N:12288]", "scales=float32[K:32, N:12288]"])
+    g = torch.Generator().manual_seed(K + N)
+    lin = gptq_linear(g, K, N)
+    x = torch.randn(K, generator=g)
+    for name, xs, ss in [('unit', 1.0, 1.0), ('tiny', 1e-3, 1e-4), ('huge', 1e3, 1e3)]:
+        print(f'[case] gptq fp32 magnitudes K={K} N={N} {name}', flush=True)
+        xv, sv = x * xs, lin['scales'] * ss
+        got = f(xv.to(dev), lin['qweight'].to(dev), sv.to(dev))
+        again = f(xv.to(dev), lin['qweight'].to(dev), sv.to(dev))
+        assert torch.equal(got, again)
+        got = got.cpu().numpy()
+        want = hot_ops.gemv_gptq_f32(xv.numpy(), lin['qweight'].numpy(), sv.numpy())
+        assert np.isfinite(got).all()
+        # relative to the size of the sums involved: an fp32 sum of K terms is good to about sqrt(K) * 2^-24 of the
+        # magnitude of its terms, whatever that magnitude is
+        scale = float(np.abs(want).mean())
+        assert np.abs(got - want).max() < 2e-4 * scale, (name, np.abs(got - want).max(), scale)

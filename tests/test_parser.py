@@ -179,3 +179,30 @@ def test_config_strings_are_parsed_leniently():
     assert parse_config('tune:5') == {'tune': 5}
     assert parse_config('~N~:[256,8,32],~S~:[64,8]') == {'~N~': [256, 8, 32], '~S~': [64, 8]}
     assert parse_config(None) == {} and parse_config('whatever') == {'whatever': ''}
+
+
+def test_hand_kernel_roles_follow_the_program_not_the_names():
+    """A program spelled with other tensor names than the registered pattern still selects the hand-written kernel,
+    and each of its tensors is bound to the part it plays in the program (first appearance in the fused statements)."""
+    from antares_amd.autort import patterns
+    from antares_amd.autort.op import ExportedOp
+    gemm = ExportedOp('''
+        mid[M, N] +=! input0[M, K].to(`float32`) * input1[K, N].to(`float32`)
+        output0[M, N] = mid[M, N].to(`float16`)
+    ''', ['input1=float16[K:64, N:64]', 'input0=float16[M:64, K:64]'])
+    assert gemm.fast_path is patterns._gemm_f16_handler
+    assert {r: gemm.fast_roles[r] for r in ('a', 'b', 'c')} == {'a': 'input0', 'b': 'input1', 'c': 'output0'}
+    w4 = ExportedOp(patterns.W4A16_IR.replace('qweight', 'qw').replace('scales', 'sc').replace('qzeros', 'qz')
+                    .replace('x[', 'lhs[').replace('y[', 'out[').replace('acc[', 'tmp['),
+                    ['qz=int8[G:32, NH:5504]', 'lhs=float16[M:1, K:4096]', 'sc=float16[G:32, N:11008]', 'qw=int8[KH:2048, N:11008]'])
+    assert w4.fast_path is patterns._w4a16_handler
+    assert {r: w4.fast_roles[r] for r in ('x', 'qweight', 'scales', 'qzeros', 'y')} == \
+        {'x': 'lhs', 'qweight': 'qw', 'scales': 'sc', 'qzeros': 'qz', 'y': 'out'}
+    gptq = ExportedOp(patterns.GPTQ_GEMV_IR.replace('input0', 'vec').replace('qweight', 'packed').replace('scales', 'sc')
+                      .replace('my_result', 'res'), ['vec=float32[S:4096]', 'packed=int32[L:512, N:12288]', 'sc=float16[K:32, N:12288]'])
+    assert gptq.fast_path is patterns._gptq_handler
+    assert {r: gptq.fast_roles[r] for r in ('input0', 'qweight', 'scales', 'my_result')} == \
+        {'input0': 'vec', 'qweight': 'packed', 'scales': 'sc', 'my_result': 'res'}
+    # the registered spelling maps to itself
+    own = ExportedOp(patterns.GEMM_F16_IR, patterns.GEMM_F16_INPUTS)
+    assert own.fast_roles['a'] == 'a' and own.fast_roles['c'] == 'c'
