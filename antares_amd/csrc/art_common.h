@@ -16,8 +16,22 @@ struct Workspace {
   void* base = nullptr;      // device memory
   size_t bytes = 0;
 };
-// Workspace of the current device (allocated by art_init).
-Workspace& workspace();
+// Workspace of (current device, stream).  Launches on one stream are ordered, so they can share partial-result
+// memory; launches on different streams are not, so every stream gets a workspace of its own, allocated and zeroed
+// the first time the stream is seen (up to kMaxStreamsPerDevice streams per device; that first use must not happen
+// while the stream is being captured into a graph, because it allocates).  Returns nullptr with the error set.
+Workspace* workspace(hipStream_t stream);
+constexpr int kMaxStreamsPerDevice = 8;
+
+// Blocks per head the split decode attention may use, shared by its producer (art_llm.hip) and the projection that
+// merges the per-part records (art_gemv_w4.hip).
+constexpr int kMaxAttnParts = 8;
+
+// True when the byte ranges [a, a + an) and [b, b + bn) overlap.
+inline bool overlaps(const void* a, size_t an, const void* b, size_t bn) {
+  const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+  return a0 < b0 + bn && b0 < a0 + an;
+}
 
 // Workspace layout.  Ticket words must read zero whenever no kernel is running,
 // so they never share bytes with scratch data.

@@ -322,8 +322,9 @@ extern "C" int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const 
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0 && ((uintptr_t)qzeros_dev % 8) == 0 &&
                   ((uintptr_t)y_dev % 8) == 0,
               "art_gemm_w4a16: x and qweight must be 16-byte aligned, qzeros and y 8-byte aligned");
-  art::Workspace& ws = art::workspace();
-  ART_REQUIRE(ws.base != nullptr, "art_gemm_w4a16: art_init has not been called on this device");
+  art::Workspace* wsp = art::workspace((hipStream_t)stream);
+  if (!wsp) return 1;
+  art::Workspace& ws = *wsp;
   float* scratch = reinterpret_cast<float*>((char*)ws.base + art::kScratchOffset);
   const size_t scratch_bytes = ws.bytes - art::kScratchOffset;
   static int compute_units = 0;

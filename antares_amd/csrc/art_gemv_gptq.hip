@@ -179,8 +179,9 @@ int launch(const void* x, const void* qw, const void* sc, void* y, int K, int N,
   const int tiles = (N + CT - 1) / CT;
   const int splits = (K + kBlockK - 1) / kBlockK;
   ART_REQUIRE(splits <= 127, "art_gemv_gptq: K too large (%d)", K);
-  art::Workspace& ws = art::workspace();
-  ART_REQUIRE(ws.base != nullptr, "art_gemv_gptq: call art_init first");
+  art::Workspace* wsp = art::workspace(stream);
+  if (!wsp) return 1;
+  art::Workspace& ws = *wsp;
   ART_REQUIRE(art::kSlotOffset + (size_t)N * 16 <= art::kScratchOffset, "art_gemv_gptq: N too large (%d)", N);
   unsigned long long* slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(ws.base) + art::kSlotOffset);
   gemv_gptq_kernel<XT, ST><<<dim3(tiles, splits), dim3(kThreads), 0, stream>>>(

@@ -185,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
   // head and left, per (head, part), 128 unnormalised sums, the running maximum and the running sum of
   // exp.  As with SwiGLU each column lane produces one pair of the k lane's 16 values.
   constexpr bool attn = (M == 1) && (MODE == 3);
-  constexpr int kMaxParts = 8, kPartStride = 132;         // record layout of the attention kernel
+  constexpr int kMaxParts = art::kMaxAttnParts, kPartStride = 132;         // record layout of the attention kernel
   f32x2 pacc[kMaxParts], pml[kMaxParts];
   if (attn) {
     const int k = 2 * r0c + 2 * cl, head = k >> 7, d = k & 127;
@@ -385,8 +385,9 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
   const int tiles = (N + CT - 1) / CT;
   const int splits = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
   ART_REQUIRE(splits <= 127, "art_gemv_w4a16: K too large (%d)", K);
-  art::Workspace& ws = art::workspace();
-  ART_REQUIRE(ws.base != nullptr, "art_gemv_w4a16: call art_init first");
+  art::Workspace* wsp = art::workspace(stream);
+  if (!wsp) return 1;
+  art::Workspace& ws = *wsp;
   ART_REQUIRE(art::kSlotOffset + (size_t)M * N * 8 <= art::kScratchOffset, "art_gemv_w4a16: N too large (%d)", N);
   unsigned long long* slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(ws.base) + art::kSlotOffset);
   const Magic magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
@@ -413,6 +414,8 @@ extern "C" int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const 
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0,
               "art_gemv_w4a16: x and qweight must be 16-byte aligned");
   ART_REQUIRE(M >= 1 && M <= 8, "art_gemv_w4a16: M must be in 1..8 (got %d); larger batches go through art_gemm_w4a16", M);
+  // blocks of one column tile write y while blocks of other tiles still read x
+  ART_REQUIRE(!art::overlaps(x_dev, (size_t)M * K * 2, y_dev, (size_t)M * N * 2), "art_gemv_w4a16: y must not overlap x");
   hipStream_t st = (hipStream_t)stream;
   int m = 0;
   while (m < M) {       // rows of x are handled up to four at a time
@@ -437,7 +440,9 @@ extern "C" int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, 
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_fused: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0 && ((uintptr_t)norm_weight_dev % 16) == 0,
               "art_gemv_w4a16_fused: x, qweight and the norm weight must be 16-byte aligned");
-  ART_REQUIRE(x_dev != y_dev || norm_weight_dev == nullptr, "art_gemv_w4a16_fused: y may alias the residual, not a normalised x");
+  // blocks of one column tile write y while blocks of other tiles still read x: only the residual may alias y
+  ART_REQUIRE(!art::overlaps(x_dev, (size_t)(swiglu_input ? 2 : 1) * K * 2, y_dev, (size_t)N * 2),
+              "art_gemv_w4a16_fused: y must not overlap x (it may alias the residual)");
   Fused f{(const _Float16*)norm_weight_dev, (const _Float16*)residual_dev, swiglu_input ? (const _Float16*)x_dev : nullptr,
           1.0f / (float)K, eps, nullptr, 0};
   return launch<1>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, (hipStream_t)stream, f);
@@ -446,10 +451,12 @@ extern "C" int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, 
 extern "C" int art_gemv_w4a16_attn(const void* partial_dev, int parts, const void* qweight_dev, const void* scales_dev,
                                    const void* qzeros_dev, void* y_dev, int K, int N, const void* residual_dev, void* stream) {
   ART_REQUIRE(partial_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16_attn: null pointer");
-  ART_REQUIRE(parts >= 2 && parts <= 8, "art_gemv_w4a16_attn: parts must be in 2..8 (got %d)", parts);
+  ART_REQUIRE(parts >= 2 && parts <= art::kMaxAttnParts, "art_gemv_w4a16_attn: parts must be in 2..%d (got %d)", art::kMaxAttnParts, parts);
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_attn: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)partial_dev % 16) == 0,
               "art_gemv_w4a16_attn: partial records and qweight must be 16-byte aligned");
+  ART_REQUIRE(!art::overlaps(partial_dev, (size_t)(K / 128) * parts * 132 * 4, y_dev, (size_t)N * 2),
+              "art_gemv_w4a16_attn: y must not overlap the partial records");
   Fused f{nullptr, (const _Float16*)residual_dev, nullptr, 0.f, 0.f, (const float*)partial_dev, parts};
   return launch<1>(partial_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, (hipStream_t)stream, f);
 }

@@ -460,7 +460,8 @@ extern "C" int art_decode_attention_rope_split(const void* qkv_dev, const void* 
   ART_REQUIRE(qkv_dev && inv_freq_dev && key_cache_dev && val_cache_dev && att_f_dev && out_dev && pos_dev,
               "art_decode_attention_rope: null pointer");
   ART_REQUIRE(head_dim == 128 && heads >= 1, "art_decode_attention_rope: head_dim must be 128 (got %d)", head_dim);
-  ART_REQUIRE(parts >= 1 && parts <= 16, "art_decode_attention_rope: parts must be in 1..16 (got %d)", parts);
+  ART_REQUIRE(parts >= 1 && parts <= art::kMaxAttnParts, "art_decode_attention_rope_split: parts must be in 1..%d (got %d)",
+              art::kMaxAttnParts, parts);
   ART_REQUIRE(max_positions >= 1, "art_decode_attention_rope: the caches have no rows");
   ART_REQUIRE(((uintptr_t)key_cache_dev % 16) == 0 && ((uintptr_t)val_cache_dev % 16) == 0 && ((uintptr_t)out_dev % 16) == 0,
               "art_decode_attention_rope: caches and output must be 16-byte aligned");

@@ -194,8 +194,9 @@ extern "C" int art_partition_even_first_i32(const void* in_dev, void* out_dev, l
   ART_REQUIRE(in_dev && out_dev && in_dev != out_dev, "art_partition_even_first_i32: null or aliased pointers");
   ART_REQUIRE(((uintptr_t)in_dev % 16) == 0, "art_partition_even_first_i32: input must be 16-byte aligned");
   ART_REQUIRE(((uintptr_t)out_dev % 4) == 0, "art_partition_even_first_i32: output must be 4-byte aligned");
-  art::Workspace& ws = art::workspace();
-  ART_REQUIRE(ws.base != nullptr, "art_partition_even_first_i32: call art_init first");
+  art::Workspace* wsp = art::workspace((hipStream_t)stream);
+  if (!wsp) return 1;
+  art::Workspace& ws = *wsp;
   const long long tiles = (n + kTile - 1) / kTile;
   constexpr long long kMaxBlocks = 1024;                        // bounds the counts every block adds up (4 KiB from L2)
   const int tiles_per_block = (int)((tiles + kMaxBlocks - 1) / kMaxBlocks);

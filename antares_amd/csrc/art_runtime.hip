@@ -28,13 +28,63 @@ int fail(const char* fmt, ...) {
 }
 
 static constexpr int kMaxDevices = 16;
-static Workspace g_ws[kMaxDevices];
+// 64 MiB: split-K accumulators, partial tiles of the split-K GEMM and tile states of the scan kernels.
+static constexpr size_t kWorkspaceBytes = 64u << 20;
+struct StreamWorkspace {
+  hipStream_t stream;
+  Workspace ws;
+};
+struct DeviceState {
+  bool initialised = false;
+  int used = 0;
+  StreamWorkspace slot[kMaxStreamsPerDevice];
+};
+static DeviceState g_dev[kMaxDevices];
 static std::mutex g_mu;
 
-Workspace& workspace() {
+static int allocate_workspace(Workspace* ws) {
+  ART_HIP(hipMalloc(&ws->base, kWorkspaceBytes));
+  hipError_t e = hipMemset(ws->base, 0, kWorkspaceBytes);
+  if (e == hipSuccess) e = hipDeviceSynchronize();        // the zeroes are in place before any stream uses them
+  if (e != hipSuccess) {
+    (void)hipFree(ws->base);
+    ws->base = nullptr;
+    return fail("zeroing the workspace failed: %s", hipGetErrorString(e));
+  }
+  ws->bytes = kWorkspaceBytes;
+  return 0;
+}
+
+Workspace* workspace(hipStream_t stream) {
   int dev = 0;
-  (void)hipGetDevice(&dev);
-  return g_ws[dev < 0 || dev >= kMaxDevices ? 0 : dev];
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail("workspace: no current device");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_mu);
+  DeviceState& d = g_dev[dev];
+  if (!d.initialised) {
+    fail("call art_init first");
+    return nullptr;
+  }
+  for (int i = 0; i < d.used; ++i)
+    if (d.slot[i].stream == stream) return &d.slot[i].ws;
+  if (d.used == kMaxStreamsPerDevice) {
+    fail("more than %d streams use split-K / two-pass kernels on device %d; order them on fewer streams", kMaxStreamsPerDevice, dev);
+    return nullptr;
+  }
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    fail("the first split-K / two-pass launch on a stream allocates its workspace and cannot be captured into a graph: "
+         "run the operator once on this stream before capturing");
+    return nullptr;
+  }
+  StreamWorkspace& sw = d.slot[d.used];
+  sw.stream = stream;
+  sw.ws = Workspace{};
+  if (allocate_workspace(&sw.ws)) return nullptr;
+  ++d.used;
+  return &sw.ws;
 }
 
 static std::string& compile_log() {
@@ -51,28 +101,23 @@ struct art_func {
   hipFunction_t handle;
 };
 
-// 64 MiB: split-K accumulators, partial tiles of the split-K GEMM and tile states of the scan kernels.
-static constexpr size_t kWorkspaceBytes = 64u << 20;
-
 extern "C" {
 
 const char* art_last_error(void) { return art::last_error().c_str(); }
 const char* art_compile_log(void) { return art::compile_log().c_str(); }
-size_t art_workspace_bytes(void) { return kWorkspaceBytes; }
+size_t art_workspace_bytes(void) { return art::kWorkspaceBytes; }
 
 int art_init(int device) {
   int count = 0;
   ART_HIP(hipGetDeviceCount(&count));
   ART_REQUIRE(device >= 0 && device < count && device < art::kMaxDevices, "art_init: no such device %d (have %d)", device, count);
   ART_HIP(hipSetDevice(device));
-  std::lock_guard<std::mutex> lock(art::g_mu);
-  art::Workspace& ws = art::g_ws[device];
-  if (!ws.base) {
-    ART_HIP(hipMalloc(&ws.base, kWorkspaceBytes));
-    ART_HIP(hipMemset(ws.base, 0, kWorkspaceBytes));
-    ws.bytes = kWorkspaceBytes;
+  {
+    std::lock_guard<std::mutex> lock(art::g_mu);
+    art::g_dev[device].initialised = true;
   }
-  return 0;
+  // the workspace of the default stream now; other streams get theirs when they first need one
+  return art::workspace(nullptr) ? 0 : 1;
 }
 
 int art_device_props(art_props* out) {
@@ -232,6 +277,39 @@ extern "C" int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, 
   return 0;
 }
 
+// ------------------------------------------------------------ read-only kernel
+// The access pattern of the weight stream of the int4 GEMV with nothing behind it: a block of 256 threads owns 32 KiB,
+// every thread issues its eight 16-byte loads (128 contiguous bytes per 8 lanes, rows `pitch` bytes apart) before it
+// looks at any of them, and the block leaves one word that depends on all of them.  What this takes for a buffer is
+// what a single dependent launch spends on getting the bytes on chip, whatever arithmetic follows.
+__global__ __launch_bounds__(256) void art_read_kernel(const unsigned char* __restrict__ src, size_t pitch, int tiles,
+                                                       unsigned int* __restrict__ sink) {
+  const int tid = threadIdx.x, cl = tid & 7, kl = tid >> 3;
+  const int tile = blockIdx.x % tiles, split = blockIdx.x / tiles;
+  const unsigned char* p = src + ((size_t)split * 256 + (size_t)kl * 8) * pitch + (size_t)tile * 128 + cl * 16;
+  u32x4 w[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)i * pitch));
+  unsigned int acc = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc ^= w[i][0] ^ w[i][1] ^ w[i][2] ^ w[i][3];
+  if (acc == 0x9E3779B9u) sink[blockIdx.x] = acc;        // (almost) never true: the loads stay, the stores do not happen
+}
+
+extern "C" int art_read_bytes(const void* src_dev, size_t bytes, void* sink_dev, void* stream) {
+  // viewed as rows of 11008 bytes when the size allows it (the headline weight matrix), else rows of 128 bytes
+  ART_REQUIRE(src_dev && sink_dev && ((uintptr_t)src_dev % 16) == 0 && bytes % 32768 == 0 && bytes > 0,
+              "art_read_bytes: need a 16-byte aligned buffer of a multiple of 32768 bytes");
+  const size_t pitch = (bytes % (11008u * 256u) == 0) ? 11008 : 128;
+  const int tiles = (int)(pitch / 128);
+  const size_t blocks = bytes / 32768;
+  ART_REQUIRE(blocks <= 4096, "art_read_bytes: at most 128 MiB per launch (sink has 4096 words)");
+  art_read_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>((const unsigned char*)src_dev, pitch, tiles,
+                                                                               (unsigned int*)sink_dev);
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---- device memory for callers that own no allocator (the reference's evaluator; the torch plugin uses torch's)
 extern "C" int art_alloc(size_t bytes, void** out_dev) {
   ART_REQUIRE(out_dev != nullptr, "art_alloc: null output");
@@ -248,6 +326,11 @@ extern "C" int art_free(void* dev) {
 
 extern "C" int art_memcpy_htod(void* dst_dev, const void* src_host, size_t bytes, void* stream) {
   if (bytes) ART_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+  return 0;
+}
+
+extern "C" int art_memcpy_dtod(void* dst_dev, const void* src_dev, size_t bytes, void* stream) {
+  if (bytes) ART_HIP(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
   return 0;
 }
 

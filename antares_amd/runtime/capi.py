@@ -50,6 +50,8 @@ _SIGNATURES = {
     'art_free': (c_int, [c_void_p]),
     'art_memcpy_htod': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     'art_memcpy_dtoh': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    'art_memcpy_dtod': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    'art_read_bytes': (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     'art_gemv_w4a16': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_decode_attention_rope_split': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p]),
     'art_gemv_w4a16_attn': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),

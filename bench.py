@@ -1,7 +1,9 @@
 #!/usr/bin/env python
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra] [--no-decode]
+    python bench.py --calibrate-copy MIB LAUNCHES     # plain copy of known size, for scaling memory-traffic counters
+    python bench.py --read-floor                      # only the read-only launch over the headline's weight bytes
 
 Headline workload (BASELINE.json: "int4-GEMV HBM GB/s"): the int4 group-128
 GEMV y[1,11008] = x[1,4096] @ dequant(W), through ``autort.export`` and the
@@ -32,9 +34,21 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LAYERS = 32
-# HBM bytes per launch of the headline GEMV kernel, from FETCH_SIZE / WRITE_SIZE counters scaled by
-# the copy-kernel calibration (profiles/gemv_w4a16_4096x11008_traffic_pmc.md): 23.80 MB read + 0.81 MB written.
-GEMV_4096x11008_TRAFFIC_BYTES = 24_614_000
+# HBM bytes per launch of the headline GEMV kernel come from the committed counter summary (FETCH_SIZE / WRITE_SIZE
+# scaled by the copy-kernel calibration), which states them on a line `traffic_bytes_per_launch: <integer>`.
+TRAFFIC_SUMMARY = os.path.join(ROOT, 'profiles', 'gemv_w4a16_4096x11008_traffic_pmc.md')
+
+
+def traffic_from_summary(path=TRAFFIC_SUMMARY):
+    """Measured HBM bytes per launch as recorded in the counter summary, or None when there is none."""
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.strip().startswith('traffic_bytes_per_launch:'):
+                    return int(line.split(':', 1)[1].strip().replace('_', ''))
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 def parse_args():
@@ -48,7 +62,43 @@ def parse_args():
     ap.add_argument('--decode-cpu-steps', type=int, default=4, help='decode steps timed on the CPU oracle (0 = skip)')
     ap.add_argument('--att-parts', type=int, default=8, help='blocks per head of the decode attention (1 = unsplit)')
     ap.add_argument('--seed', type=int, default=0)
+    ap.add_argument('--calibrate-copy', nargs=2, type=int, metavar=('MIB', 'LAUNCHES'),
+                    help='run only the plain copy kernel on MIB MiB, LAUNCHES times (counter calibration), and exit')
+    ap.add_argument('--read-floor', action='store_true',
+                    help='run only the read-only launch over 32 distinct buffers of the headline weight size, and exit')
     return ap.parse_args()
+
+
+def calibrate_copy(torch, capi, mib, launches):
+    """The library's plain copy kernel on a buffer of known size: it reads and writes exactly mib * 2^20 bytes per
+    launch, so the ratio of a memory-traffic counter to that figure is the scale to apply to other kernels' readings."""
+    from ctypes import c_void_p
+    n = mib << 20
+    src = torch.full((n,), 7, dtype=torch.uint8, device='cuda')
+    dst = torch.empty_like(src)
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(launches):
+        capi.check(capi.lib().art_copy_bytes(c_void_p(dst.data_ptr()), c_void_p(src.data_ptr()), n, c_void_p(stream)))
+    torch.cuda.synchronize()
+    assert bool((dst == 7).all())
+    return {'copied_bytes_per_launch': n, 'launches': launches}
+
+
+def bench_read_floor(torch, capi, steps, warmup, nbytes=2048 * 11008, layers=LAYERS):
+    """What one dependent launch needs to bring the headline GEMV's weight bytes on chip with no arithmetic behind
+    them: `art_read_bytes` (same blocks, same loads as the GEMV's weight stream) over `layers` distinct buffers
+    recorded in one HIP graph, exactly as the GEMV itself is timed."""
+    from ctypes import c_void_p
+    bufs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device='cuda') for _ in range(layers)]
+    sink = torch.zeros(4096, dtype=torch.int32, device='cuda')
+
+    def one_pass():
+        stream = torch.cuda.current_stream().cuda_stream
+        for b in bufs:
+            capi.check(capi.lib().art_read_bytes(c_void_p(b.data_ptr()), nbytes, c_void_p(sink.data_ptr()), c_void_p(stream)))
+    sec = time_graph(torch, capi, one_pass, steps, warmup) / layers
+    return {'kernel': 'art_read_kernel', 'bytes_per_launch': nbytes, 'us_per_launch': round(sec * 1e6, 3),
+            'gbps': round(nbytes / sec / 1e9, 1), 'frac_of_peak': round(nbytes / sec / 1e9 / HBM_PEAK_GBPS, 4)}
 
 
 def time_graph(torch, capi, fn, steps, warmup, warm_ms=0.0):
@@ -307,6 +357,12 @@ def main():
     from antares_amd import workloads
     from antares_amd.runtime import capi
     capi.init(0)
+    if args.calibrate_copy:
+        print(json.dumps(calibrate_copy(torch, capi, *args.calibrate_copy)), flush=True)
+        return
+    if args.read_floor:
+        print(json.dumps(bench_read_floor(torch, capi, args.steps, args.warmup)), flush=True)
+        return
     K, N, M = 4096, 11008, 1
     head = bench_gemv(torch, autort, capi, workloads, K, N, M, args.steps, args.warmup, args.seed)
     result = {
@@ -317,11 +373,13 @@ def main():
                    'weights': 'uint8 [K/2,N] two nibbles along K; fp16 scale + 4-bit zero per group',
                    'distinct_weight_sets': head['launches_per_step'], 'timed_through': 'HIP graph replay'},
         'roofline': {'bound': 'hbm', 'achieved': round(head['gbps'], 2), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-                     'frac': round(head['gbps'] / HBM_PEAK_GBPS, 4), 'traffic': GEMV_4096x11008_TRAFFIC_BYTES,
+                     'frac': round(head['gbps'] / HBM_PEAK_GBPS, 4), 'traffic': traffic_from_summary(),
                      'kernel': 'gemv_w4a16_kernel', 'bytes_per_launch': head['bytes_per_launch'],
                      'us_per_launch': round(head['us_per_launch'], 3)},
     }
     if not args.no_extra:
+        # the floor of a single launch over the same weight bytes (no arithmetic), measured the same way
+        result['roofline']['read_only_launch'] = bench_read_floor(torch, capi, args.steps, args.warmup)
         extra = []
         for (k, n) in [(4096, 4096), (11008, 4096), (4096, 32000)]:
             r = bench_gemv(torch, autort, capi, workloads, k, n, 1, max(10, args.steps // 2), args.warmup, args.seed,

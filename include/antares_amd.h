@@ -7,16 +7,19 @@
  * Nothing here calls exit().  All pointers named *_dev are raw device
  * addresses (e.g. torch `tensor.data_ptr()`); `stream` is a hipStream_t passed
  * as void* (NULL = the default stream).  The caller owns all tensor memory;
- * the library owns loaded modules for the life of the process and one internal
- * workspace per device that is allocated by art_init().
+ * the library owns loaded modules for the life of the process and internal
+ * workspaces (64 MiB each) that it never frees.
  *
  * The kernels that split K or work in two passes (art_gemv_w4a16*, art_gemv_gptq,
  * art_gemm_w4a16, art_partition_even_first_i32) keep their partial results in
- * that workspace, so on one device two of their launches must not be in flight
- * at the same time: enqueue them on one stream, or order the streams with
- * events.  The reference has the same single-caller contract (static state, no
- * locks: frameworks/pytorch/main_ops.cc:14-15).  Launches leave the workspace
- * clean, also when their inputs hold NaN or infinities.
+ * a workspace.  Launches on one stream are ordered and share one; every stream
+ * gets a workspace of its own the first time such a kernel is launched on it
+ * (art_init allocates the default stream's), so launches on different streams
+ * do not disturb each other.  At most 8 streams per device may do so, and a
+ * stream's first such launch must happen outside graph capture (it allocates).
+ * Host calls may come from several threads (the reference allows one: static
+ * state, no locks, frameworks/pytorch/main_ops.cc:14-15).  Launches leave
+ * the workspace clean, also when their inputs hold NaN or infinities.
  *
  * The first group replaces the reference's header-only `namespace ab` device
  * runtime and its ExecutionModule; the second group are typed entry points for
@@ -103,10 +106,19 @@ int art_alloc(size_t bytes, void** out_dev);
 int art_free(void* dev);
 int art_memcpy_htod(void* dst_dev, const void* src_host, size_t bytes, void* stream);
 int art_memcpy_dtoh(void* dst_host, const void* src_dev, size_t bytes, void* stream);
+/* Device to device, asynchronous on `stream`; replaces ab::memcpyDtoD (backend.hpp:225-227). */
+int art_memcpy_dtod(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
 
 /* Plain device copy kernel (dst, src: 16-byte aligned, bytes % 16 == 0); used
  * as the calibration workload for memory-traffic counters. */
 int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+
+/* Read-only counterpart: one launch that fetches `bytes` (a multiple of 32768, at most 128 MiB; 16-byte aligned)
+ * with the access pattern of the int4 GEMV's weight stream (blocks of 256 threads x eight 16-byte loads, rows of
+ * 11008 bytes when bytes is a multiple of 11008 * 256, else of 128 bytes) and computes nothing.  Its duration is the
+ * floor of any single launch that has to bring these bytes on chip.  sink_dev: 4096 words of scratch (never
+ * written in practice). */
+int art_read_bytes(const void* src_dev, size_t bytes, void* sink_dev, void* stream);
 
 /* ---------------------------------------------------- hand-written kernels */
 
@@ -137,7 +149,8 @@ int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const void* scale
  *   residual_dev != NULL:    y = fp16(fp16(product) + residual)             (lines :168,:173)
  *   swiglu_input != 0:       x_dev holds gate | up (2*K values) and the product is taken with
  *       fp16(silu(gate[k]) * up[k])                                         (line :171)
- * y may alias residual.  Same roundings as the separate operators. */
+ * y may alias residual and nothing else (x and y must not overlap in any of the three entry points).
+ * Same roundings as the separate operators. */
 int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                          void* y_dev, int K, int N, const void* norm_weight_dev, float eps, const void* residual_dev,
                          int swiglu_input, void* stream);
@@ -233,7 +246,7 @@ int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev
 int art_greedy_next(const void* logits_dev, int vocab, const void* prompt_dev, int prompt_len, void* token_dev,
                     void* pos_dev, const void* embed_dev, int dim, void* x_out_dev, void* stream);
 
-/* Bytes of library workspace art_partition_even_first_i32 / split-K kernels may use. */
+/* Bytes of one library workspace (one per stream that launches split-K / two-pass kernels). */
 size_t art_workspace_bytes(void);
 
 #ifdef __cplusplus

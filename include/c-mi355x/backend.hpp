@@ -130,6 +130,7 @@ namespace ab {
   }
 
   inline void memcpyHtoD(void* dptr, void* hptr, size_t byteSize, void* stream) { ART_OK(art_memcpy_htod(dptr, hptr, byteSize, stream)); }   // :221
+  inline void memcpyDtoD(void* dptr, void* dptr0, size_t byteSize, void* stream) { ART_OK(art_memcpy_dtod(dptr, dptr0, byteSize, stream)); }  // :225
   inline void memcpyDtoH(void* hptr, void* dptr, size_t byteSize, void* stream) { ART_OK(art_memcpy_dtoh(hptr, dptr, byteSize, stream)); }   // :229
   inline void synchronize(void* stream) { ART_OK(art_stream_synchronize(stream)); }                                                           // :233
 

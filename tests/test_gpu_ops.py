@@ -391,3 +391,37 @@ def test_permutation_copies_go_through_lds_tiles(autort, ir, spec, shape, perm):
     if '* 2' in ir:
         want = want * 2
     assert torch.equal(op(x.to(dev)).cpu(), want)
+
+
+def test_split_k_launches_on_two_streams_do_not_disturb_each_other(autort):
+    """Every stream has a workspace of its own: GEMVs with K-splits enqueued on two streams at the same time give
+    the bits they give alone, and an aliasing y is refused."""
+    from ctypes import c_void_p
+    from antares_amd.runtime import capi
+    note('split-K GEMVs on two streams')
+    dev = autort.device()
+    f = w4_op(autort)
+    pa, pb = workloads.w4_problem(31, 1, 11008, 4096), workloads.w4_problem(32, 1, 11008, 4096)
+    a = [pa[k].to(dev) for k in ('x', 'qweight', 'scales', 'qzeros')]
+    b = [pb[k].to(dev) for k in ('x', 'qweight', 'scales', 'qzeros')]
+    alone_a, alone_b = f(*a).clone(), f(*b).clone()
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs_a = [torch.empty_like(alone_a) for _ in range(20)]
+    outs_b = [torch.empty_like(alone_b) for _ in range(20)]
+    for i in range(20):
+        with torch.cuda.stream(s1):
+            f(*a, out=outs_a[i])
+        with torch.cuda.stream(s2):
+            f(*b, out=outs_b[i])
+    torch.cuda.synchronize()
+    for i in range(20):
+        assert torch.equal(outs_a[i], alone_a) and torch.equal(outs_b[i], alone_b), i
+    # y overlapping x is refused by the entry points (only the residual may alias y)
+    x = a[0]
+    rc = capi.lib().art_gemv_w4a16(c_void_p(x.data_ptr()), c_void_p(a[1].data_ptr()), c_void_p(a[2].data_ptr()),
+                                   c_void_p(a[3].data_ptr()), c_void_p(x.data_ptr() + 64), 1, 11008, 4096, None)
+    assert rc != 0 and b'overlap' in capi.lib().art_last_error()
+    rc = capi.lib().art_gemv_w4a16_fused(c_void_p(x.data_ptr()), c_void_p(a[1].data_ptr()), c_void_p(a[2].data_ptr()),
+                                         c_void_p(a[3].data_ptr()), c_void_p(x.data_ptr()), 11008, 4096, None, 1e-5, None, 0, None)
+    assert rc != 0 and b'overlap' in capi.lib().art_last_error()
