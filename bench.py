@@ -101,6 +101,17 @@ def bench_read_floor(torch, capi, steps, warmup, nbytes=2048 * 11008, layers=LAY
             'gbps': round(nbytes / sec / 1e9, 1), 'frac_of_peak': round(nbytes / sec / 1e9 / HBM_PEAK_GBPS, 4)}
 
 
+_SIDE_STREAM = None
+
+
+def side_stream(torch):
+    """One non-default stream for every recording and timed region of this run."""
+    global _SIDE_STREAM
+    if _SIDE_STREAM is None:
+        _SIDE_STREAM = torch.cuda.Stream()
+    return _SIDE_STREAM
+
+
 def time_graph(torch, capi, fn, steps, warmup, warm_ms=0.0):
     """Records ``fn`` (which enqueues kernels on the current stream) in a HIP
     graph, replays it warmup + steps times, returns mean seconds per replay of
@@ -108,7 +119,7 @@ def time_graph(torch, capi, fn, steps, warmup, warm_ms=0.0):
     keeps replaying until that much time has gone by: a kernel that loads the
     matrix cores for a millisecond at a time only settles at its sustained
     clock after some tens of milliseconds."""
-    stream = torch.cuda.Stream()
+    stream = side_stream(torch)
     with torch.cuda.stream(stream):
         fn()                                   # first call: compiles / loads modules, outside capture
         stream.synchronize()
@@ -215,7 +226,7 @@ def bench_decode(torch, autort, capi, seed, prompt_len=128, decode_steps=256, cp
     dec.key_cache.zero_()
     dec.val_cache.zero_()
     dec.reset(int(prompt[0]), 0)
-    stream = torch.cuda.Stream()
+    stream = side_stream(torch)
     tokens = []
     with torch.cuda.stream(stream):
         for _ in range(prompt_len - 1):          # positions 0 .. prompt_len-2 consume the prompt

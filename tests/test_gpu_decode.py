@@ -169,12 +169,18 @@ def test_full_width_decode_matches_the_oracle(graph):
             got = dec.logits.float().cpu().numpy()
         else:
             got = dec.step().float().cpu().numpy()
-        assert np.allclose(got, want, **LOGIT_TOL), (pos, np.abs(got - want).max())
+        # a logit here is a sum of 4096 products with a spread of about 5 (2 in the small model): the operators'
+        # fp16 roundings (each within 1e-2 of the oracle on its own) reach it scaled by that spread
+        spread = float(want.std())
+        assert 2.0 < spread < 10.0
+        assert np.allclose(got, want, rtol=2e-2, atol=2e-2 * spread), (pos, np.abs(got - want).max())
         if graph:
             top2 = np.sort(want)[-2:]
             assert int(dec.pos.item()) == pos + 1
-            if top2[1] - top2[0] > 0.1:
+            if top2[1] - top2[0] > 0.05 * spread:
                 assert int(dec.token.item()) == int(np.argmax(want))
-        for l in range(cfg.n_layers):
-            assert np.allclose(dec.key_cache[l, pos].float().cpu().numpy(), ref.key_cache[l, pos].astype(np.float32), rtol=2e-2, atol=2e-2)
-            assert np.allclose(dec.val_cache[l, pos].float().cpu().numpy(), ref.val_cache[l, pos].astype(np.float32), rtol=2e-2, atol=2e-2)
+        for l in range(cfg.n_layers):           # q | k | v are sums of 4096 products too: same scaling by their spread
+            for got_c, want_c in ((dec.key_cache[l, pos], ref.key_cache[l, pos]), (dec.val_cache[l, pos], ref.val_cache[l, pos])):
+                want_c = want_c.astype(np.float32)
+                assert np.allclose(got_c.float().cpu().numpy(), want_c, rtol=2e-2, atol=2e-2 * max(1.0, float(want_c.std()))), \
+                    (pos, l, np.abs(got_c.float().cpu().numpy() - want_c).max(), float(want_c.std()))
