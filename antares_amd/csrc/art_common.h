@@ -23,6 +23,10 @@ struct Workspace {
 Workspace* workspace(hipStream_t stream);
 constexpr int kMaxStreamsPerDevice = 8;
 
+// Looks up, for the current device, the address of the scratch array built into the code object (used by
+// art_gemv_w4a16_noalloc).  Called once per device by art_init.
+int gemv_noalloc_setup(int device);
+
 // Blocks per head the split decode attention may use, shared by its producer (art_llm.hip) and the projection that
 // merges the per-part records (art_gemv_w4.hip).
 constexpr int kMaxAttnParts = 8;

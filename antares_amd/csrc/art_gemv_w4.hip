@@ -378,18 +378,27 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
   }
 }
 
+// Split-K accumulators of the entry point that allocates nothing (art_gemv_w4a16_noalloc): 64-bit slots, one per
+// (row of x, column), in device memory that belongs to the code object itself.  Zero when the code object is loaded;
+// every launch leaves the slots it used at zero again.  Each GPU has its own copy at its own address.
+constexpr int kNoAllocSlots = 131072;                   // 1 MiB per GPU: M * N <= 131072
+static __device__ __align__(256) unsigned long long scratch[kNoAllocSlots];
+constexpr int kMaxDevices = 16;
+unsigned long long* g_scratch_ptr[kMaxDevices];          // device address of `scratch` on each GPU (set by art_init)
+
 template <int M>
 int launch(const void* x, const void* qw, const void* sc, const void* qz, void* y, int K, int N, hipStream_t stream,
-           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0}) {
+           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0}, unsigned long long* slots = nullptr) {
   const int rows = K / 2;
   const int tiles = (N + CT - 1) / CT;
   const int splits = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
   ART_REQUIRE(splits <= 127, "art_gemv_w4a16: K too large (%d)", K);
-  art::Workspace* wsp = art::workspace(stream);
-  if (!wsp) return 1;
-  art::Workspace& ws = *wsp;
-  ART_REQUIRE(art::kSlotOffset + (size_t)M * N * 8 <= art::kScratchOffset, "art_gemv_w4a16: N too large (%d)", N);
-  unsigned long long* slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(ws.base) + art::kSlotOffset);
+  if (slots == nullptr) {         // the library's own workspace for this stream
+    art::Workspace* wsp = art::workspace(stream);
+    if (!wsp) return 1;
+    ART_REQUIRE(art::kSlotOffset + (size_t)M * N * 8 <= art::kScratchOffset, "art_gemv_w4a16: N too large (%d)", N);
+    slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(wsp->base) + art::kSlotOffset);
+  }
   const Magic magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
   const dim3 grid(tiles, splits), block(kThreads);
 #define ART_GEMV_LAUNCH(MODE)                                                                                          \
@@ -430,6 +439,39 @@ extern "C" int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const 
     m += step;
   }
   return 0;
+}
+
+// Called by art_init with `device` current: finds where this GPU keeps `scratch`.
+int art::gemv_noalloc_setup(int device) {
+  ART_REQUIRE(device >= 0 && device < kMaxDevices, "gemv_noalloc_setup: bad device %d", device);
+  if (g_scratch_ptr[device] != nullptr) return 0;
+  unsigned long long* ptr = nullptr;
+  ART_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+  ART_REQUIRE(ptr != nullptr, "gemv_noalloc_setup: no device address for the scratch array");
+  g_scratch_ptr[device] = ptr;
+  return 0;
+}
+
+extern "C" int art_gemv_w4a16_noalloc(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                                      void* y_dev, int M, int K, int N, void* stream) {
+  ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16_noalloc: null pointer");
+  ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_noalloc: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
+  ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0,
+              "art_gemv_w4a16_noalloc: x and qweight must be 16-byte aligned");
+  ART_REQUIRE(M >= 1 && M <= 4, "art_gemv_w4a16_noalloc: M must be in 1..4 (got %d)", M);
+  ART_REQUIRE((long long)M * N <= kNoAllocSlots, "art_gemv_w4a16_noalloc: M * N = %lld exceeds the %d accumulators of the built-in scratch array",
+              (long long)M * N, kNoAllocSlots);
+  ART_REQUIRE(!art::overlaps(x_dev, (size_t)M * K * 2, y_dev, (size_t)M * N * 2), "art_gemv_w4a16_noalloc: y must not overlap x");
+  int dev = 0;
+  ART_HIP(hipGetDevice(&dev));
+  ART_REQUIRE(dev >= 0 && dev < kMaxDevices && g_scratch_ptr[dev] != nullptr, "art_gemv_w4a16_noalloc: call art_init(%d) first", dev);
+  unsigned long long* slots = g_scratch_ptr[dev];
+  const Fused none{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0};
+  hipStream_t st = (hipStream_t)stream;
+  return M == 4 ? launch<4>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, st, none, slots)
+       : M == 3 ? launch<3>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, st, none, slots)
+       : M == 2 ? launch<2>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, st, none, slots)
+                : launch<1>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, st, none, slots);
 }
 
 extern "C" int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,

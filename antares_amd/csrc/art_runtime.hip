@@ -116,6 +116,7 @@ int art_init(int device) {
     std::lock_guard<std::mutex> lock(art::g_mu);
     art::g_dev[device].initialised = true;
   }
+  if (art::gemv_noalloc_setup(device)) return 1;
   // the workspace of the default stream now; other streams get theirs when they first need one
   return art::workspace(nullptr) ? 0 : 1;
 }

@@ -135,6 +135,16 @@ int art_read_bytes(const void* src_dev, size_t bytes, void* sink_dev, void* stre
 int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                    void* y_dev, int M, int K, int N, void* stream);
 
+/* art_gemv_w4a16 for callers that cannot allocate device memory or let a library do it (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * operands, constraints and results (bit for bit) as art_gemv_w4a16, with M in 1..4 and M * N <= 131072: the
+ * split-K accumulators live in a 1 MiB array that is part of the library's code object on every GPU, so the call
+ * allocates nothing, on any stream, first call included (art_init(device) must have run once on that device).  Larger
+ * sizes are refused with an error.  All calls on one GPU share that array: calls that overlap in time on one GPU
+ * (two streams) race; order them on one stream or with events. */
+int art_gemv_w4a16_noalloc(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                           void* y_dev, int M, int K, int N, void* stream);
+
 /* The same product for any M >= 1 on the matrix cores (prefill batches; the samples' decode loop uses
  * M = 1): operands, layouts and constraints as for art_gemv_w4a16, plus qzeros and y 8-byte aligned.
  * Rows are processed 64 at a time; each pass reads the weights once.  K-splits are combined through the
