@@ -15,7 +15,7 @@
  * a workspace.  Launches on one stream are ordered and share one; every stream
  * gets a workspace of its own the first time such a kernel is launched on it
  * (art_init allocates the default stream's), so launches on different streams
- * do not disturb each other.  At most 8 streams per device may do so, and a
+ * do not disturb each other.  At most 40 streams per device may do so, and a
  * stream's first such launch must happen outside graph capture (it allocates).
  * Host calls may come from several threads (the reference allows one: static
  * state, no locks, frameworks/pytorch/main_ops.cc:14-15).  Launches leave
