@@ -25,8 +25,10 @@
 //     pair, v_dot2_f32_f16 multiplies it with the matching pair of x and adds
 //     into fp32.  The constants 1024 / 64 leave together with the zero point,
 //     once per (group, column): s * (acc - 1024*sum(x_even) - 64*sum(x_odd) - z*sum(x));
-//   * the k lanes of a block meet in LDS (16 KiB), the owner of a column applies
-//     scale and zero point;
+//   * the eight k lanes of a wavefront meet by a reduce-scatter over lane bits 5, 4, 3 (v_permlane32_swap,
+//     v_permlane16_swap, row_ror:8 DPP): 16 -> 8 -> 4 -> 2 columns per lane, 30 vector operations; a wavefront is
+//     one quantisation group, so each lane applies scale and zero point to its two columns right there, and the
+//     four wavefronts of the block meet in 2 KiB of LDS;
 //   * the K-splits of a column meet in ONE returning 64-bit atomic per block:
 //     the partial sum travels as a fixed-point integer (steps of 2^-22) with an
 //     arrival count in the top byte and a count of non-finite partial sums in the
@@ -94,9 +96,24 @@ __device__ __forceinline__ float from_fixed(long long total) {
   return (total & 255) ? __builtin_nanf("") : (float)total * (1.f / kFix);
 }
 
+__device__ __forceinline__ float dpp_ror8(float v) {      // the value of lane ^ 8 (row_ror:8)
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+}
+// One step of a reduce-scatter between lanes l and l ^ 32 (l ^ 16): the lower lane of the pair keeps `a`, the upper
+// one keeps `b`; returns the pair's sum of what this lane keeps.  The swap exchanges the upper lanes' `a` with the
+// lower lanes' `b`, so both operands of the addition are the kept quantity afterwards.
+__device__ __forceinline__ float swap32_add(float a, float b) {
+  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned int, a), __builtin_bit_cast(unsigned int, b), false, false);
+  return __builtin_bit_cast(float, (unsigned int)r[0]) + __builtin_bit_cast(float, (unsigned int)r[1]);
+}
+__device__ __forceinline__ float swap16_add(float a, float b) {
+  auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned int, a), __builtin_bit_cast(unsigned int, b), false, false);
+  return __builtin_bit_cast(float, (unsigned int)r[0]) + __builtin_bit_cast(float, (unsigned int)r[1]);
+}
+
 // Sum over the 8 k lanes of a wavefront (lanes that share lane % 8); all lanes get the sum.
 __device__ __forceinline__ float sum_k_lanes_of_wave(float v) {
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));   // row_ror:8
+  v += dpp_ror8(v);
   {
     const unsigned int u = __builtin_bit_cast(unsigned int, v);
     auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
@@ -136,13 +153,14 @@ struct Fused {
   int att_parts;
 };
 
+// The register allocator is told that four wavefronts per SIMD are plenty (a launch has three): with the default
+// target of eight it postpones two of the eight weight loads until registers free up, a second memory round trip.
 template <int M, int MODE>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused, 3: x = merged split attention
-__global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_w4a16_kernel(
     const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight, const _Float16* __restrict__ scales,
     const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y, int K, int N, int splits,
     unsigned long long* __restrict__ slots, Magic magic, Fused fused) {
-  __shared__ __align__(16) float red[M][KL][CT];        // 16 KiB per row of x
-  __shared__ float aux[M][4][2];                        // per wavefront (= group): magic-number term, sum of x
+  __shared__ __align__(16) float part[M][4][CT];        // per wavefront (= group): scaled sums of the tile's columns
   __shared__ float s_ss[4];
   __shared__ __align__(16) unsigned int s_x[KL][CL];    // SwiGLU input, one fp16 pair per lane
 
@@ -198,14 +216,8 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     }
   }
 
-  // ---- every other global load of this lane
-  u32x4 w[R];
-  {
-    const unsigned char* wp = qweight + (size_t)r0c * N + n0c;
-#pragma unroll
-    // streamed once, never reused: the non-temporal hint measured 1-3 % faster on all four benchmark shapes
-    for (int i = 0; i < R; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + (size_t)i * N));
-  }
+  // ---- every other global load of this lane: x first (small, returns first), then the whole weight patch, then the
+  // scale and zero point of the two columns this lane holds after the reduce-scatter
   u32x4 xv[M][2];                                         // 16 halves of x per row of x
 #pragma unroll
   for (int m = 0; m < M; ++m) {
@@ -214,11 +226,27 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     xv[m][0] = xp[0];
     xv[m][1] = xp[1];
   }
+  u32x4 w[R];
+  {
+    const unsigned char* wp = qweight + (size_t)r0c * N + n0c;
+#pragma unroll
+    // streamed once, never reused: the non-temporal hint measured 1-3 % faster on all four benchmark shapes
+    for (int i = 0; i < R; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + (size_t)i * N));
+  }
+  const int pc = cl * 16 + 2 * (lane >> 3);               // column pair of this lane inside the tile (even)
+  const int pcol = tile * CT + pc;
+  const int pcolc = pcol < N ? pcol : 0;
+  const int groups = K >> 7;
+  const int g = split * 4 + wave;                         // the wavefront's quantisation group
+  const int gc = g < groups ? g : groups - 1;             // a group past the edge has x = 0: it contributes 0 * scale
+  const unsigned int sc2 = *reinterpret_cast<const unsigned int*>(scales + (size_t)gc * N + pcolc);
+  const unsigned char zb = qzeros[(size_t)gc * (N >> 1) + (pcolc >> 1)];
+  __builtin_amdgcn_sched_barrier(0);                      // nothing below may move above the loads, no load below them
   if (swiglu || attn) {       // part 2: pair -> LDS -> all 16 values of the k lane (same wavefront: no block barrier needed)
     half2_t o;
     if (swiglu) {
-      const half2_t g = as_h2(gpair), u = as_h2(upair);
-      const float g0f = (float)g.x, g1f = (float)g.y;
+      const half2_t gt = as_h2(gpair), u = as_h2(upair);
+      const float g0f = (float)gt.x, g1f = (float)gt.y;
       o = half2_t{(_Float16)(g0f / (1.0f + expf(0.0f - g0f)) * (float)u.x), (_Float16)(g1f / (1.0f + expf(0.0f - g1f)) * (float)u.y)};
     } else {                  // softmax merge: out = sum_p e^(m_p - M) acc_p / sum_p e^(m_p - M) l_p, rounded once to fp16
       float mm = -INFINITY;
@@ -241,19 +269,6 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     xv[0][0] = *reinterpret_cast<const u32x4*>(&s_x[kl][0]);
     xv[0][1] = *reinterpret_cast<const u32x4*>(&s_x[kl][4]);
-  }
-  // column owners (tid < 128) fetch scale and zero point of their column for the four groups of the block
-  const int col = tile * CT + tid;
-  const bool owner = (tid < CT) && (col < N);
-  const int colc = owner ? col : 0;
-  const int g0 = split * 4, groups = K >> 7;
-  _Float16 sc[4];
-  unsigned char zb[4];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const int gc = (g0 + g < groups) ? g0 + g : groups - 1;    // a group past the edge contributes 0 * scale
-    sc[g] = scales[(size_t)gc * N + colc];
-    zb[g] = qzeros[(size_t)gc * (N >> 1) + (colc >> 1)];
   }
   if (!k_ok) {
 #pragma unroll
@@ -330,52 +345,75 @@ __global__ __launch_bounds__(kThreads) void gemv_w4a16_kernel(
     }
   }
 
-  // ---- k lanes meet in LDS; the x-only terms of a group are the same for every column
+  // ---- the 8 k lanes of the wavefront meet by reduce-scatter (lane bits 5, 4, 3): afterwards this lane holds the
+  // group's sums of columns pc and pc + 1; the x-only terms of a group are the same for every column
+  const half2_t s2 = as_h2(sc2);
+  const float z0 = (float)(zb & 15), z1 = (float)(zb >> 4);
+  const bool upper8 = (lane & 8) != 0;
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    float* dst = &red[m][kl][cl * 16];
+    float v8[8], v4[4], v2[2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      *reinterpret_cast<f32x4*>(dst + 4 * j) = f32x4{acc[m][4 * j], acc[m][4 * j + 1], acc[m][4 * j + 2], acc[m][4 * j + 3]};
-    // se/so do not depend on the column lane: sum them over the 8 k lanes of the wavefront
-    const float se_g = sum_k_lanes_of_wave(se[m]), so_g = sum_k_lanes_of_wave(so[m]);
-    if (lane == 0) {
-      aux[m][wave][0] = 1024.f * se_g + 64.f * so_g;
-      aux[m][wave][1] = se_g + so_g;
+    for (int j = 0; j < 8; ++j) v8[j] = swap32_add(acc[m][j], acc[m][8 + j]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v4[j] = swap16_add(v8[j], v8[4 + j]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const float send = upper8 ? v4[j] : v4[2 + j], keep = upper8 ? v4[2 + j] : v4[j];
+      v2[j] = keep + dpp_ror8(send);
     }
+    const float se_g = sum_k_lanes_of_wave(se[m]), so_g = sum_k_lanes_of_wave(so[m]);
+    const float a0 = 1024.f * se_g + 64.f * so_g, a1 = se_g + so_g;
+    *reinterpret_cast<f32x2*>(&part[m][wave][pc]) = f32x2{(float)s2.x * (v2[0] - a0 - z0 * a1), (float)s2.y * (v2[1] - a0 - z1 * a1)};
   }
   __syncthreads();
-  if (!owner) return;
+  if (tid >= 64) return;
+  const int c2 = 2 * tid, col = tile * CT + c2;           // the first wavefront finishes two columns per lane
+  if (col >= N) return;
 
+  float r[M][2];
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    float r = 0.f;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      float a = 0.f;
-#pragma unroll
-      for (int q = 0; q < 8; ++q) a += red[m][g * 8 + q][tid];
-      const float z = (float)((col & 1) ? (zb[g] >> 4) : (zb[g] & 15));
-      r += (float)sc[g] * (a - aux[m][g][0] - z * aux[m][g][1]);
-    }
-    if (splits == 1) {
-      _Float16 o = (_Float16)r;
-      if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)fused.residual[col]);
-      y[(size_t)m * N + col] = o;
-      continue;
-    }
-    // one returning atomic: [arrival count : 8][fixed-point sum : 56]
-    unsigned long long* slot = slots + (size_t)m * N + col;
-    const long long mine = (1LL << 56) + to_fixed(r, splits);
-    const long long old = (long long)__hip_atomic_fetch_add(slot, (unsigned long long)mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (((old + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
-      const long long total = old + mine - ((long long)splits << 56);
-      _Float16 o = (_Float16)from_fixed(total);
-      if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)fused.residual[col]);
-      y[(size_t)m * N + col] = o;
-      *slot = 0ull;                     // ready for the next launch (stream order makes this visible)
-    }
+    const f32x2 p0 = *reinterpret_cast<const f32x2*>(&part[m][0][c2]), p1 = *reinterpret_cast<const f32x2*>(&part[m][1][c2]);
+    const f32x2 p2 = *reinterpret_cast<const f32x2*>(&part[m][2][c2]), p3 = *reinterpret_cast<const f32x2*>(&part[m][3][c2]);
+    r[m][0] = (p0[0] + p1[0]) + (p2[0] + p3[0]);
+    r[m][1] = (p0[1] + p1[1]) + (p2[1] + p3[1]);
   }
+  if (splits == 1) {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      half2_t o = {(_Float16)r[m][0], (_Float16)r[m][1]};
+      if (M == 1 && fused.residual != nullptr) {
+        const half2_t res = *reinterpret_cast<const half2_t*>(fused.residual + col);
+        o = half2_t{(_Float16)((float)o.x + (float)res.x), (_Float16)((float)o.y + (float)res.y)};
+      }
+      *reinterpret_cast<half2_t*>(y + (size_t)m * N + col) = o;
+    }
+    return;
+  }
+  // returning atomics, one per (row, column): [arrival count : 8][fixed-point sum : 56].  All of them go out before
+  // the first result is looked at, so the lane pays one round trip.
+  long long mine[M][2], old[M][2];
+#pragma unroll
+  for (int m = 0; m < M; ++m)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      mine[m][j] = (1LL << 56) + to_fixed(r[m][j], splits);
+      old[m][j] = (long long)__hip_atomic_fetch_add(slots + (size_t)m * N + col + j, (unsigned long long)mine[m][j], __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+  for (int m = 0; m < M; ++m)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (((old[m][j] + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
+        const long long total = old[m][j] + mine[m][j] - ((long long)splits << 56);
+        _Float16 o = (_Float16)from_fixed(total);
+        if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)fused.residual[col + j]);
+        y[(size_t)m * N + col + j] = o;
+        slots[(size_t)m * N + col + j] = 0ull;            // ready for the next launch (stream order makes this visible)
+      }
+    }
 }
 
 // Split-K accumulators of the entry point that allocates nothing (art_gemv_w4a16_noalloc): 64-bit slots, one per
@@ -422,6 +460,7 @@ extern "C" int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const 
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0,
               "art_gemv_w4a16: x and qweight must be 16-byte aligned");
+  ART_REQUIRE(((uintptr_t)y_dev % 4) == 0 && ((uintptr_t)scales_dev % 4) == 0, "art_gemv_w4a16: y and scales must be 4-byte aligned");
   ART_REQUIRE(M >= 1 && M <= 8, "art_gemv_w4a16: M must be in 1..8 (got %d); larger batches go through art_gemm_w4a16", M);
   // blocks of one column tile write y while blocks of other tiles still read x
   ART_REQUIRE(!art::overlaps(x_dev, (size_t)M * K * 2, y_dev, (size_t)M * N * 2), "art_gemv_w4a16: y must not overlap x");
@@ -458,6 +497,7 @@ extern "C" int art_gemv_w4a16_noalloc(const void* x_dev, const void* qweight_dev
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_noalloc: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0,
               "art_gemv_w4a16_noalloc: x and qweight must be 16-byte aligned");
+  ART_REQUIRE(((uintptr_t)y_dev % 4) == 0 && ((uintptr_t)scales_dev % 4) == 0, "art_gemv_w4a16_noalloc: y and scales must be 4-byte aligned");
   ART_REQUIRE(M >= 1 && M <= 4, "art_gemv_w4a16_noalloc: M must be in 1..4 (got %d)", M);
   ART_REQUIRE((long long)M * N <= kNoAllocSlots, "art_gemv_w4a16_noalloc: M * N = %lld exceeds the %d accumulators of the built-in scratch array",
               (long long)M * N, kNoAllocSlots);
@@ -482,6 +522,8 @@ extern "C" int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, 
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_fused: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0 && ((uintptr_t)norm_weight_dev % 16) == 0,
               "art_gemv_w4a16_fused: x, qweight and the norm weight must be 16-byte aligned");
+  ART_REQUIRE(((uintptr_t)y_dev % 4) == 0 && ((uintptr_t)scales_dev % 4) == 0 && ((uintptr_t)residual_dev % 4) == 0,
+              "art_gemv_w4a16_fused: y, scales and the residual must be 4-byte aligned");
   // blocks of one column tile write y while blocks of other tiles still read x: only the residual may alias y
   ART_REQUIRE(!art::overlaps(x_dev, (size_t)(swiglu_input ? 2 : 1) * K * 2, y_dev, (size_t)N * 2),
               "art_gemv_w4a16_fused: y must not overlap x (it may alias the residual)");
@@ -497,6 +539,8 @@ extern "C" int art_gemv_w4a16_attn(const void* partial_dev, int parts, const voi
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_attn: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)partial_dev % 16) == 0,
               "art_gemv_w4a16_attn: partial records and qweight must be 16-byte aligned");
+  ART_REQUIRE(((uintptr_t)y_dev % 4) == 0 && ((uintptr_t)scales_dev % 4) == 0 && ((uintptr_t)residual_dev % 4) == 0,
+              "art_gemv_w4a16_attn: y, scales and the residual must be 4-byte aligned");
   ART_REQUIRE(!art::overlaps(partial_dev, (size_t)(K / 128) * parts * 132 * 4, y_dev, (size_t)N * 2),
               "art_gemv_w4a16_attn: y must not overlap the partial records");
   Fused f{nullptr, (const _Float16*)residual_dev, nullptr, 0.f, 0.f, (const float*)partial_dev, parts};
