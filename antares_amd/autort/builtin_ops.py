@@ -27,6 +27,53 @@ class PartitionEvenFirst:
     of the classify / cumsum / bucket pipeline of samples/01_sort_even_first.py:9-27
     in one fused operator."""
     name = 'partition_even_first_i32'
+    BLOCK_CAPS = (1024, 512, 2048, 256, 4096)          # values of the launch parameter a tuning run tries, default first
+
+    def __init__(self):
+        self.tuned = {}                                 # str(n) -> {'value': cap on blocks, 'us': ...}
+        self._loaded = False
+
+    def _saved(self):
+        """Winners of earlier tuning runs, kept in the operator store as `partition_even_first_i32.tuned.json`."""
+        if not self._loaded:
+            self._loaded = True
+            import json
+            import os
+            from . import store
+            try:
+                with open(os.path.join(store.ops_dir(), self.name + '.tuned.json')) as f:
+                    self.tuned.update(json.load(f))
+            except (OSError, ValueError):
+                pass
+        return self.tuned
+
+    def persist(self):
+        import json
+        import os
+        from . import store
+        try:
+            os.makedirs(store.ops_dir(), exist_ok=True)
+            path = os.path.join(store.ops_dir(), self.name + '.tuned.json')
+            with open(f'{path}.{os.getpid()}.tmp', 'w') as f:
+                json.dump(self.tuned, f, sort_keys=True)
+            os.replace(f'{path}.{os.getpid()}.tmp', path)
+        except OSError:
+            pass
+
+    def _launch(self, x, out, cap):
+        capi.check(capi.lib().art_partition_even_first_i32_tuned(c_void_p(x.data_ptr()), c_void_p(out.data_ptr()), x.numel(),
+                                                                int(cap), c_void_p(current_stream_handle())))
+
+    def tune(self, x: torch.Tensor, trials: int = 5):
+        """Times up to `trials` caps on the number of blocks for vectors of x's length (on rotating copies of x, into
+        scratch outputs) and keeps the fastest for later calls and later sessions; returns the record."""
+        from .patterns import tune_hand_kernel
+        _require_cuda(x)
+        n = x.numel()
+        copies = max(1, min(4, (256 << 20) // max(8 * n, 1)))
+        clones = [(x if c == 0 else x.clone(), torch.empty_like(x)) for c in range(copies)]
+        self.config = {}
+        return tune_hand_kernel(self, str(n), list(self.BLOCK_CAPS), lambda v, t: self._launch(t[0], t[1], v), trials, clones)
 
     def __call__(self, x: torch.Tensor, out: torch.Tensor = None, extra=None):
         if x.dtype != torch.int32 or x.dim() != 1:
@@ -36,8 +83,8 @@ class PartitionEvenFirst:
         if out.dtype != torch.int32 or out.numel() != x.numel():
             raise TypeError('partition_even_first_i32: out must be int32 with as many elements as the input')
         _require_cuda(x, out)
-        capi.check(capi.lib().art_partition_even_first_i32(c_void_p(x.data_ptr()), c_void_p(out.data_ptr()),
-                                                          x.numel(), c_void_p(current_stream_handle())))
+        saved = self._saved().get(str(x.numel()))
+        self._launch(x, out, saved['value'] if saved else 0)
         return out
 
 

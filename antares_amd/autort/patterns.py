@@ -85,6 +85,32 @@ W4A16_INPUTS = ['x=float16[M:1, K:4096]', 'qweight=int8[KH:2048, N:11008]', 'sca
                 'qzeros=int8[G:32, NH:5504]']
 
 
+def tune_hand_kernel(op, key: str, candidates, run, trials: int, clones):
+    """``config="tune:N"`` for a hand-written kernel: times up to N values of its launch parameter for the shape of
+    this call (the reference's tuner walks the knob space of the schedule that runs, tuner/OpEvo/main.py:467-616; a
+    hand kernel has one knob with a handful of values, so the walk is exhaustive up to N).  ``run(value, tensors)``
+    enqueues one launch; ``clones`` yields sets of operand tensors - the timing rotates over several copies, since
+    one buffer launched over and over would be served by the memory-side cache and favour the wrong choice - whose
+    outputs are scratch, never the caller's.  The winner is kept in ``op.tuned[key]`` and in the module file."""
+    sets = list(clones)
+    stream = torch.cuda.current_stream().cuda_stream
+    best = None
+    for value in candidates[:max(1, trials)]:
+        run(value, sets[0])                                   # warm-up (and the first use of a code path)
+        start, stop = capi.Event(), capi.Event()
+        start.record(stream)
+        runs = max(6, 2 * len(sets))
+        for i in range(runs):
+            run(value, sets[i % len(sets)])
+        stop.record(stream)
+        us = start.elapsed_ms(stop) * 1e3 / runs
+        if best is None or us < best['us']:
+            best = {'value': int(value), 'us': round(us, 3)}
+    op.tuned[key] = best
+    op.persist()
+    return best
+
+
 def _w4a16_handler(op, bound, env, stream) -> bool:
     r = op.fast_roles
     x, q, s, z, y = bound[r['x']], bound[r['qweight']], bound[r['scales']], bound[r['qzeros']], bound[r['y']]
@@ -96,9 +122,26 @@ def _w4a16_handler(op, bound, env, stream) -> bool:
     # the vector-unit kernel streams the weights once per four rows (7.5 / 11.1 / 13.0 / 15.3 us for 1..4 rows of
     # 4096 x 11008, 22 us for five), the matrix-core kernel once per 64 rows (16 us for 4..32 rows): four rows and
     # more go there
-    entry = capi.lib().art_gemv_w4a16 if M <= 3 else capi.lib().art_gemm_w4a16
-    capi.check(entry(c_void_p(x.data_ptr()), c_void_p(q.data_ptr()), c_void_p(s.data_ptr()),
-                                        c_void_p(z.data_ptr()), c_void_p(y.data_ptr()), M, K, N, c_void_p(stream)))
+    lib = capi.lib()
+    gemv = M <= 3
+    entry = lib.art_gemv_w4a16_tuned if gemv else lib.art_gemm_w4a16_tuned
+
+    def run(value, t, st=None):
+        capi.check(entry(c_void_p(t[0].data_ptr()), c_void_p(t[1].data_ptr()), c_void_p(t[2].data_ptr()), c_void_p(t[3].data_ptr()),
+                         c_void_p(t[4].data_ptr()), M, K, N, int(value), c_void_p(stream if st is None else st)))
+
+    # the launch parameter of the kernel that runs: rows per lane of the GEMV (0 = 8, or 4), K-splits of the GEMM
+    key = f"{'gemv_w4a16.rows_per_lane' if gemv else 'gemm_w4a16.k_splits'}|{M},{K},{N}"
+    saved = op.tuned.get(key)
+    trials = op.config.get('tune')
+    if saved is None and isinstance(trials, int) and trials > 0 and not torch.cuda.is_current_stream_capturing():
+        per_set = q.numel() + 2 * s.numel() + z.numel()
+        copies = max(1, min(8, (256 << 20) // max(per_set, 1)))
+        clones = [(x, q.clone(), s.clone(), z.clone(), torch.empty_like(y)) for _ in range(copies)]
+        cands = [8, 4] if gemv else [0] + [v for v in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32) if v <= K // 128]
+        saved = tune_hand_kernel(op, key, cands, lambda v, t: run(v, t, torch.cuda.current_stream().cuda_stream), trials, clones)
+        del clones
+    run(saved['value'] if saved is not None else 0, (x, q, s, z, y))
     return True
 
 

@@ -316,6 +316,12 @@ int choose_splits(int rows, int N, int K, size_t scratch_bytes, int compute_unit
 
 extern "C" int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                               void* y_dev, int M, int K, int N, void* stream) {
+  return art_gemm_w4a16_tuned(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, M, K, N, 0, stream);
+}
+
+extern "C" int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                                    void* y_dev, int M, int K, int N, int k_splits, void* stream) {
+  ART_REQUIRE(k_splits >= 0, "art_gemm_w4a16: k_splits must be 0 (library's choice) or positive (got %d)", k_splits);
   ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemm_w4a16: null pointer");
   ART_REQUIRE(M >= 1, "art_gemm_w4a16: M must be positive (got %d)", M);
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemm_w4a16: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
@@ -342,7 +348,12 @@ extern "C" int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const 
   const int G = K / GK, col_tiles = (N + BN - 1) / BN;
   for (int m0 = 0; m0 < M; m0 += BM) {      // 64 rows of x per pass over the weights
     const int rows = M - m0 < BM ? M - m0 : BM;
-    const int splits = choose_splits(rows, N, K, scratch_bytes, compute_units);
+    int splits = choose_splits(rows, N, K, scratch_bytes, compute_units);
+    if (k_splits > 0) {           // the caller's choice, within what the kernel and the scratch space take
+      const int cap = (int)(scratch_bytes / ((size_t)rows * N * sizeof(float)));
+      splits = k_splits > G ? G : k_splits;
+      if (splits > cap) splits = cap < 1 ? 1 : cap;
+    }
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m0 * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m0 * N;
     const dim3 grid(col_tiles * splits);

@@ -76,11 +76,12 @@ __device__ __forceinline__ void mac_word_pair(unsigned int a, unsigned int b, ha
 }
 
 constexpr int kThreads = 256;
-constexpr int R = 8;                   // packed rows per lane
 constexpr int CL = 8;                  // column lanes per block
-constexpr int KL = kThreads / CL;      // 32 k lanes per block, 8 per wavefront = one group of 128 k
+constexpr int KL = kThreads / CL;      // 32 k lanes per block, 8 per wavefront
 constexpr int CT = 16 * CL;            // 128 columns per block
-constexpr int kRowsPerBlock = KL * R;  // 256 packed rows = 512 values of k
+// Packed rows per lane, R, is a launch parameter (template): 8 rows make a block 128 columns x 512 k with each
+// wavefront on exactly one quantisation group of 128 k; 4 rows make it 128 x 256 with two wavefronts per group -
+// twice the blocks (and twice the returning atomics), which pays when 8 rows leave compute units without a block.
 constexpr float kFix = 1073741824.f;   // 2^30
 
 // A partial sum on its way through the 64-bit slot: a multiple of 256 in units of 2^-30 (so 2^-22 is the step), which
@@ -155,12 +156,14 @@ struct Fused {
 
 // The register allocator is told that four wavefronts per SIMD are plenty (a launch has three): with the default
 // target of eight it postpones two of the eight weight loads until registers free up, a second memory round trip.
-template <int M, int MODE>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused, 3: x = merged split attention
+template <int M, int MODE, int R>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused, 3: x = merged split attention
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_w4a16_kernel(
     const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight, const _Float16* __restrict__ scales,
     const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y, int K, int N, int splits,
     unsigned long long* __restrict__ slots, Magic magic, Fused fused) {
-  __shared__ __align__(16) float part[M][4][CT];        // per wavefront (= group): scaled sums of the tile's columns
+  static_assert(R == 8 || (R == 4 && MODE == 0), "the fused prologues are written for 8 rows per lane");
+  constexpr int kRowsPerBlock = KL * R;                 // packed rows per block: 256 (512 values of k) or 128
+  __shared__ __align__(16) float part[M][4][CT];        // per wavefront: scaled sums of the tile's columns
   __shared__ float s_ss[4];
   __shared__ __align__(16) unsigned int s_x[KL][CL];    // SwiGLU input, one fp16 pair per lane
 
@@ -181,7 +184,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
   // still in flight; issued after the weights they would wait for the whole stream.
   constexpr bool norm = (M == 1) && (MODE == 1);
   u32x4 sq[2];
-  if (norm) {
+  if constexpr (norm) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int c = tid + i * kThreads;
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
   // computes one pair; its two loads also go out ahead of the weight stream.
   constexpr bool swiglu = (M == 1) && (MODE == 2);
   unsigned int gpair = 0, upair = 0;
-  if (swiglu) {
+  if constexpr (swiglu) {
     const int k = 2 * r0c + 2 * cl;
     gpair = *reinterpret_cast<const unsigned int*>(fused.gate_up + k);
     upair = *reinterpret_cast<const unsigned int*>(fused.gate_up + K + k);
@@ -205,7 +208,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
   constexpr bool attn = (M == 1) && (MODE == 3);
   constexpr int kMaxParts = art::kMaxAttnParts, kPartStride = 132;         // record layout of the attention kernel
   f32x2 pacc[kMaxParts], pml[kMaxParts];
-  if (attn) {
+  if constexpr (attn) {
     const int k = 2 * r0c + 2 * cl, head = k >> 7, d = k & 127;
     const float* rec = fused.att_partial + (size_t)head * fused.att_parts * kPartStride;
 #pragma unroll
@@ -218,13 +221,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
 
   // ---- every other global load of this lane: x first (small, returns first), then the whole weight patch, then the
   // scale and zero point of the two columns this lane holds after the reduce-scatter
-  u32x4 xv[M][2];                                         // 16 halves of x per row of x
+  u32x4 xv[M][R / 4];                                     // 2 R halves of x per row of x
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     if (swiglu || attn) continue;
     const u32x4* xp = reinterpret_cast<const u32x4*>(x + (size_t)m * K + 2 * r0c);
-    xv[m][0] = xp[0];
-    xv[m][1] = xp[1];
+#pragma unroll
+    for (int i = 0; i < R / 4; ++i) xv[m][i] = xp[i];
   }
   u32x4 w[R];
   {
@@ -237,12 +240,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
   const int pcol = tile * CT + pc;
   const int pcolc = pcol < N ? pcol : 0;
   const int groups = K >> 7;
-  const int g = split * 4 + wave;                         // the wavefront's quantisation group
+  const int g = (split * kRowsPerBlock * 2 + wave * 16 * R) >> 7;      // the wavefront's quantisation group
   const int gc = g < groups ? g : groups - 1;             // a group past the edge has x = 0: it contributes 0 * scale
   const unsigned int sc2 = *reinterpret_cast<const unsigned int*>(scales + (size_t)gc * N + pcolc);
   const unsigned char zb = qzeros[(size_t)gc * (N >> 1) + (pcolc >> 1)];
   __builtin_amdgcn_sched_barrier(0);                      // nothing below may move above the loads, no load below them
-  if (swiglu || attn) {       // part 2: pair -> LDS -> all 16 values of the k lane (same wavefront: no block barrier needed)
+  if constexpr (swiglu || attn) {       // part 2: pair -> LDS -> all 16 values of the k lane (same wavefront: no block barrier needed)
     half2_t o;
     if (swiglu) {
       const half2_t gt = as_h2(gpair), u = as_h2(upair);
@@ -272,15 +275,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
   }
   if (!k_ok) {
 #pragma unroll
-    for (int m = 0; m < M; ++m) {
-      xv[m][0] = u32x4{0, 0, 0, 0};
-      xv[m][1] = u32x4{0, 0, 0, 0};
-    }
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int i = 0; i < R / 4; ++i) xv[m][i] = u32x4{0, 0, 0, 0};
   }
 
   // ---- fused RMSNorm, part 2 (while the weight loads are in flight): sum of squares over all of x.
   // Every block recomputes it from the 2*K bytes of x (served by L2) rather than waiting for another kernel.
-  if (norm) {
+  if constexpr (norm) {
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -426,11 +428,13 @@ unsigned long long* g_scratch_ptr[kMaxDevices];          // device address of `s
 
 template <int M>
 int launch(const void* x, const void* qw, const void* sc, const void* qz, void* y, int K, int N, hipStream_t stream,
-           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0}, unsigned long long* slots = nullptr) {
+           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0}, unsigned long long* slots = nullptr,
+           int rows_per_lane = 8) {
   const int rows = K / 2;
   const int tiles = (N + CT - 1) / CT;
-  const int splits = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-  ART_REQUIRE(splits <= 127, "art_gemv_w4a16: K too large (%d)", K);
+  const int rows_per_block = KL * rows_per_lane;
+  const int splits = (rows + rows_per_block - 1) / rows_per_block;
+  ART_REQUIRE(splits <= 127, "art_gemv_w4a16: K too large (%d) for %d rows per lane", K, rows_per_lane);
   if (slots == nullptr) {         // the library's own workspace for this stream
     art::Workspace* wsp = art::workspace(stream);
     if (!wsp) return 1;
@@ -439,14 +443,15 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
   }
   const Magic magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
   const dim3 grid(tiles, splits), block(kThreads);
-#define ART_GEMV_LAUNCH(MODE)                                                                                          \
-  gemv_w4a16_kernel<M, MODE><<<grid, block, 0, stream>>>((const _Float16*)x, (const unsigned char*)qw, (const _Float16*)sc, \
-                                                         (const unsigned char*)qz, (_Float16*)y, K, N, splits, slots, magic, fused)
+#define ART_GEMV_LAUNCH(MODE, R)                                                                                          \
+  gemv_w4a16_kernel<M, MODE, R><<<grid, block, 0, stream>>>((const _Float16*)x, (const unsigned char*)qw, (const _Float16*)sc, \
+                                                            (const unsigned char*)qz, (_Float16*)y, K, N, splits, slots, magic, fused)
   // the plain product is its own instantiation: it carries none of the fused prologues
-  if (M == 1 && fused.norm_w != nullptr) ART_GEMV_LAUNCH(1);
-  else if (M == 1 && fused.gate_up != nullptr) ART_GEMV_LAUNCH(2);
-  else if (M == 1 && fused.att_partial != nullptr) ART_GEMV_LAUNCH(3);
-  else ART_GEMV_LAUNCH(0);
+  if (M == 1 && fused.norm_w != nullptr) ART_GEMV_LAUNCH(1, 8);
+  else if (M == 1 && fused.gate_up != nullptr) ART_GEMV_LAUNCH(2, 8);
+  else if (M == 1 && fused.att_partial != nullptr) ART_GEMV_LAUNCH(3, 8);
+  else if (rows_per_lane == 4) ART_GEMV_LAUNCH(0, 4);
+  else ART_GEMV_LAUNCH(0, 8);
 #undef ART_GEMV_LAUNCH
   ART_LAUNCH_CHECK();
   return 0;
@@ -456,6 +461,14 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
 
 extern "C" int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                               void* y_dev, int M, int K, int N, void* stream) {
+  return art_gemv_w4a16_tuned(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, M, K, N, 0, stream);
+}
+
+extern "C" int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                                    void* y_dev, int M, int K, int N, int rows_per_lane, void* stream) {
+  ART_REQUIRE(rows_per_lane == 0 || rows_per_lane == 4 || rows_per_lane == 8,
+              "art_gemv_w4a16: rows_per_lane must be 0 (library's choice), 4 or 8 (got %d)", rows_per_lane);
+  const int rpl = rows_per_lane ? rows_per_lane : 8;
   ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16: null pointer");
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0,
@@ -470,10 +483,11 @@ extern "C" int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const 
     const int step = (M - m >= 4) ? 4 : (M - m);
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m * N;
-    int rc = step == 4 ? launch<4>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st)
-           : step == 3 ? launch<3>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st)
-           : step == 2 ? launch<2>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st)
-                       : launch<1>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st);
+    const Fused none{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0};
+    int rc = step == 4 ? launch<4>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl)
+           : step == 3 ? launch<3>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl)
+           : step == 2 ? launch<2>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl)
+                       : launch<1>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl);
     if (rc) return rc;
     m += step;
   }

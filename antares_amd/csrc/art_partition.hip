@@ -9,10 +9,11 @@
 //   count    block b reads its span of the input (a whole number of
 //            4096-element tiles) and stores the number of even values in
 //            counts[b].
-//   scatter  block b adds up counts[0..b) and counts[b..B) (B <= 1024 words,
-//            served by L2) to get the number of evens before its span and the
-//            total; then, tile by tile, it ranks the even values with a
-//            wavefront prefix + a 4-wave prefix through LDS, compacts evens
+//   scatter  block b adds up counts[0..b) and counts[b..B) (B = 1024 words unless
+//            the caller chooses otherwise, served by L2) to get the number of
+//            evens before its span and the total; then, tile by tile, it ranks
+//            the even values with wavefront ballots (v_mbcnt for the lanes below,
+//            a population count for the total) + a 4-wave prefix through LDS, compacts evens
 //            and odds of the tile in LDS and writes both runs with fully
 //            coalesced 16-byte non-temporal stores:
 //              even -> out[evens_before + rank]
@@ -117,19 +118,21 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
       for (int j = 0; j < kVecPerThread; ++j) vn[j] = load_vec<true>(in, base + kTile, j, n);
     }
     const long long valid = (n - base < kTile) ? (n - base) : kTile;      // elements of this tile that exist
-    unsigned int cnt[kVecPerThread], incl[kVecPerThread];
-    // inclusive prefix of the per-vector even counts over the lanes of the wavefront
+    // Evens of vector j in the lanes below this one, and in the whole wavefront: one ballot per element slot, the
+    // lanes below counted with v_mbcnt, the wavefront total with a scalar population count.
+    unsigned int excl[kVecPerThread];
 #pragma unroll
     for (int j = 0; j < kVecPerThread; ++j) {
-      cnt[j] = even_count4(v[j]);
-      unsigned int p = cnt[j];
+      const int items[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+      unsigned int below = 0, total = 0;
 #pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const unsigned int up = __shfl_up(p, off, 64);
-        if (lane >= off) p += up;
+      for (int e = 0; e < 4; ++e) {
+        const unsigned long long m = __ballot((items[e] & 1) == 0);
+        below = __builtin_amdgcn_mbcnt_hi((unsigned int)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned int)m, below));
+        total += (unsigned int)__popcll(m);
       }
-      incl[j] = p;
-      if (lane == 63) s_wave[wave][j] = p;
+      excl[j] = below;
+      if (lane == 0) s_wave[wave][j] = total;
     }
     art_lds_barrier();
     // evens before (j, wave, lane) in tile order (j outermost, then thread id)
@@ -142,7 +145,7 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
         if (w < wave) acc += s_wave[w][j];
         tile_even += s_wave[w][j];
       }
-      before[j] = acc + incl[j] - cnt[j];
+      before[j] = acc + excl[j];
     }
     // compact into LDS: evens to [0, tile_even), odds to [tile_even, kTile)
 #pragma unroll
@@ -189,6 +192,12 @@ __global__ __launch_bounds__(kThreads) void partition_scatter_kernel(const int* 
 }  // namespace
 
 extern "C" int art_partition_even_first_i32(const void* in_dev, void* out_dev, long long n, void* stream) {
+  return art_partition_even_first_i32_tuned(in_dev, out_dev, n, 0, stream);
+}
+
+extern "C" int art_partition_even_first_i32_tuned(const void* in_dev, void* out_dev, long long n, int max_blocks, void* stream) {
+  ART_REQUIRE(max_blocks == 0 || (max_blocks >= 64 && max_blocks <= 16384),
+              "art_partition_even_first_i32: max_blocks must be 0 (library's choice) or in 64..16384 (got %d)", max_blocks);
   ART_REQUIRE(n >= 0, "art_partition_even_first_i32: negative length");
   if (n == 0) return 0;
   ART_REQUIRE(in_dev && out_dev && in_dev != out_dev, "art_partition_even_first_i32: null or aliased pointers");
@@ -198,7 +207,7 @@ extern "C" int art_partition_even_first_i32(const void* in_dev, void* out_dev, l
   if (!wsp) return 1;
   art::Workspace& ws = *wsp;
   const long long tiles = (n + kTile - 1) / kTile;
-  constexpr long long kMaxBlocks = 1024;                        // bounds the counts every block adds up (4 KiB from L2)
+  const long long kMaxBlocks = max_blocks ? max_blocks : 1024;  // bounds the counts every block adds up (4 KiB from L2 at 1024)
   const int tiles_per_block = (int)((tiles + kMaxBlocks - 1) / kMaxBlocks);
   const int blocks = (int)((tiles + tiles_per_block - 1) / tiles_per_block);
   unsigned int* counts = reinterpret_cast<unsigned int*>(reinterpret_cast<char*>(ws.base) + art::kScratchOffset);

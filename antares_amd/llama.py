@@ -289,6 +289,49 @@ class LlamaInt4Decoder:
                                          norm_weight=self.w['final_norm'], eps=cfg.rms_eps)
         return self.logits
 
+    def tune_att_parts(self, pos: int, candidates=(8, 4, 2, 1), runs: int = 20) -> Dict[str, object]:
+        """The decode attention's launch parameter - blocks per head - for a cache filled up to `pos`: times the
+        attention + o-projection pair of every layer for each candidate and keeps the fastest in `self.att_parts`
+        (call before `capture`; the caches are used as scratch only in row `pos`, which a real step rewrites)."""
+        if not self.fused:
+            raise RuntimeError('the unfused decoder has no split attention to tune')
+        from .runtime import capi
+        ops = self.autort.ops
+        saved_pos = self.pos.clone()
+        self.pos.fill_(pos)
+        best = None
+        stream = torch.cuda.current_stream().cuda_stream
+        for parts in candidates:
+            partial = torch.zeros(self.cfg.n_heads, max(parts, 2), 132, dtype=torch.float32, device=self.dev)
+
+            def pair(l, lw):
+                o = lw['o']
+                if parts > 1:
+                    ops.attention_rope_split_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f,
+                                                 partial, extra=[self.pos])
+                    ops.gemv_w4a16_attn(partial, o['qweight'], o['scales'], o['qzeros'], self.proj)
+                else:
+                    ops.attention_rope_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f, self.att,
+                                           extra=[self.pos])
+                    ops.gemv_w4a16_fused(self.att.view(-1), o['qweight'], o['scales'], o['qzeros'], self.proj)
+            pair(0, self.w['layers'][0])
+            start, stop = capi.Event(), capi.Event()
+            start.record(stream)
+            n = 0
+            while n < runs:
+                for l, lw in enumerate(self.w['layers']):
+                    pair(l, lw)
+                    n += 1
+            stop.record(stream)
+            us = start.elapsed_ms(stop) * 1e3 / n
+            if best is None or us < best['us']:
+                best = {'value': parts, 'us': round(us, 3)}
+        self.pos.copy_(saved_pos)
+        self.att_parts = best['value']
+        self.att_partial = torch.zeros(self.cfg.n_heads, max(self.att_parts, 2), 132, dtype=torch.float32, device=self.dev)
+        self.graph = None
+        return best
+
     def advance(self, prompt: Optional[torch.Tensor] = None):
         """pos <- pos + 1; token <- prompt[pos] while the prompt lasts, else argmax(logits).
         All on the device, so it can be part of the recorded graph.  The fused decoder does it in one launch,

@@ -135,6 +135,19 @@ int art_read_bytes(const void* src_dev, size_t bytes, void* sink_dev, void* stre
 int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                    void* y_dev, int M, int K, int N, void* stream);
 
+/* The same three operators with the launch parameter a tuning run may vary (the knobs that
+ * `config="tune:N"` searches, as the reference's tuner searches the knobs of its schedules:
+ * tuner/OpEvo/main.py:467-616, antares/common.py:81-118).  0 always means the library's own choice, and results do
+ * not depend on the parameter beyond fp32 re-association.
+ *   rows_per_lane: 4 or 8 packed rows per lane = 256 or 512 values of k per block of the int4 GEMV;
+ *   k_splits:      number of K-splits of the int4 GEMM (clamped to K/128 and to what the workspace holds);
+ *   max_blocks:    cap on the blocks of the partition, 64..16384 (each walks its span tile by tile). */
+int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                         void* y_dev, int M, int K, int N, int rows_per_lane, void* stream);
+int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                         void* y_dev, int M, int K, int N, int k_splits, void* stream);
+int art_partition_even_first_i32_tuned(const void* in_dev, void* out_dev, long long n, int max_blocks, void* stream);
+
 /* art_gemv_w4a16 for callers that cannot allocate device memory or let a library do it (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
  * operands, constraints and results (bit for bit) as art_gemv_w4a16, with M in 1..4 and M * N <= 131072: the

@@ -184,3 +184,25 @@ def test_full_width_decode_matches_the_oracle(graph):
                 want_c = want_c.astype(np.float32)
                 assert np.allclose(got_c.float().cpu().numpy(), want_c, rtol=2e-2, atol=2e-2 * max(1.0, float(want_c.std()))), \
                     (pos, l, np.abs(got_c.float().cpu().numpy() - want_c).max(), float(want_c.std()))
+
+
+def test_attention_blocks_per_head_can_be_tuned_and_the_step_still_matches_the_oracle():
+    """`tune_att_parts` times the attention + o-projection pair for each number of blocks per head and keeps the
+    fastest; whatever it picks, the next decode steps match the oracle."""
+    from antares_amd.llama import LlamaInt4Decoder, random_weights
+    from oracle.llama_ref import LlamaRef
+    cfg = small_config()
+    w = random_weights(cfg, seed=6)
+    ref = LlamaRef(cfg, w)
+    dec = LlamaInt4Decoder(cfg, w, fused=True, att_parts=8)
+    tokens = [9, 100, 731, 2]
+    for pos, tok in enumerate(tokens):
+        want = ref.forward(tok, pos).astype(np.float32)
+        if pos == 2:
+            print('[case] tune blocks per head', flush=True)
+            rec = dec.tune_att_parts(pos=pos, candidates=(8, 4, 2, 1), runs=8)
+            assert rec['value'] in (8, 4, 2, 1) and rec['us'] > 0 and dec.att_parts == rec['value']
+        print(f'[case] step {pos} with {dec.att_parts} blocks per head', flush=True)
+        dec.reset(tok, pos)
+        got = dec.step().float().cpu().numpy()
+        assert np.allclose(got, want, **LOGIT_TOL), (pos, np.abs(got - want).max())

@@ -425,3 +425,39 @@ def test_split_k_launches_on_two_streams_do_not_disturb_each_other(autort):
     rc = capi.lib().art_gemv_w4a16_fused(c_void_p(x.data_ptr()), c_void_p(a[1].data_ptr()), c_void_p(a[2].data_ptr()),
                                          c_void_p(a[3].data_ptr()), c_void_p(x.data_ptr()), 11008, 4096, None, 1e-5, None, 0, None)
     assert rc != 0 and b'overlap' in capi.lib().art_last_error()
+
+
+def test_fp16_reductions_where_tree_order_leaves_the_sequential_oracle(autort):
+    """A reduction written in fp16 accumulates in fp16 on both sides (the reference's rule), but the GPU adds in tree
+    order and the oracle in index order.  For 64 to 1024 terms of N(0,1) data the GPU stays within the fp16 tolerance
+    of the float64 sum; the sequential oracle itself drifts from it (0.03 at 64 terms, 0.4 at 1024, where 1e-2 of the
+    result's size is 0.3), so the two are compared with the oracle's own drift added to the tolerance.  Far beyond
+    that they part for good: 16384 positive terms stall a sequential fp16 sum (at 2048 an addend below 1 is rounded
+    away), while the tree keeps adding numbers of similar size - there the GPU result must be the one closer to the
+    float64 sum, and within the fp16 tolerance of it."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    dev = autort.device()
+    ir = 'output0[N] +=! input0[N, C]'
+    for C in (64, 256, 1024):
+        note(f'fp16 row sums, C={C}')
+        x = torch.randn(48, C, generator=torch.Generator().manual_seed(C)).half()
+        f = autort.export(ir=ir, inputs=[f'input0=float16[48, {C}]'], name=f'rowsum_f16_{C}')
+        got = f(x.to(dev)).float().cpu().numpy()
+        want = CpuModule(parse_program(ir, {'input0': {'dtype': 'float16', 'shape': [48, C]}}), fast_math=False)(input0=x.numpy())['output0']
+        exact = x.double().sum(1).numpy()
+        # sums of C terms of unit variance: sqrt(C) in size; fp16 keeps 2^-11 of that per addition
+        tol = 1e-2 * max(1.0, C ** 0.5)
+        assert np.abs(got - exact).max() <= tol, (C, np.abs(got - exact).max())
+        drift = np.abs(want.astype(np.float64) - exact).max()
+        assert np.abs(got - want.astype(np.float32)).max() <= tol + drift, (C, np.abs(got - want.astype(np.float32)).max(), drift)
+    C = 16384
+    note(f'fp16 row sums of positive data, C={C}')
+    x = torch.rand(8, C, generator=torch.Generator().manual_seed(7)).half()
+    f = autort.export(ir=ir, inputs=[f'input0=float16[8, {C}]'], name=f'rowsum_f16_{C}')
+    got = f(x.to(dev)).float().cpu().numpy()
+    want = CpuModule(parse_program(ir, {'input0': {'dtype': 'float16', 'shape': [8, C]}}), fast_math=False)(input0=x.numpy())['output0'].astype(np.float32)
+    exact = x.double().sum(1).numpy()                      # about 8192
+    assert np.all(want < 0.5 * exact)                      # the sequential fp16 sum has stalled (near 2048)
+    assert np.allclose(got, exact, rtol=1e-2)              # the tree-ordered one has not
+    assert np.all(np.abs(got - exact) < np.abs(want - exact))

@@ -3,6 +3,7 @@ import os
 import subprocess
 import sys
 
+import numpy as np
 import pytest
 import torch
 
@@ -119,6 +120,8 @@ def test_tune_config_times_candidates_and_keeps_the_winner(ops_dir):
     want = plain(x)
     got = tuned(x)
     assert torch.equal(got, want)
+    from oracle import hot_ops                                   # the checker: the tuned operator against the oracle
+    assert np.allclose(got.cpu().numpy(), hot_ops.sigmoid_f32(x.cpu().numpy()), rtol=1e-5, atol=1e-5)
     assert len(tuned.tuned) == 1
     (key, choice), = tuned.tuned.items()
     assert key.startswith('autort_sigmoid_tuned_k0|1000000|') and choice['variant'] in ('vec', 'scalar') and choice['grid'] >= 1
@@ -134,3 +137,80 @@ def test_tune_config_times_candidates_and_keeps_the_winner(ops_dir):
     hist = torch.zeros(16, dtype=torch.int32, device=dev)
     acc(data, torch.ones(1, dtype=torch.int32, device=dev), hist)
     assert hist.tolist() == [256] * 16
+
+
+@pytest.mark.gpu
+def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
+    """config="tune:N" on a program that runs on a hand-written kernel searches that kernel's launch parameter (rows
+    per lane of the int4 GEMV, K-splits of the int4 GEMM) for the shape of the call, keeps the winner in the module
+    file, and the tuned operator - like every value of the parameter - matches the oracle."""
+    import subprocess
+    from ctypes import c_void_p
+    import autort
+    from antares_amd import workloads
+    from antares_amd.autort import patterns, store
+    from antares_amd.runtime import capi
+    from oracle import hot_ops
+    subprocess.check_call(['make', '-s', '-C', os.path.join(ROOT, 'oracle'), 'libref_hotops.so'])
+    dev = autort.device()
+    f = autort.export(ir=patterns.W4A16_IR, inputs=patterns.W4A16_INPUTS, name='w4a16_tuned', config='tune:8')
+    lib = capi.lib()
+    for M, K, N, key, entry, values in [
+            (1, 4096, 4096, 'gemv_w4a16.rows_per_lane|1,4096,4096', lib.art_gemv_w4a16_tuned, (0, 4, 8)),
+            (2, 1024, 1040, 'gemv_w4a16.rows_per_lane|2,1024,1040', lib.art_gemv_w4a16_tuned, (4, 8)),
+            (64, 4096, 4096, 'gemm_w4a16.k_splits|64,4096,4096', lib.art_gemm_w4a16_tuned, (0, 1, 3, 8, 32, 1000))]:
+        print(f'[case] tuned int4 product M={M} K={K} N={N}', flush=True)
+        p = workloads.w4_problem(M + K + N, M, K, N)
+        want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy()).astype(np.float32)
+        d = [p[k].to(dev) for k in ('x', 'qweight', 'scales', 'qzeros')]
+        got = f(*d)
+        assert np.allclose(got.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
+        choice = f.tuned[key]
+        assert choice['us'] > 0 and (choice['value'] in (4, 8) if 'gemv' in key else 0 <= choice['value'] <= K // 128)
+        assert store.load('w4a16_tuned')['tuned'][key] == choice
+        assert torch.equal(f(*d), got)                              # the stored choice is used again, no new search
+        for v in values:                                            # every value of the parameter gives the oracle's result
+            y = torch.full((M, N), float('nan'), dtype=torch.float16, device=dev)
+            capi.check(entry(c_void_p(d[0].data_ptr()), c_void_p(d[1].data_ptr()), c_void_p(d[2].data_ptr()), c_void_p(d[3].data_ptr()),
+                             c_void_p(y.data_ptr()), M, K, N, v, None))
+            torch.cuda.synchronize()
+            assert np.allclose(y.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2), v
+    # a later session finds the choices
+    again = type(autort.ops)().w4a16_tuned
+    assert again.tuned == f.tuned and len(again.tuned) == 3
+    # a value outside the parameter's range is refused
+    assert lib.art_gemv_w4a16_tuned(None, None, None, None, None, 1, 4096, 4096, 5, None) != 0
+    assert b'rows_per_lane' in lib.art_last_error()
+
+
+@pytest.mark.gpu
+def test_partition_tuning_keeps_results_bit_exact(ops_dir):
+    """The fused partition's launch parameter (cap on the number of blocks): every value gives the oracle's bits, a
+    tuning run keeps the fastest for that length and later sessions read it back."""
+    import subprocess
+    from ctypes import c_void_p
+    import autort
+    from antares_amd import workloads
+    from antares_amd.autort.builtin_ops import PartitionEvenFirst
+    from antares_amd.runtime import capi
+    from oracle import hot_ops
+    subprocess.check_call(['make', '-s', '-C', os.path.join(ROOT, 'oracle'), 'libref_hotops.so'])
+    dev = autort.device()
+    n = 3_000_017
+    x = workloads.partition_input(5, n)
+    want = hot_ops.sort_even_first_i32(x.numpy())
+    xd = x.to(dev)
+    capi.init(0)
+    for cap in (0, 64, 100, 1024, 16384):
+        print(f'[case] partition with at most {cap} blocks', flush=True)
+        out = torch.zeros_like(xd)
+        capi.check(capi.lib().art_partition_even_first_i32_tuned(c_void_p(xd.data_ptr()), c_void_p(out.data_ptr()), n, cap, None))
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want), cap
+    assert capi.lib().art_partition_even_first_i32_tuned(c_void_p(xd.data_ptr()), c_void_p(out.data_ptr()), n, 63, None) != 0
+    op = PartitionEvenFirst()
+    rec = op.tune(xd, trials=4)
+    assert rec['value'] in PartitionEvenFirst.BLOCK_CAPS[:4] and rec['us'] > 0
+    assert np.array_equal(op(xd).cpu().numpy(), want)
+    fresh = PartitionEvenFirst()
+    assert np.array_equal(fresh(xd).cpu().numpy(), want) and fresh.tuned[str(n)] == rec
