@@ -223,6 +223,33 @@ class DecodeAttention:
         return out
 
 
+class CausalAttention:
+    """``attention_causal_f16(q[T,H,D], k[S,H,D], v[S,H,D], att_f[1]) -> out[T,H,D]`` with S >= T: position t attends to
+    rows 0..t of k and v (views of the key / value cache), i.e. ``attention_f16`` for the T positions of a prompt in
+    one launch on the matrix cores."""
+    name = 'attention_causal_f16'
+
+    def __call__(self, q, k, v, att_f, out=None, extra=None):
+        if q.dim() != 3 or k.dim() != 3 or k.shape != v.shape or k.shape[1:] != q.shape[1:] or k.shape[0] < q.shape[0]:
+            raise ValueError(f'{self.name}: expected q[T,H,D], k[S,H,D], v[S,H,D] with S >= T; got {list(q.shape)}, {list(k.shape)}, {list(v.shape)}')
+        for t in (q, k, v):
+            if t.dtype != torch.float16:
+                raise TypeError(f'{self.name}: q, k and v must be float16')
+        if att_f.dtype != torch.float32 or att_f.numel() != 1:
+            raise TypeError(f'{self.name}: att_f must be a 1-element float32 tensor')
+        if out is None:
+            out = torch.empty_like(q)
+        if out.dtype != torch.float16 or out.shape != q.shape:
+            raise TypeError(f'{self.name}: out must be float16 of the shape of q')
+        _require_cuda(q, k, v, att_f, out)
+        T, H, D = q.shape
+        capi.check(capi.lib().art_prefill_attention(c_void_p(q.data_ptr()), c_void_p(k.data_ptr()), c_void_p(v.data_ptr()),
+                                                   c_void_p(att_f.data_ptr()), c_void_p(out.data_ptr()), T, H, D, H * D,
+                                                   c_void_p(current_stream_handle())))
+        return out
+
+
+builtin('attention_causal_f16')(lambda: CausalAttention())
 builtin('rmsnorm_f32')(lambda: RmsNorm(torch.float32))
 builtin('rmsnorm_f16')(lambda: RmsNorm(torch.float16))
 builtin('rotary_f32')(lambda: Rotary('rotary_f32', False))

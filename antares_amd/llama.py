@@ -125,6 +125,8 @@ class LlamaInt4Decoder:
         self.logits = torch.empty(cfg.vocab, **f16)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self._prefill_cache: Dict[int, Dict[str, object]] = {}      # prompt length -> operators of `prefill`
+        self._prefill_graphs: Dict[int, tuple] = {}                  # prompt length -> (recorded pass, its token buffer)
+        self._stream: Optional[torch.cuda.Stream] = None             # the one side stream recordings are made on
         self._ops()
 
     def _ops(self):
@@ -216,7 +218,6 @@ class LlamaInt4Decoder:
         ang = f'(T{f32} * freq[J]{f32})'
         rope = (f'(src[T, {{base}} + H * {D} + P * {J} + J]{f32} * {ang}.call(`cos`) + (P * 2 - 1){f32} * '
                 f'src[T, {{base}} + H * {D} + (1 - P) * {J} + J]{f32} * {ang}.call(`sin`)).to(`float16`) where H in {H}, P in 2, J in {J}')
-        scale = repr(1.0 / math.sqrt(D))
         ops = {
             'embed': program(ir='emb[T, D] = table[tok[T], D]', inputs=[f'table=float16[{V}, {d}]', f'tok=int32[{T}]'],
                               name=f'prefill_embed_{T}'),
@@ -229,15 +230,6 @@ class LlamaInt4Decoder:
                                name=f'prefill_rope_k_{T}'),
             'copy_v': program(ir=f'vc[T, D] = src[T, {2 * d} + D] where D in {d}', inputs=[f'src=float16[{T}, {3 * d}]'],
                                name=f'prefill_copy_v_{T}'),
-            'scores': program(ir=f'sc[H, T, S] +=! qr[T, H, D]{f32} * kc[S, H, D]{f32}',
-                               inputs=[f'qr=float16[{T}, {H}, {D}]', f'kc=float16[{T}, {H}, {D}]'], name=f'prefill_scores_{T}'),
-            'softmax_v': program(
-                ir=f'mx[H, T] >=! (sc[H, T, S] * {scale}).when([S <= T], -3.0e38); '
-                   f'ex[H, T, S] = (sc[H, T, S] * {scale} - mx[H, T]).call(`exp`).when([S <= T], 0.0); '
-                   f'den[H, T] +=! ex[H, T, S]; '
-                   f'av[T, H, D] +=! ex[H, T, S] * vc[S, H, D]{f32}; '
-                   f'att[T, H, D] = (av[T, H, D] / den[H, T]).to(`float16`)',
-                inputs=[f'sc=float32[{H}, {T}, {T}]', f'vc=float16[{T}, {H}, {D}]'], name=f'prefill_softmax_v_{T}'),
             'silu_mul': program(
                 ir=f'hid[T, N] = (gu[T, N]{f32} / (1.0 + (0.0 - gu[T, N]{f32}).call(`exp`)) * gu[T, {F} + N]{f32}).to(`float16`) where N in {F}',
                 inputs=[f'gu=float16[{T}, {2 * F}]'], name=f'prefill_silu_mul_{T}'),
@@ -245,17 +237,46 @@ class LlamaInt4Decoder:
         self._prefill_cache[T] = ops
         return ops
 
-    def prefill(self, tokens: torch.Tensor) -> torch.Tensor:
+    def prefill(self, tokens: torch.Tensor, graph: bool = True) -> torch.Tensor:
         """Ingests a whole prompt (int32 [T] on the device, T >= 4, positions 0..T-1) in one pass: the projections
         run as batched int4 GEMMs on the matrix cores (`gemv_w4a16` with T rows), attention is causal over the
-        prompt, keys and values land in cache rows 0..T-1.  Leaves the step state at the last prompt position
-        (self.pos = T - 1, self.x = its hidden state, self.logits = its logits), so `advance()` and the recorded
-        decode step continue from there.  Same operators and roundings as the one-token step, applied to T rows."""
+        prompt (`attention_causal_f16`, matrix cores), keys and values land in cache rows 0..T-1.  Leaves the step
+        state at the last prompt position (self.pos = T - 1, self.x = its hidden state, self.logits = its logits), so
+        `advance()` and the recorded decode step continue from there.  Same operators and roundings as the one-token
+        step, applied to T rows.  With ``graph`` the pass is recorded once per prompt length in a HIP graph (about 450
+        launches) and replayed on later calls with the new tokens copied into the recorded input."""
+        T = int(tokens.numel())
+        if not 4 <= T <= self.cfg.max_seq:
+            raise ValueError(f'prefill takes 4..{self.cfg.max_seq} tokens, got {T}')
+        if not graph or torch.cuda.is_current_stream_capturing():
+            return self._prefill_eager(tokens)
+        rec = self._prefill_graphs.get(T)
+        if rec is None:
+            static_tokens = tokens.view(T).clone()
+            stream = self._side_stream()
+            stream.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(stream):
+                self._prefill_eager(static_tokens)          # loads every module and workspace outside the capture
+                stream.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    self._prefill_eager(static_tokens)
+            torch.cuda.current_stream().wait_stream(stream)
+            rec = self._prefill_graphs[T] = (g, static_tokens)
+        g, static_tokens = rec
+        static_tokens.copy_(tokens.view(T))
+        g.replay()
+        return self.logits
+
+    def _side_stream(self):
+        if self._stream is None:
+            self._stream = torch.cuda.Stream()
+        return self._stream
+
+    def _prefill_eager(self, tokens: torch.Tensor) -> torch.Tensor:
         cfg = self.cfg
         T = int(tokens.numel())
         d, H, D, F = cfg.dim, cfg.n_heads, cfg.head_dim, cfg.ffn
-        if not 4 <= T <= cfg.max_seq:
-            raise ValueError(f'prefill takes 4..{cfg.max_seq} tokens, got {T}')
         ops = self._prefill_ops(T)
         f16 = dict(dtype=torch.float16, device=self.dev)
         x = ops['embed'](self.w['embed'], tokens.view(T))
@@ -272,8 +293,8 @@ class LlamaInt4Decoder:
             qr = ops['rope_q'](qkv, self.inv_freq)
             ops['rope_k'](qkv, self.inv_freq, out=kc.view(T, H, 2, D // 2))
             ops['copy_v'](qkv, out=vc)
-            sc = ops['scores'](qr.view(T, H, D), kc.view(T, H, D))
-            att = ops['softmax_v'](sc, vc.view(T, H, D))
+            att = self.autort.ops.attention_causal_f16(qr.view(T, H, D), self.key_cache[l].view(cfg.max_seq, H, D),
+                                                       self.val_cache[l].view(cfg.max_seq, H, D), self.att_f)
             linear(att.view(T, d), lw['o'], proj)
             self.add(x.view(-1), proj.view(-1))
             xb = ops['rms'](x, lw['ffn_norm'])
@@ -350,7 +371,8 @@ class LlamaInt4Decoder:
     def capture(self, greedy: bool = True, prompt: Optional[torch.Tensor] = None):
         """Record one step (+ advance) in a HIP graph.  ``prompt`` (int32 on the device)
         is fed token by token before greedy decoding takes over."""
-        stream = torch.cuda.Stream()
+        stream = self._side_stream()
+        stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(stream):
             self.step()                       # loads every module outside the capture
             stream.synchronize()

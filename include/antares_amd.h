@@ -262,6 +262,14 @@ int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev
                          int seq_len, int heads, int head_dim, const void* pos_dev, int q_dtype, int kv_dtype, int out_dtype,
                          void* stream);
 
+/* Causal attention over a whole prompt (fp16, fp32 accumulation, matrix cores): query position t (row t of q,
+ * [T, heads, 128]) attends to rows 0..t of k and v (row s at k_dev + s * kv_row_stride halves, holding [heads, 128]:
+ * the rows of a key / value cache), out[t] = softmax_s(att_f[0] * q[t] . k[s]) v, [T, heads, 128].  The same
+ * arithmetic as art_decode_attention applied to T positions at once (torch spelling: samples/03_llama_tiny.py:94-99);
+ * replaces the two generated contraction kernels of a whole-prompt pass. */
+int art_prefill_attention(const void* q_dev, const void* k_dev, const void* v_dev, const void* att_f_dev, void* out_dev,
+                          int T, int heads, int head_dim, long long kv_row_stride, void* stream);
+
 /* The bookkeeping between two decode steps of samples/05_llama2_7b_int4.py:196-201, one launch, all on the
  * device:  *pos += 1;  *token = (*pos < prompt_len) ? prompt[*pos] : argmax(logits[0..vocab));
  * x_out[0..dim) = embed[*token][0..dim).  logits, embed, x_out fp16; prompt, token, pos int32.  Ties of the

@@ -10,9 +10,9 @@ pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures('oracle_built')]
 LOGIT_TOL = dict(rtol=2e-2, atol=2e-2)
 
 
-def small_config():
+def small_config(max_seq=32):
     from antares_amd.llama import LlamaConfig
-    return LlamaConfig(n_layers=2, dim=512, n_heads=4, ffn=1024, vocab=1024, max_seq=32)
+    return LlamaConfig(n_layers=2, dim=512, n_heads=4, ffn=1024, vocab=1024, max_seq=max_seq)
 
 
 @pytest.mark.parametrize('fused,att_parts', [(False, 1), (True, 1), (True, 4), (True, 8)])
@@ -90,14 +90,14 @@ def test_fused_projection_matches_operator_chain():
         assert torch.equal(buf, got)
 
 
-@pytest.mark.parametrize('T', [5, 20])
+@pytest.mark.parametrize('T', [5, 20, 128])
 def test_prefill_of_a_whole_prompt_matches_the_oracle_token_by_token(T):
     """`prefill` (projections as batched int4 GEMMs, causal attention over the prompt) must leave the logits of the
     last prompt position and the key / value cache rows that the oracle reaches token by token, and the one-token
     step must carry on from there."""
     from antares_amd.llama import LlamaInt4Decoder, random_weights
     from oracle.llama_ref import LlamaRef
-    cfg = small_config()
+    cfg = small_config(max_seq=32 if T < 32 else 160)
     w = random_weights(cfg, seed=4)
     ref = LlamaRef(cfg, w)
     g = torch.Generator().manual_seed(T)
@@ -107,7 +107,16 @@ def test_prefill_of_a_whole_prompt_matches_the_oracle_token_by_token(T):
         want = ref.forward(int(prompt[pos]), pos).astype(np.float32)
     dec = LlamaInt4Decoder(cfg, w, fused=True, att_parts=4)
     print(f'[case] prefill T={T}', flush=True)
-    got = dec.prefill(prompt.to(dec.dev)).float().cpu().numpy()
+    eager = dec.prefill(prompt.to(dec.dev), graph=False).clone()
+    dec.key_cache.zero_()
+    dec.val_cache.zero_()
+    # recorded in a graph, then replayed with other tokens in between: the replay must use the tokens of its call
+    other = torch.randint(0, cfg.vocab, (T,), generator=g, dtype=torch.int32).to(dec.dev)
+    dec.prefill(other)
+    got_t = dec.prefill(prompt.to(dec.dev))
+    torch.cuda.synchronize()
+    assert torch.equal(got_t, eager)
+    got = got_t.float().cpu().numpy()
     # logits of spread ~2 after two layers: the batched path sums in another order than the one-token path (which
     # is itself up to 0.03 away from the oracle here) and measured up to 0.05; the cache rows below pin each layer
     assert np.allclose(got, want, rtol=4e-2, atol=4e-2), np.abs(got - want).max()

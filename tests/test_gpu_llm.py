@@ -290,3 +290,33 @@ def test_fused_decode_attention_against_the_oracle(parts, pos):
     assert np.array_equal(vg[pos], vc_want[pos])
     keep = np.arange(S) != pos
     assert np.array_equal(kg[keep], kc.numpy()[keep]) and np.array_equal(vg[keep], vc.numpy()[keep])
+
+
+@pytest.mark.usefixtures('oracle_built')
+@pytest.mark.parametrize('T,H', [(1, 4), (5, 4), (31, 4), (32, 32), (33, 4), (100, 32), (128, 32), (200, 4), (384, 32)])
+def test_causal_attention_over_a_prompt_against_the_oracle(T, H):
+    """attention_causal_f16 (matrix cores, one wavefront per 32 queries) against the oracle's attention applied position by
+    position: query t sees rows 0..t of cache views that have more rows than the prompt."""
+    import autort
+    from oracle import hot_ops
+    dev = autort.device()
+    D, S = 128, T + 7
+    g = torch.Generator().manual_seed(31 * T + H)
+    note(f'causal attention T={T} H={H}')
+    q = torch.randn(T, H, D, generator=g).half()
+    kc = (torch.randn(S, H * D, generator=g) * 0.7).half()
+    vc = torch.randn(S, H * D, generator=g).half()
+    att_f = 1 / math.sqrt(D)
+    out = autort.ops.attention_causal_f16(q.to(dev), kc.to(dev).view(S, H, D), vc.to(dev).view(S, H, D),
+                                          torch.tensor([att_f], dtype=torch.float32, device=dev)).cpu().numpy()
+    assert out.shape == (T, H, D)
+    ks, vs = kc.numpy().reshape(S, H, D), vc.numpy().reshape(S, H, D)
+    for t in sorted({0, 1, T // 3, T // 2, T - 2, T - 1} & set(range(T))) if T > 40 else range(T):
+        want = hot_ops.attention(q[t].numpy(), ks[:t + 1], vs[:t + 1], att_f)
+        assert np.allclose(out[t].astype(np.float32), want.astype(np.float32), **FP16_TOL), (t, np.abs(out[t].astype(np.float32) - want.astype(np.float32)).max())
+    # the probabilities are rounded to fp16 before they meet V: compare every position with float64 as well
+    qd, kd, vd = q.double(), kc.double().view(S, H, D), vc.double().view(S, H, D)
+    sc = torch.einsum('thd,shd->hts', qd, kd[:T]) * att_f
+    sc = sc.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float('-inf'))
+    exact = torch.einsum('hts,shd->thd', torch.softmax(sc, -1), vd[:T]).numpy()
+    assert np.allclose(out.astype(np.float64), exact, rtol=1e-2, atol=1e-2)
