@@ -130,15 +130,15 @@ def _w4a16_handler(op, bound, env, stream) -> bool:
         capi.check(entry(c_void_p(t[0].data_ptr()), c_void_p(t[1].data_ptr()), c_void_p(t[2].data_ptr()), c_void_p(t[3].data_ptr()),
                          c_void_p(t[4].data_ptr()), M, K, N, int(value), c_void_p(stream if st is None else st)))
 
-    # the launch parameter of the kernel that runs: rows per lane of the GEMV (0 = 8, or 4), K-splits of the GEMM
-    key = f"{'gemv_w4a16.rows_per_lane' if gemv else 'gemm_w4a16.k_splits'}|{M},{K},{N}"
+    # the launch parameter of the kernel that runs: k per block of the GEMV, K-splits of the GEMM
+    key = f"{'gemv_w4a16.k_per_block' if gemv else 'gemm_w4a16.k_splits'}|{M},{K},{N}"
     saved = op.tuned.get(key)
     trials = op.config.get('tune')
     if saved is None and isinstance(trials, int) and trials > 0 and not torch.cuda.is_current_stream_capturing():
         per_set = q.numel() + 2 * s.numel() + z.numel()
         copies = max(1, min(8, (256 << 20) // max(per_set, 1)))
         clones = [(x, q.clone(), s.clone(), z.clone(), torch.empty_like(y)) for _ in range(copies)]
-        cands = [8, 4] if gemv else [0] + [v for v in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32) if v <= K // 128]
+        cands = ([512, 256, 1024] if M == 1 else [512, 256]) if gemv else [0] + [v for v in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32) if v <= K // 128]
         saved = tune_hand_kernel(op, key, cands, lambda v, t: run(v, t, torch.cuda.current_stream().cuda_stream), trials, clones)
         del clones
     run(saved['value'] if saved is not None else 0, (x, q, s, z, y))

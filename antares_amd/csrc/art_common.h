@@ -27,6 +27,9 @@ constexpr int kMaxStreamsPerDevice = 40;      // torch hands out 32 pooled strea
 // art_gemv_w4a16_noalloc).  Called once per device by art_init.
 int gemv_noalloc_setup(int device);
 
+// Compute units of the current device (queried once per device).
+int compute_units();
+
 // Blocks per head the split decode attention may use, shared by its producer (art_llm.hip) and the projection that
 // merges the per-part records (art_gemv_w4.hip).
 constexpr int kMaxAttnParts = 8;

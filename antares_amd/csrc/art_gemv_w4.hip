@@ -75,10 +75,10 @@ __device__ __forceinline__ void mac_word_pair(unsigned int a, unsigned int b, ha
   acc[3] = __builtin_amdgcn_fdot2(nib(p23s, k.mask_hi, k.bias_hi), xo, acc[3], false);
 }
 
-constexpr int kThreads = 256;
-constexpr int CL = 8;                  // column lanes per block
-constexpr int KL = kThreads / CL;      // 32 k lanes per block, 8 per wavefront
+constexpr int CL = 8;                  // column lanes per block (8 k lanes per wavefront)
 constexpr int CT = 16 * CL;            // 128 columns per block
+// Wavefronts per block, W, is the other launch parameter (template): 4 (256 threads) or 8 (512 threads).  Eight
+// double the k range of a block, so a column receives half as many returning atomics; a tuning run may pick it.
 // Packed rows per lane, R, is a launch parameter (template): 8 rows make a block 128 columns x 512 k with each
 // wavefront on exactly one quantisation group of 128 k; 4 rows make it 128 x 256 with two wavefronts per group -
 // twice the blocks (and twice the returning atomics), which pays when 8 rows leave compute units without a block.
@@ -156,15 +156,17 @@ struct Fused {
 
 // The register allocator is told that four wavefronts per SIMD are plenty (a launch has three): with the default
 // target of eight it postpones two of the eight weight loads until registers free up, a second memory round trip.
-template <int M, int MODE, int R>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused, 3: x = merged split attention
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_w4a16_kernel(
+template <int M, int MODE, int R, int W>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused, 3: x = merged split attention
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_w4a16_kernel(
     const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight, const _Float16* __restrict__ scales,
     const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y, int K, int N, int splits,
     unsigned long long* __restrict__ slots, Magic magic, Fused fused) {
   static_assert(R == 8 || (R == 4 && MODE == 0), "the fused prologues are written for 8 rows per lane");
-  constexpr int kRowsPerBlock = KL * R;                 // packed rows per block: 256 (512 values of k) or 128
-  __shared__ __align__(16) float part[M][4][CT];        // per wavefront: scaled sums of the tile's columns
-  __shared__ float s_ss[4];
+  static_assert(W == 4 || W == 8, "four or eight wavefronts per block");
+  constexpr int kThreads = 64 * W, KL = kThreads / CL;  // k lanes per block: 32 or 64
+  constexpr int kRowsPerBlock = KL * R;                 // packed rows per block: 256 (512 values of k) at R = 8, W = 4
+  __shared__ __align__(16) float part[M][W][CT];        // per wavefront: scaled sums of the tile's columns
+  __shared__ float s_ss[W];
   __shared__ __align__(16) unsigned int s_x[KL][CL];    // SwiGLU input, one fp16 pair per lane
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -183,10 +185,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
   // return in order, so these can be consumed (and the block-wide reduction done) while the weights are
   // still in flight; issued after the weights they would wait for the whole stream.
   constexpr bool norm = (M == 1) && (MODE == 1);
-  u32x4 sq[2];
+  constexpr int kSq = 512 / kThreads;                     // 16-byte chunks of x per thread that cover K = 4096
+  u32x4 sq[kSq];
   if constexpr (norm) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kSq; ++i) {
       const int c = tid + i * kThreads;
       sq[i] = (c < (K >> 3)) ? reinterpret_cast<const u32x4*>(x)[c] : u32x4{0, 0, 0, 0};
     }
@@ -285,7 +288,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
   if constexpr (norm) {
     float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kSq; ++i) {
       const unsigned int wds[4] = {sq[i][0], sq[i][1], sq[i][2], sq[i][3]};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -294,7 +297,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
         ss = fmaf((float)h.y, (float)h.y, ss);
       }
     }
-    for (int c = tid + 2 * kThreads; c < (K >> 3); c += kThreads) {      // K > 4096
+    for (int c = tid + kSq * kThreads; c < (K >> 3); c += kThreads) {      // K > 4096
       const u32x4 v = reinterpret_cast<const u32x4*>(x)[c];
       const unsigned int wds[4] = {v[0], v[1], v[2], v[3]};
 #pragma unroll
@@ -307,7 +310,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
     ss = wave_sum_all(ss);
     if (lane == 0) s_ss[wave] = ss;
     art_lds_barrier();      // LDS only: the weight loads issued above stay in flight
-    const float r = 1.0f / sqrtf(((s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3])) * fused.inv_n + fused.eps);
+    float ss_all = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
+    if constexpr (W == 8) ss_all += (s_ss[4] + s_ss[5]) + (s_ss[6] + s_ss[7]);
+    const float r = 1.0f / sqrtf(ss_all * fused.inv_n + fused.eps);
     const u32x4* np = reinterpret_cast<const u32x4*>(fused.norm_w + 2 * r0c);
     const u32x4 n0v = np[0], n1v = np[1];
     const unsigned int nw[8] = {n0v[0], n0v[1], n0v[2], n0v[3], n1v[0], n1v[1], n1v[2], n1v[3]};
@@ -380,6 +385,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4))
     const f32x2 p2 = *reinterpret_cast<const f32x2*>(&part[m][2][c2]), p3 = *reinterpret_cast<const f32x2*>(&part[m][3][c2]);
     r[m][0] = (p0[0] + p1[0]) + (p2[0] + p3[0]);
     r[m][1] = (p0[1] + p1[1]) + (p2[1] + p3[1]);
+    if constexpr (W == 8) {
+      const f32x2 p4 = *reinterpret_cast<const f32x2*>(&part[m][4][c2]), p5 = *reinterpret_cast<const f32x2*>(&part[m][5][c2]);
+      const f32x2 p6 = *reinterpret_cast<const f32x2*>(&part[m][6][c2]), p7 = *reinterpret_cast<const f32x2*>(&part[m][7][c2]);
+      r[m][0] += (p4[0] + p5[0]) + (p6[0] + p7[0]);
+      r[m][1] += (p4[1] + p5[1]) + (p6[1] + p7[1]);
+    }
   }
   if (splits == 1) {
 #pragma unroll
@@ -429,10 +440,13 @@ unsigned long long* g_scratch_ptr[kMaxDevices];          // device address of `s
 template <int M>
 int launch(const void* x, const void* qw, const void* sc, const void* qz, void* y, int K, int N, hipStream_t stream,
            Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0}, unsigned long long* slots = nullptr,
-           int rows_per_lane = 8) {
+           int rows_per_lane = 8, int waves = 0) {
   const int rows = K / 2;
   const int tiles = (N + CT - 1) / CT;
-  const int rows_per_block = KL * rows_per_lane;
+  // Four wavefronts unless the caller asks for eight: halving the atomics did not pay on any shape of the decode
+  // step (4096 x 22016: 13.5 -> 13.9 us, 4096 x 32000: 17.0 -> 17.6 us), the blocks' larger k range costs more.
+  if (waves == 0) waves = 4;
+  const int rows_per_block = 8 * waves * rows_per_lane;
   const int splits = (rows + rows_per_block - 1) / rows_per_block;
   ART_REQUIRE(splits <= 127, "art_gemv_w4a16: K too large (%d) for %d rows per lane", K, rows_per_lane);
   if (slots == nullptr) {         // the library's own workspace for this stream
@@ -442,16 +456,29 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
     slots = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(wsp->base) + art::kSlotOffset);
   }
   const Magic magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
-  const dim3 grid(tiles, splits), block(kThreads);
-#define ART_GEMV_LAUNCH(MODE, R)                                                                                          \
-  gemv_w4a16_kernel<M, MODE, R><<<grid, block, 0, stream>>>((const _Float16*)x, (const unsigned char*)qw, (const _Float16*)sc, \
-                                                            (const unsigned char*)qz, (_Float16*)y, K, N, splits, slots, magic, fused)
-  // the plain product is its own instantiation: it carries none of the fused prologues
-  if (M == 1 && fused.norm_w != nullptr) ART_GEMV_LAUNCH(1, 8);
-  else if (M == 1 && fused.gate_up != nullptr) ART_GEMV_LAUNCH(2, 8);
-  else if (M == 1 && fused.att_partial != nullptr) ART_GEMV_LAUNCH(3, 8);
-  else if (rows_per_lane == 4) ART_GEMV_LAUNCH(0, 4);
-  else ART_GEMV_LAUNCH(0, 8);
+  const dim3 grid(tiles, splits), block(64 * waves);
+#define ART_GEMV_LAUNCH(MODE, R, W)                                                                                          \
+  gemv_w4a16_kernel<M, MODE, R, W><<<grid, block, 0, stream>>>((const _Float16*)x, (const unsigned char*)qw, (const _Float16*)sc, \
+                                                               (const unsigned char*)qz, (_Float16*)y, K, N, splits, slots, magic, fused)
+  // the plain product is its own instantiation: it carries none of the fused prologues; rows of x beyond the first
+  // and four rows per lane come with four wavefronts only
+  if constexpr (M == 1) {
+    if (waves == 8) {
+      if (fused.norm_w != nullptr) ART_GEMV_LAUNCH(1, 8, 8);
+      else if (fused.gate_up != nullptr) ART_GEMV_LAUNCH(2, 8, 8);
+      else if (fused.att_partial != nullptr) ART_GEMV_LAUNCH(3, 8, 8);
+      else ART_GEMV_LAUNCH(0, 8, 8);
+    } else {
+      if (fused.norm_w != nullptr) ART_GEMV_LAUNCH(1, 8, 4);
+      else if (fused.gate_up != nullptr) ART_GEMV_LAUNCH(2, 8, 4);
+      else if (fused.att_partial != nullptr) ART_GEMV_LAUNCH(3, 8, 4);
+      else if (rows_per_lane == 4) ART_GEMV_LAUNCH(0, 4, 4);
+      else ART_GEMV_LAUNCH(0, 8, 4);
+    }
+  } else {
+    if (rows_per_lane == 4) ART_GEMV_LAUNCH(0, 4, 4);
+    else ART_GEMV_LAUNCH(0, 8, 4);
+  }
 #undef ART_GEMV_LAUNCH
   ART_LAUNCH_CHECK();
   return 0;
@@ -465,10 +492,12 @@ extern "C" int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const 
 }
 
 extern "C" int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
-                                    void* y_dev, int M, int K, int N, int rows_per_lane, void* stream) {
-  ART_REQUIRE(rows_per_lane == 0 || rows_per_lane == 4 || rows_per_lane == 8,
-              "art_gemv_w4a16: rows_per_lane must be 0 (library's choice), 4 or 8 (got %d)", rows_per_lane);
-  const int rpl = rows_per_lane ? rows_per_lane : 8;
+                                    void* y_dev, int M, int K, int N, int k_per_block, void* stream) {
+  ART_REQUIRE(k_per_block == 0 || k_per_block == 256 || k_per_block == 512 || k_per_block == 1024,
+              "art_gemv_w4a16: k_per_block must be 0 (library's choice), 256, 512 or 1024 (got %d)", k_per_block);
+  ART_REQUIRE(k_per_block != 1024 || M == 1, "art_gemv_w4a16: k_per_block = 1024 is for M = 1 (got M = %d)", M);
+  // 256: four rows per lane, four wavefronts; 512: eight rows, four wavefronts; 1024: eight rows, eight wavefronts
+  const int rpl = k_per_block == 256 ? 4 : 8, waves = k_per_block == 0 ? 0 : (k_per_block == 1024 ? 8 : 4);
   ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16: null pointer");
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0,
@@ -484,10 +513,10 @@ extern "C" int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, 
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m * N;
     const Fused none{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0};
-    int rc = step == 4 ? launch<4>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl)
-           : step == 3 ? launch<3>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl)
-           : step == 2 ? launch<2>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl)
-                       : launch<1>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl);
+    int rc = step == 4 ? launch<4>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl, 4)
+           : step == 3 ? launch<3>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl, 4)
+           : step == 2 ? launch<2>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl, 4)
+                       : launch<1>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl, waves);
     if (rc) return rc;
     m += step;
   }

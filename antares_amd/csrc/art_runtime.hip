@@ -42,6 +42,18 @@ struct DeviceState {
 static DeviceState g_dev[kMaxDevices];
 static std::mutex g_mu;
 
+int compute_units() {
+  static int cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 static int allocate_workspace(Workspace* ws) {
   ART_HIP(hipMalloc(&ws->base, kWorkspaceBytes));
   hipError_t e = hipMemset(ws->base, 0, kWorkspaceBytes);

@@ -139,11 +139,13 @@ int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scale
  * `config="tune:N"` searches, as the reference's tuner searches the knobs of its schedules:
  * tuner/OpEvo/main.py:467-616, antares/common.py:81-118).  0 always means the library's own choice, and results do
  * not depend on the parameter beyond fp32 re-association.
- *   rows_per_lane: 4 or 8 packed rows per lane = 256 or 512 values of k per block of the int4 GEMV;
+ *   k_per_block:   256, 512 or 1024 values of k per block of the int4 GEMV (4 or 8 packed rows per lane in four
+ *                  wavefronts, or 8 rows in eight wavefronts; 1024 needs M = 1): fewer k per block = more blocks and
+ *                  more returning atomics per column;
  *   k_splits:      number of K-splits of the int4 GEMM (clamped to K/128 and to what the workspace holds);
  *   max_blocks:    cap on the blocks of the partition, 64..16384 (each walks its span tile by tile). */
 int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
-                         void* y_dev, int M, int K, int N, int rows_per_lane, void* stream);
+                         void* y_dev, int M, int K, int N, int k_per_block, void* stream);
 int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                          void* y_dev, int M, int K, int N, int k_splits, void* stream);
 int art_partition_even_first_i32_tuned(const void* in_dev, void* out_dev, long long n, int max_blocks, void* stream);

@@ -156,8 +156,9 @@ def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
     f = autort.export(ir=patterns.W4A16_IR, inputs=patterns.W4A16_INPUTS, name='w4a16_tuned', config='tune:8')
     lib = capi.lib()
     for M, K, N, key, entry, values in [
-            (1, 4096, 4096, 'gemv_w4a16.rows_per_lane|1,4096,4096', lib.art_gemv_w4a16_tuned, (0, 4, 8)),
-            (2, 1024, 1040, 'gemv_w4a16.rows_per_lane|2,1024,1040', lib.art_gemv_w4a16_tuned, (4, 8)),
+            (1, 4096, 4096, 'gemv_w4a16.k_per_block|1,4096,4096', lib.art_gemv_w4a16_tuned, (0, 256, 512, 1024)),
+            (1, 11008, 528, 'gemv_w4a16.k_per_block|1,11008,528', lib.art_gemv_w4a16_tuned, (256, 512, 1024)),
+            (2, 1024, 1040, 'gemv_w4a16.k_per_block|2,1024,1040', lib.art_gemv_w4a16_tuned, (256, 512)),
             (64, 4096, 4096, 'gemm_w4a16.k_splits|64,4096,4096', lib.art_gemm_w4a16_tuned, (0, 1, 3, 8, 32, 1000))]:
         print(f'[case] tuned int4 product M={M} K={K} N={N}', flush=True)
         p = workloads.w4_problem(M + K + N, M, K, N)
@@ -166,7 +167,7 @@ def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
         got = f(*d)
         assert np.allclose(got.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
         choice = f.tuned[key]
-        assert choice['us'] > 0 and (choice['value'] in (4, 8) if 'gemv' in key else 0 <= choice['value'] <= K // 128)
+        assert choice['us'] > 0 and (choice['value'] in (256, 512, 1024) if 'gemv' in key else 0 <= choice['value'] <= K // 128)
         assert store.load('w4a16_tuned')['tuned'][key] == choice
         assert torch.equal(f(*d), got)                              # the stored choice is used again, no new search
         for v in values:                                            # every value of the parameter gives the oracle's result
@@ -177,10 +178,10 @@ def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
             assert np.allclose(y.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2), v
     # a later session finds the choices
     again = type(autort.ops)().w4a16_tuned
-    assert again.tuned == f.tuned and len(again.tuned) == 3
+    assert again.tuned == f.tuned and len(again.tuned) == 4
     # a value outside the parameter's range is refused
     assert lib.art_gemv_w4a16_tuned(None, None, None, None, None, 1, 4096, 4096, 5, None) != 0
-    assert b'rows_per_lane' in lib.art_last_error()
+    assert b'k_per_block' in lib.art_last_error()
 
 
 @pytest.mark.gpu
