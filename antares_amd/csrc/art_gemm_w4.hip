@@ -67,17 +67,26 @@ template <int MT>   // MT accumulator tiles of 32 rows: 1 for M <= 32, 2 for M <
 __global__ __launch_bounds__(kThreads, 512 / kThreads) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
                                                              const _Float16* __restrict__ scales,
                                                              const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y,
-                                                             float* __restrict__ partial, int M, int K, int N, int splits,
-                                                             int col_tiles, Magic mg) {
+                                                             float* __restrict__ partial, int M_total, int K, int N, int splits,
+                                                             int col_tiles, int m_blocks, Magic mg) {
   extern __shared__ __align__(16) _Float16 smem[];
   _Float16* Ws = smem;                           // [2][SK][W_LD]
   _Float16* Xs = smem + 2 * W_TILE;              // [2][BM][X_LD]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-  // block -> (column tile, K split)
+  // block -> (column tile, K split, block of 64 rows).  The row blocks of one (tile, split) stream the same weights:
+  // they get block ids that are 8 apart, which the dispatcher places on the same XCD at the same time, so that the
+  // weights come from HBM once and from that XCD's L2 for the others.
   const int G = K / GK;
-  const int split = blockIdx.x / col_tiles;
-  const int n0 = (blockIdx.x % col_tiles) * BN;
+  const int unit = (int)(blockIdx.x / (8 * m_blocks)) * 8 + (int)(blockIdx.x % 8);      // (tile, split) pair
+  const int m_block = (int)(blockIdx.x % (8 * m_blocks)) / 8;
+  if (unit >= col_tiles * splits) return;
+  const int split = unit / col_tiles;
+  const int n0 = (unit % col_tiles) * BN;
+  const int m0 = m_block * BM;
+  const int M = M_total - m0 < BM ? M_total - m0 : BM;          // rows of this block
+  x += (size_t)m0 * K;
+  y += (size_t)m0 * N;
   const int g_begin = (int)((long long)G * split / splits), g_end = (int)((long long)G * (split + 1) / splits);
   const int groups = g_end - g_begin;
 
@@ -280,7 +289,7 @@ __global__ __launch_bounds__(kThreads, 512 / kThreads) void gemm_w4a16_kernel(co
       const int row = t * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
       if (row < M) {
         if (splits == 1) y[(size_t)row * N + my_col] = (_Float16)total[t][r];
-        else partial[((size_t)split * M + row) * N + my_col] = total[t][r];
+        else partial[((size_t)split * M_total + m0 + row) * N + my_col] = total[t][r];
       }
     }
 }
@@ -346,9 +355,13 @@ extern "C" int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, 
   const Magic mg{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
   hipStream_t st = (hipStream_t)stream;
   const int G = K / GK, col_tiles = (N + BN - 1) / BN;
-  for (int m0 = 0; m0 < M; m0 += BM) {      // 64 rows of x per pass over the weights
-    const int rows = M - m0 < BM ? M - m0 : BM;
-    int splits = choose_splits(rows, N, K, scratch_bytes, compute_units);
+  // Up to kMaxRowBlocks blocks of 64 rows go into one launch (they share the weight stream through L2, and the K-splits
+  // are combined once); longer batches take several passes over the weights.
+  constexpr int kMaxRowBlocks = 8;
+  for (int m0 = 0; m0 < M; m0 += BM * kMaxRowBlocks) {
+    const int rows = M - m0 < BM * kMaxRowBlocks ? M - m0 : BM * kMaxRowBlocks;
+    const int m_blocks = (rows + BM - 1) / BM;
+    int splits = choose_splits(rows, N, K, scratch_bytes, compute_units / m_blocks);
     if (k_splits > 0) {           // the caller's choice, within what the kernel and the scratch space take
       const int cap = (int)(scratch_bytes / ((size_t)rows * N * sizeof(float)));
       splits = k_splits > G ? G : k_splits;
@@ -356,15 +369,15 @@ extern "C" int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, 
     }
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m0 * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m0 * N;
-    const dim3 grid(col_tiles * splits);
+    const dim3 grid((unsigned)((col_tiles * splits + 7) / 8 * 8 * m_blocks));
     if (rows <= 32)
       gemm_w4a16_kernel<1><<<grid, kThreads, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
-                                                         col_tiles, mg);
+                                                         col_tiles, m_blocks, mg);
     else
       gemm_w4a16_kernel<2><<<grid, kThreads, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
-                                                         col_tiles, mg);
+                                                         col_tiles, m_blocks, mg);
     ART_LAUNCH_CHECK();
     if (splits > 1) {
       const long long count4 = (long long)rows * N / 4;
