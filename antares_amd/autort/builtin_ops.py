@@ -391,6 +391,29 @@ class RopeQkvStore:
         return q_out
 
 
+class RopeQkvStoreRows:
+    """``rope_qkv_store_rows_f16(qkv[T, 3*H*D], inv_freq[D], q_out[T,H,D], key_cache[S,H*D], val_cache[S,H*D], extra=[first_pos])``:
+    ``rope_qkv_store_f16`` for the T tokens of a prompt, token t at position first_pos + t (a host integer, default 0)."""
+    name = 'rope_qkv_store_rows_f16'
+
+    def __call__(self, qkv, inv_freq, q_out, key_cache, val_cache, extra=None):
+        T, heads, head_dim = q_out.shape
+        if qkv.shape != (T, 3 * heads * head_dim) or key_cache.shape[-1] != heads * head_dim or val_cache.shape != key_cache.shape:
+            raise ValueError(f'{self.name}: shapes do not fit together')
+        for t in (qkv, inv_freq, q_out, key_cache, val_cache):
+            if t.dtype != torch.float16:
+                raise TypeError(f'{self.name}: tensors must be float16')
+        first = int(extra[0]) if extra else 0
+        _require_cuda(qkv, inv_freq, q_out, key_cache, val_cache)
+        capi.check(capi.lib().art_rope_qkv_store_rows(c_void_p(qkv.data_ptr()), c_void_p(inv_freq.data_ptr()), c_void_p(q_out.data_ptr()),
+                                                     c_void_p(key_cache.data_ptr()), c_void_p(val_cache.data_ptr()), T, heads, head_dim,
+                                                     first, key_cache.numel() // (heads * head_dim), c_void_p(current_stream_handle())))
+        return q_out
+
+
+builtin('rope_qkv_store_rows_f16')(lambda: RopeQkvStoreRows())
+
+
 class GreedyNext:
     """``greedy_next_f16(logits[V], prompt[L] or None, token[1], pos[1], embed[V, D], x[D])``: the bookkeeping
     between two decode steps in one launch - pos += 1; token = prompt[pos] while the prompt lasts, else

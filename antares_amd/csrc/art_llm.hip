@@ -356,6 +356,35 @@ __global__ __launch_bounds__(256) void rope_qkv_store_kernel(const T* __restrict
   }
 }
 
+// The same for the T tokens of a prompt (row t of qkv at position first_pos + t): rotated q to q_out[t], rotated k and
+// v into cache rows first_pos + t.  grid.y = t; the threads of a block walk the row's pairs with j fastest, so loads and
+// stores of a wavefront are 128 contiguous bytes.
+__global__ __launch_bounds__(256) void rope_qkv_store_rows_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ freq,
+                                                                   _Float16* __restrict__ q_out, _Float16* __restrict__ key_cache,
+                                                                   _Float16* __restrict__ val_cache, int heads, int half,
+                                                                   int first_pos) {
+  const int t = blockIdx.y, pos = first_pos + t;
+  const int dim = heads * half * 2, pairs = heads * half;
+  const _Float16* row = qkv + (size_t)t * 3 * dim;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < 2 * pairs) {                       // q pairs, then k pairs
+    const bool is_k = i >= pairs;
+    const int p = is_k ? i - pairs : i;
+    const int h = p / half, j = p % half;
+    const _Float16* src = row + (is_k ? dim : 0);
+    _Float16* dst = is_k ? key_cache + (size_t)pos * dim : q_out + (size_t)t * dim;
+    float s, c;
+    sincosf((float)pos * (float)freq[j], &s, &c);
+    const size_t a = (size_t)h * 2 * half + j, b = a + half;
+    const float xa = (float)src[a], xb = (float)src[b];
+    dst[a] = (_Float16)(xa * c - xb * s);
+    dst[b] = (_Float16)(xb * c + xa * s);
+  } else if (i < 2 * pairs + dim) {          // v row copy
+    const int e = i - 2 * pairs;
+    val_cache[(size_t)pos * dim + e] = row[2 * (size_t)dim + e];
+  }
+}
+
 }  // namespace
 
 // dtype codes: 0 = float32, 1 = float16
@@ -443,6 +472,22 @@ extern "C" int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, voi
   if (dtype == 0) { if (freq_dtype == 0) ART_RQS(float, float); else ART_RQS(float, _Float16); }
   else { if (freq_dtype == 0) ART_RQS(_Float16, float); else ART_RQS(_Float16, _Float16); }
 #undef ART_RQS
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int art_rope_qkv_store_rows(const void* qkv_dev, const void* freq_dev, void* q_out_dev, void* key_cache_dev,
+                                       void* val_cache_dev, int rows, int heads, int head_dim, int first_pos, int max_positions,
+                                       void* stream) {
+  ART_REQUIRE(qkv_dev && freq_dev && q_out_dev && key_cache_dev && val_cache_dev, "art_rope_qkv_store_rows: null pointer");
+  ART_REQUIRE(heads >= 1 && head_dim >= 2 && head_dim % 2 == 0, "art_rope_qkv_store_rows: bad shape");
+  ART_REQUIRE(rows >= 1 && rows <= 65535 && first_pos >= 0 && first_pos + rows <= max_positions,
+              "art_rope_qkv_store_rows: positions %d..%d do not fit caches of %d rows", first_pos, first_pos + rows - 1, max_positions);
+  const int half = head_dim / 2, dim = heads * head_dim;
+  const dim3 grid((2 * heads * half + dim + 255) / 256, rows), block(256);
+  rope_qkv_store_rows_kernel<<<grid, block, 0, (hipStream_t)stream>>>((const _Float16*)qkv_dev, (const _Float16*)freq_dev,
+                                                                      (_Float16*)q_out_dev, (_Float16*)key_cache_dev,
+                                                                      (_Float16*)val_cache_dev, heads, half, first_pos);
   ART_LAUNCH_CHECK();
   return 0;
 }

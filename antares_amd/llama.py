@@ -213,23 +213,10 @@ class LlamaInt4Decoder:
             return ExportedOp(ir, list(inputs), name=name)
         cfg = self.cfg
         d, H, D, F, V = cfg.dim, cfg.n_heads, cfg.head_dim, cfg.ffn, cfg.vocab
-        J = D // 2
         f32 = '.to(`float32`)'
-        ang = f'(T{f32} * freq[J]{f32})'
-        rope = (f'(src[T, {{base}} + H * {D} + P * {J} + J]{f32} * {ang}.call(`cos`) + (P * 2 - 1){f32} * '
-                f'src[T, {{base}} + H * {D} + (1 - P) * {J} + J]{f32} * {ang}.call(`sin`)).to(`float16`) where H in {H}, P in 2, J in {J}')
         ops = {
             'embed': program(ir='emb[T, D] = table[tok[T], D]', inputs=[f'table=float16[{V}, {d}]', f'tok=int32[{T}]'],
                               name=f'prefill_embed_{T}'),
-            'rms': program(ir=f'ss[T] +=! x[T, D]{f32} * x[T, D]{f32}; '
-                               f'out[T, D] = (x[T, D]{f32} * (ss[T] * {1.0 / d!r} + {cfg.rms_eps!r}).call(`rsqrt`) * w[D]{f32}).to(`float16`)',
-                            inputs=[f'x=float16[{T}, {d}]', f'w=float16[{d}]'], name=f'prefill_rmsnorm_{T}'),
-            'rope_q': program(ir='qr[T, H, P, J] = ' + rope.format(base=0), inputs=[f'src=float16[{T}, {3 * d}]', f'freq=float16[{D}]'],
-                               name=f'prefill_rope_q_{T}'),
-            'rope_k': program(ir='kr[T, H, P, J] = ' + rope.format(base=d), inputs=[f'src=float16[{T}, {3 * d}]', f'freq=float16[{D}]'],
-                               name=f'prefill_rope_k_{T}'),
-            'copy_v': program(ir=f'vc[T, D] = src[T, {2 * d} + D] where D in {d}', inputs=[f'src=float16[{T}, {3 * d}]'],
-                               name=f'prefill_copy_v_{T}'),
             'silu_mul': program(
                 ir=f'hid[T, N] = (gu[T, N]{f32} / (1.0 + (0.0 - gu[T, N]{f32}).call(`exp`)) * gu[T, {F} + N]{f32}).to(`float16`) where N in {F}',
                 inputs=[f'gu=float16[{T}, {2 * F}]'], name=f'prefill_silu_mul_{T}'),
@@ -243,7 +230,7 @@ class LlamaInt4Decoder:
         prompt (`attention_causal_f16`, matrix cores), keys and values land in cache rows 0..T-1.  Leaves the step
         state at the last prompt position (self.pos = T - 1, self.x = its hidden state, self.logits = its logits), so
         `advance()` and the recorded decode step continue from there.  Same operators and roundings as the one-token
-        step, applied to T rows.  With ``graph`` the pass is recorded once per prompt length in a HIP graph (about 450
+        step, applied to T rows.  With ``graph`` the pass is recorded once per prompt length in a HIP graph (about 420
         launches) and replayed on later calls with the new tokens copied into the recorded input."""
         T = int(tokens.numel())
         if not 4 <= T <= self.cfg.max_seq:
@@ -282,22 +269,23 @@ class LlamaInt4Decoder:
         x = ops['embed'](self.w['embed'], tokens.view(T))
         qkv, proj = torch.empty(T, 3 * d, **f16), torch.empty(T, d, **f16)
         gu = torch.empty(T, 2 * F, **f16)
+        qr = torch.empty(T, H, D, **f16)
 
         def linear(inp, lin, out):
             self.gemv(inp, lin['qweight'], lin['scales'], lin['qzeros'], out=out)
 
+        def rms(inp, weight):           # the built-in operator takes rows: one launch for the T positions
+            return self.autort.ops.rmsnorm_f16(inp, None, weight, extra=[1.0 / d, cfg.rms_eps])
+
         for l, lw in enumerate(self.w['layers']):
-            xb = ops['rms'](x, lw['att_norm'])
+            xb = rms(x, lw['att_norm'])
             linear(xb, lw['qkv'], qkv)
-            kc, vc = self.key_cache[l][:T], self.val_cache[l][:T]
-            qr = ops['rope_q'](qkv, self.inv_freq)
-            ops['rope_k'](qkv, self.inv_freq, out=kc.view(T, H, 2, D // 2))
-            ops['copy_v'](qkv, out=vc)
-            att = self.autort.ops.attention_causal_f16(qr.view(T, H, D), self.key_cache[l].view(cfg.max_seq, H, D),
+            self.autort.ops.rope_qkv_store_rows_f16(qkv, self.inv_freq, qr, self.key_cache[l], self.val_cache[l])
+            att = self.autort.ops.attention_causal_f16(qr, self.key_cache[l].view(cfg.max_seq, H, D),
                                                        self.val_cache[l].view(cfg.max_seq, H, D), self.att_f)
             linear(att.view(T, d), lw['o'], proj)
             self.add(x.view(-1), proj.view(-1))
-            xb = ops['rms'](x, lw['ffn_norm'])
+            xb = rms(x, lw['ffn_norm'])
             linear(xb, lw['gate_up'], gu)
             hid = ops['silu_mul'](gu)
             linear(hid, lw['down'], proj)

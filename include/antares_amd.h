@@ -239,6 +239,11 @@ int art_rotary(const void* x_dev, const void* freq_dev, void* out_dev, int heads
 int art_rope_qkv_store(const void* qkv_dev, const void* freq_dev, void* q_out_dev, void* key_cache_dev, void* val_cache_dev,
                        int heads, int head_dim, const void* pos_dev, int max_positions, int dtype, int freq_dtype,
                        void* stream);
+/* art_rope_qkv_store for the `rows` tokens of a prompt (fp16; qkv [rows, 3 * heads * head_dim], row t at position
+ * first_pos + t): rotated q into q_out [rows, heads, head_dim], rotated k and v into cache rows first_pos + t.  The
+ * positions are host values here; they must fit the caches (max_positions rows). */
+int art_rope_qkv_store_rows(const void* qkv_dev, const void* freq_dev, void* q_out_dev, void* key_cache_dev, void* val_cache_dev,
+                            int rows, int heads, int head_dim, int first_pos, int max_positions, void* stream);
 /* art_rope_qkv_store and art_decode_attention in one launch (fp16): block h rotates its head's q and k,
  * writes k and v into cache row *pos_dev and attends over rows 0..*pos_dev.  The caches have max_positions rows:
  * a position outside 0..max_positions-1 (a recorded graph replayed once too often) touches no cache row and

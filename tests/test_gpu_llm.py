@@ -320,3 +320,34 @@ def test_causal_attention_over_a_prompt_against_the_oracle(T, H):
     sc = sc.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float('-inf'))
     exact = torch.einsum('hts,shd->thd', torch.softmax(sc, -1), vd[:T]).numpy()
     assert np.allclose(out.astype(np.float64), exact, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.usefixtures('oracle_built')
+def test_rope_qkv_store_rows_against_the_oracle():
+    """The prompt form of rope_qkv_store: row t rotated at position first_pos + t, k and v into those cache rows."""
+    import autort
+    from oracle import hot_ops
+    dev = autort.device()
+    T, H, D, S, first = 9, 4, 128, 20, 3
+    g = torch.Generator().manual_seed(77)
+    note('rope_qkv_store_rows')
+    qkv = torch.randn(T, 3 * H * D, generator=g).half()
+    inv = (1.0 / (10000 ** (torch.arange(0, D, 2).float() / D))).half()
+    inv_freq = torch.cat([inv, inv])
+    kc = torch.randn(S, H * D, generator=g).half()
+    vc = torch.randn(S, H * D, generator=g).half()
+    kd, vd = kc.to(dev), vc.to(dev)
+    q_out = torch.zeros(T, H, D, dtype=torch.float16, device=dev)
+    autort.ops.rope_qkv_store_rows_f16(qkv.to(dev), inv_freq.to(dev), q_out, kd, vd, extra=[first])
+    for t in range(T):
+        q, k, v = qkv[t, :H * D].numpy(), qkv[t, H * D:2 * H * D].numpy(), qkv[t, 2 * H * D:].numpy()
+        want_q = hot_ops.rotary(q.reshape(H, 2, D // 2), inv_freq.numpy(), first + t)
+        want_k = hot_ops.rotary(k.reshape(H, 2, D // 2), inv_freq.numpy(), first + t)
+        assert np.allclose(q_out[t].float().cpu().numpy(), want_q.astype(np.float32), **FP16_TOL)
+        assert np.allclose(kd[first + t].float().cpu().numpy(), want_k.reshape(-1).astype(np.float32), **FP16_TOL)
+        assert np.array_equal(vd[first + t].cpu().numpy(), v)
+    keep = [s for s in range(S) if not first <= s < first + T]
+    assert torch.equal(kd.cpu()[keep], kc[keep]) and torch.equal(vd.cpu()[keep], vc[keep])
+    # positions that do not fit the caches are refused on the host
+    with pytest.raises(Exception, match='do not fit'):
+        autort.ops.rope_qkv_store_rows_f16(qkv.to(dev), inv_freq.to(dev), q_out, kd, vd, extra=[S - T + 1])
