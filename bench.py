@@ -97,8 +97,18 @@ def bench_read_floor(torch, capi, steps, warmup, nbytes=2048 * 11008, layers=LAY
         for b in bufs:
             capi.check(capi.lib().art_read_bytes(c_void_p(b.data_ptr()), nbytes, c_void_p(sink.data_ptr()), c_void_p(stream)))
     sec = time_graph(torch, capi, one_pass, steps, warmup) / layers
+
+    # the same launch over 32 KiB (one block): what a dependent kernel node costs before it has moved any bytes
+    small = [b[:32768] for b in bufs]
+
+    def tiny_pass():
+        stream = torch.cuda.current_stream().cuda_stream
+        for b in small:
+            capi.check(capi.lib().art_read_bytes(c_void_p(b.data_ptr()), 32768, c_void_p(sink.data_ptr()), c_void_p(stream)))
+    tiny = time_graph(torch, capi, tiny_pass, steps, warmup) / layers
     return {'kernel': 'art_read_kernel', 'bytes_per_launch': nbytes, 'us_per_launch': round(sec * 1e6, 3),
-            'gbps': round(nbytes / sec / 1e9, 1), 'frac_of_peak': round(nbytes / sec / 1e9 / HBM_PEAK_GBPS, 4)}
+            'gbps': round(nbytes / sec / 1e9, 1), 'frac_of_peak': round(nbytes / sec / 1e9 / HBM_PEAK_GBPS, 4),
+            'us_per_launch_of_one_block': round(tiny * 1e6, 3)}
 
 
 _SIDE_STREAM = None

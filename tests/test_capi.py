@@ -70,3 +70,26 @@ def test_operator_refuses_cpu_tensors():
         f(torch.zeros(8))
     with pytest.raises(TypeError, match='must be float32'):
         f(torch.zeros(8, dtype=torch.int32))
+
+
+@pytest.mark.gpu
+def test_device_copies_and_the_read_only_launch():
+    """art_memcpy_dtod (ab::memcpyDtoD) copies on the stream it is given; art_read_bytes reads a buffer and writes nothing."""
+    import torch
+    from ctypes import c_void_p
+    from antares_amd.runtime import capi
+    capi.init(0)
+    l = capi.lib()
+    src = torch.arange(1 << 20, dtype=torch.int32, device='cuda')
+    dst = torch.zeros_like(src)
+    capi.check(l.art_memcpy_dtod(c_void_p(dst.data_ptr()), c_void_p(src.data_ptr()), src.numel() * 4, None))
+    capi.check(l.art_stream_synchronize(None))
+    assert torch.equal(dst, src)
+    sink = torch.zeros(4096, dtype=torch.int32, device='cuda')
+    buf = torch.randint(0, 256, (2048 * 11008,), dtype=torch.uint8, device='cuda')
+    before = buf.clone()
+    capi.check(l.art_read_bytes(c_void_p(buf.data_ptr()), buf.numel(), c_void_p(sink.data_ptr()), None))
+    capi.check(l.art_read_bytes(c_void_p(buf.data_ptr()), 32768 * 3, c_void_p(sink.data_ptr()), None))
+    torch.cuda.synchronize()
+    assert torch.equal(buf, before) and int(sink.abs().sum()) == 0
+    assert l.art_read_bytes(c_void_p(buf.data_ptr()), 1000, c_void_p(sink.data_ptr()), None) != 0
