@@ -347,6 +347,30 @@ class AttentionRopeSplit:
         return partial
 
 
+class GemmW4Residual:
+    """``gemm_w4a16_residual(x[M,K], qweight, scales, qzeros, out[M,N], residual=None)``: the packed int4 product for a
+    batch of rows on the matrix cores with the residual add folded in (``out`` may be the residual itself)."""
+    name = 'gemm_w4a16_residual'
+
+    def __call__(self, x, qweight, scales, qzeros, out, residual=None):
+        M, K = x.shape
+        N = qweight.shape[1]
+        if qweight.shape[0] * 2 != K or scales.shape != (K // 128, N) or qzeros.shape != (K // 128, N // 2) or out.shape != (M, N):
+            raise ValueError('gemm_w4a16_residual: operand shapes do not match M, K, N')
+        if x.dtype != torch.float16 or scales.dtype != torch.float16 or out.dtype != torch.float16 or \
+                (residual is not None and (residual.dtype != torch.float16 or residual.shape != out.shape)):
+            raise TypeError('gemm_w4a16_residual: x, scales, out and residual must be float16 (residual of the shape of out)')
+        _require_cuda(*([x, qweight, scales, qzeros, out] + ([residual] if residual is not None else [])))
+        capi.check(capi.lib().art_gemm_w4a16_residual(
+            c_void_p(x.data_ptr()), c_void_p(qweight.data_ptr()), c_void_p(scales.data_ptr()), c_void_p(qzeros.data_ptr()),
+            c_void_p(out.data_ptr()), c_void_p(residual.data_ptr() if residual is not None else 0), M, K, N, 0,
+            c_void_p(current_stream_handle())))
+        return out
+
+
+builtin('gemm_w4a16_residual')(lambda: GemmW4Residual())
+
+
 class GemvW4Attn:
     """``gemv_w4a16_attn(partial[H, P, 132], qweight, scales, qzeros, out[N], residual=None)``: the int4 projection of a
     split attention's output (merged on the fly) with the residual add folded in."""

@@ -68,7 +68,8 @@ __global__ __launch_bounds__(kThreads, 512 / kThreads) void gemm_w4a16_kernel(co
                                                              const _Float16* __restrict__ scales,
                                                              const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y,
                                                              float* __restrict__ partial, int M_total, int K, int N, int splits,
-                                                             int col_tiles, int m_blocks, Magic mg) {
+                                                             int col_tiles, int m_blocks, Magic mg,
+                                                             const _Float16* __restrict__ residual) {
   extern __shared__ __align__(16) _Float16 smem[];
   _Float16* Ws = smem;                           // [2][SK][W_LD]
   _Float16* Xs = smem + 2 * W_TILE;              // [2][BM][X_LD]
@@ -87,6 +88,7 @@ __global__ __launch_bounds__(kThreads, 512 / kThreads) void gemm_w4a16_kernel(co
   const int M = M_total - m0 < BM ? M_total - m0 : BM;          // rows of this block
   x += (size_t)m0 * K;
   y += (size_t)m0 * N;
+  if (residual) residual += (size_t)m0 * N;
   const int g_begin = (int)((long long)G * split / splits), g_end = (int)((long long)G * (split + 1) / splits);
   const int groups = g_end - g_begin;
 
@@ -288,20 +290,30 @@ __global__ __launch_bounds__(kThreads, 512 / kThreads) void gemm_w4a16_kernel(co
     for (int r = 0; r < 16; ++r) {
       const int row = t * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
       if (row < M) {
-        if (splits == 1) y[(size_t)row * N + my_col] = (_Float16)total[t][r];
+        if (splits == 1) {
+          _Float16 o = (_Float16)total[t][r];
+          if (residual) o = (_Float16)((float)o + (float)residual[(size_t)row * N + my_col]);      // may alias y: same element
+          y[(size_t)row * N + my_col] = o;
+        }
         else partial[((size_t)split * M_total + m0 + row) * N + my_col] = total[t][r];
       }
     }
 }
 
 // y[m,n] = fp16(sum over splits, in split order); four columns per thread (N % 4 == 0).
-__global__ __launch_bounds__(256) void gemm_w4a16_combine_kernel(const float* __restrict__ partial, _Float16* __restrict__ y,
-                                                                  long long count4, long long split_stride, int splits) {
+__global__ __launch_bounds__(256) void gemm_w4a16_combine_kernel(const float* __restrict__ partial, _Float16* y,
+                                                                  long long count4, long long split_stride, int splits,
+                                                                  const _Float16* residual) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i >= count4) return;
   f32x4 t = *reinterpret_cast<const f32x4*>(partial + i * 4);
   for (int s = 1; s < splits; ++s) t += *reinterpret_cast<const f32x4*>(partial + s * split_stride + i * 4);
-  const h4 out = h4{(_Float16)t[0], (_Float16)t[1], (_Float16)t[2], (_Float16)t[3]};
+  h4 out = h4{(_Float16)t[0], (_Float16)t[1], (_Float16)t[2], (_Float16)t[3]};
+  if (residual) {                    // y = fp16(fp16(product) + residual); residual may be y itself
+    const h4 res = *reinterpret_cast<const h4*>(residual + i * 4);
+    out = h4{(_Float16)((float)out[0] + (float)res[0]), (_Float16)((float)out[1] + (float)res[1]),
+             (_Float16)((float)out[2] + (float)res[2]), (_Float16)((float)out[3] + (float)res[3])};
+  }
   *reinterpret_cast<h4*>(y + i * 4) = out;
 }
 
@@ -330,6 +342,13 @@ extern "C" int art_gemm_w4a16(const void* x_dev, const void* qweight_dev, const 
 
 extern "C" int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                                     void* y_dev, int M, int K, int N, int k_splits, void* stream) {
+  return art_gemm_w4a16_residual(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, nullptr, M, K, N, k_splits, stream);
+}
+
+extern "C" int art_gemm_w4a16_residual(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                                       void* y_dev, const void* residual_dev, int M, int K, int N, int k_splits, void* stream) {
+  ART_REQUIRE(((uintptr_t)residual_dev % 8) == 0, "art_gemm_w4a16: the residual must be 8-byte aligned");
+  ART_REQUIRE(!art::overlaps(x_dev, (size_t)M * K * 2, y_dev, (size_t)M * N * 2), "art_gemm_w4a16: y must not overlap x");
   ART_REQUIRE(k_splits >= 0, "art_gemm_w4a16: k_splits must be 0 (library's choice) or positive (got %d)", k_splits);
   ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemm_w4a16: null pointer");
   ART_REQUIRE(M >= 1, "art_gemm_w4a16: M must be positive (got %d)", M);
@@ -369,20 +388,21 @@ extern "C" int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, 
     }
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m0 * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m0 * N;
+    const _Float16* rs = residual_dev ? (const _Float16*)residual_dev + (size_t)m0 * N : nullptr;
     const dim3 grid((unsigned)((col_tiles * splits + 7) / 8 * 8 * m_blocks));
     if (rows <= 32)
       gemm_w4a16_kernel<1><<<grid, kThreads, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
-                                                         col_tiles, m_blocks, mg);
+                                                         col_tiles, m_blocks, mg, rs);
     else
       gemm_w4a16_kernel<2><<<grid, kThreads, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
-                                                         col_tiles, m_blocks, mg);
+                                                         col_tiles, m_blocks, mg, rs);
     ART_LAUNCH_CHECK();
     if (splits > 1) {
       const long long count4 = (long long)rows * N / 4;
       gemm_w4a16_combine_kernel<<<dim3((unsigned)((count4 + 255) / 256)), 256, 0, st>>>(scratch, ys, count4, (long long)rows * N,
-                                                                                        splits);
+                                                                                        splits, rs);
       ART_LAUNCH_CHECK();
     }
   }

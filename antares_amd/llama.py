@@ -267,12 +267,15 @@ class LlamaInt4Decoder:
         ops = self._prefill_ops(T)
         f16 = dict(dtype=torch.float16, device=self.dev)
         x = ops['embed'](self.w['embed'], tokens.view(T))
-        qkv, proj = torch.empty(T, 3 * d, **f16), torch.empty(T, d, **f16)
+        qkv = torch.empty(T, 3 * d, **f16)
         gu = torch.empty(T, 2 * F, **f16)
         qr = torch.empty(T, H, D, **f16)
 
         def linear(inp, lin, out):
             self.gemv(inp, lin['qweight'], lin['scales'], lin['qzeros'], out=out)
+
+        def gemm_res(inp, lin, acc):    # acc += inp @ W, the residual add folded into the projection
+            self.autort.ops.gemm_w4a16_residual(inp, lin['qweight'], lin['scales'], lin['qzeros'], acc, residual=acc)
 
         def rms(inp, weight):           # the built-in operator takes rows: one launch for the T positions
             return self.autort.ops.rmsnorm_f16(inp, None, weight, extra=[1.0 / d, cfg.rms_eps])
@@ -283,13 +286,11 @@ class LlamaInt4Decoder:
             self.autort.ops.rope_qkv_store_rows_f16(qkv, self.inv_freq, qr, self.key_cache[l], self.val_cache[l])
             att = self.autort.ops.attention_causal_f16(qr, self.key_cache[l].view(cfg.max_seq, H, D),
                                                        self.val_cache[l].view(cfg.max_seq, H, D), self.att_f)
-            linear(att.view(T, d), lw['o'], proj)
-            self.add(x.view(-1), proj.view(-1))
+            gemm_res(att.view(T, d), lw['o'], x)
             xb = rms(x, lw['ffn_norm'])
             linear(xb, lw['gate_up'], gu)
             hid = ops['silu_mul'](gu)
-            linear(hid, lw['down'], proj)
-            self.add(x.view(-1), proj.view(-1))
+            gemm_res(hid, lw['down'], x)
         self.x.copy_(x[T - 1])
         self.pos.fill_(T - 1)
         self.token.copy_(tokens.view(T)[T - 1:T])

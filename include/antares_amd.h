@@ -149,6 +149,10 @@ int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void*
 int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                          void* y_dev, int M, int K, int N, int k_splits, void* stream);
 int art_partition_even_first_i32_tuned(const void* in_dev, void* out_dev, long long n, int max_blocks, void* stream);
+/* art_gemm_w4a16_tuned with the residual add that follows a projection (samples/05_llama2_7b_int4.py:168,173) folded
+ * into the last pass: y = fp16(fp16(product) + residual).  residual_dev: fp16 [M,N], may be y itself, may be NULL. */
+int art_gemm_w4a16_residual(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                            void* y_dev, const void* residual_dev, int M, int K, int N, int k_splits, void* stream);
 
 /* art_gemv_w4a16 for callers that cannot allocate device memory or let a library do it (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same

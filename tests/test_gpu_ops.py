@@ -461,3 +461,25 @@ def test_fp16_reductions_where_tree_order_leaves_the_sequential_oracle(autort):
     assert np.all(want < 0.5 * exact)                      # the sequential fp16 sum has stalled (near 2048)
     assert np.allclose(got, exact, rtol=1e-2)              # the tree-ordered one has not
     assert np.all(np.abs(got - exact) < np.abs(want - exact))
+
+
+@pytest.mark.parametrize('M,K,N', [(5, 512, 272), (64, 4096, 4096), (128, 1024, 1040), (200, 4096, 512)])
+def test_w4a16_gemm_with_the_residual_folded_in(autort, M, K, N):
+    """gemm_w4a16_residual: y = fp16(fp16(x @ W) + residual), in place on the residual, with and without K-splits."""
+    from oracle import hot_ops
+    note(f'w4a16 gemm + residual M={M} K={K} N={N}')
+    dev = autort.device()
+    p = workloads.w4_problem(K + N + M, M, K, N)
+    res = torch.randn(M, N, generator=torch.Generator().manual_seed(M)).half()
+    prod = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy())
+    want = (prod.astype(np.float32) + res.numpy().astype(np.float32)).astype(np.float16).astype(np.float32)
+    d = [p[k].to(dev) for k in ('x', 'qweight', 'scales', 'qzeros')]
+    acc = res.to(dev).clone()
+    autort.ops.gemm_w4a16_residual(*d, acc, residual=acc)
+    assert np.allclose(acc.float().cpu().numpy(), want, **FP16_TOL)
+    out = torch.empty_like(acc)
+    autort.ops.gemm_w4a16_residual(*d, out, residual=res.to(dev))
+    assert torch.equal(out, acc)
+    plain = torch.empty_like(acc)
+    autort.ops.gemm_w4a16_residual(*d, plain)
+    assert np.allclose(plain.float().cpu().numpy(), prod.astype(np.float32), **FP16_TOL)
