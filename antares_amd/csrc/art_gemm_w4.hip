@@ -1,79 +1,102 @@
 // Weight-only int4 GEMM for a batch of rows (prefill, four rows and more): the same arithmetic as the GEMV of
 // art_gemv_w4.hip,
-//     y[m,n] = sum_g s[g,n] * sum_{k in group g} x[m,k] * (q[k,n] - z[g,n]),      group = 128 k,
-// with the inner sums on the matrix cores.  Replaces the kernel the reference generates when the
-// dequant + matmul program of samples/05_llama2_7b_int4.py:135-144 is exported with a batch axis.
+//     y[m,n] = sum_k x[m,k] * w[k,n],   w[k,n] = fp16(s[g,n] * fp16(q[k,n] - z[g,n])),   group g = k / 128,
+// on the matrix cores with fp32 accumulation; w is rounded exactly as the reference's dequant + matmul program
+// does (samples/05_llama2_7b_int4.py:135-144 exported with a batch axis).
 //
 // Design for MI355X:
-//   * the weights are read from HBM exactly once; a block of eight waves owns 256 columns (two full
-//     128-byte lines of every packed row, and as many bytes of weights as of x per step) and a contiguous
-//     range of k groups;
-//   * unpacking is fused into the LDS staging: 16 bytes (16 columns x 2 k) become two rows of fp16
-//     (q - z) values - exact small integers - with one shift, four v_bitop3_b32 and four packed
-//     subtractions per word.  The columns of every group of four land in LDS in the order 0,2,1,3,
-//     which costs nothing: the column an accumulator lane owns is permuted the same way and undone
-//     in the epilogue;
-//   * v_mfma_f32_32x32x16_f16 per wave: 32 columns x 64 rows, B operand through ds_read_b64_tr_b16;
-//     the group sum is scaled by s[g,n] in fp32 afterwards (one scalar per lane, since an accumulator
-//     lane owns one column), so no scale is rounded to fp16;
-//   * a step is 64 k.  LDS holds two steps: while the matrix cores work on step t, the same waves
-//     unpack step t+1 into the other buffer; one barrier per step, and it waits for LDS only, so the
-//     register stages (a whole group = two steps each, two of them) keep their global loads in flight
-//     across it.  92 KiB of LDS and < 256 registers: one block = two waves per SIMD on every compute unit;
-//   * split-K without atomics (5.6 M float atomics cost 75 us on this chip): each K-split writes its
-//     fp32 tile to the library workspace and a second small kernel adds the splits in a fixed order
-//     and rounds once to fp16 - results do not depend on timing.
+//   * a block of eight wavefronts owns 256 columns, up to 64 rows and a contiguous range of quantisation groups; it
+//     works one group (128 k) per loop iteration;
+//   * everything a group needs - 16 KiB of packed weights, 16 KiB of x, 512 B of scales, 128 B of zero points - goes
+//     from global memory straight into LDS (global_load_lds_dwordx4 / _dword: no registers hold data in flight), into
+//     a ring of four stages, so three groups (100 KiB per compute unit) are on their way while one is multiplied.
+//     Register staging two groups ahead held a compute unit to about 45 GB/s; this ring sustains over 100 GB/s;
+//   * each lane chooses which 16-byte chunk it fetches, and LDS position (row r, chunk c) holds chunk c ^ (r & 7) of
+//     the weights (c ^ (r & 15) of x): the reads below then touch every bank once although rows are 256 bytes apart;
+//   * the packed bytes stay packed in LDS.  ds_read_b64_tr_b8 hands a lane the 8 bytes = 16 values of k of ONE column,
+//     i.e. the B operand of two v_mfma_f32_32x32x16_f16; a lane unpacks only the columns it multiplies (one shift,
+//     four v_bitop3_b32, four packed subtractions of the zero point, four packed multiplications by the scale per
+//     word).  The nibble extraction leaves k in the order 0 4 1 5 2 6 3 7; the A operand is permuted the same way
+//     (four v_perm_b32 per 16 bytes of x);
+//   * wavefront (c, h) multiplies 64 columns (c = 0..3) by the k half h of every group: per group 16 bytes of x and
+//     of packed weights per lane and MFMA, 112 KiB of LDS traffic per group instead of 280 KiB with fp16 weights in
+//     LDS; the two k halves meet in LDS once, after the loop;
+//   * the loop is rolled (one group per iteration, one barrier): the whole kernel is 7 KiB of code.  A launch fetches
+//     its code cold - straight-line code costs about 0.3 us per KiB executed - so unrolled stages are not free;
+//   * split-K without atomics (5.6 M float atomics cost 75 us on this chip): each K-split writes its fp32 tile to the
+//     library workspace and a second small kernel adds the splits in a fixed order and rounds once to fp16 - results
+//     do not depend on timing.
 #include "art_common.h"
-
-#include <type_traits>
 
 namespace {
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
 
-constexpr int kThreads = 512;                  // 8 waves: 32 columns each
-constexpr int BM = 64, BN = kThreads / 2, GK = 128;   // rows and columns of a block, k of a quantisation group
-constexpr int SK = 64;                         // k of a step (half a group)
-constexpr int W_LD = BN + 32;                  // halves per weight row in LDS: 320 bytes, so the four k rows
-                                               // a transposing read touches fall on disjoint banks
-constexpr int X_LD = SK + 8;                   // halves per x row in LDS (144 bytes)
-constexpr int W_TILE = SK * W_LD, X_TILE = BM * X_LD;
-constexpr size_t kLdsBytes = (size_t)2 * (W_TILE + X_TILE) * sizeof(_Float16);
+constexpr int kThreads = 512;                       // 8 wavefronts: 4 column quarters x 2 k halves
+constexpr int BM = 64, BN = 256, GK = 128;          // rows and columns of a block, k of a quantisation group
+constexpr int NS = 4;                               // stages of the LDS ring, one quantisation group each
+constexpr int W_BYTES = (GK / 2) * BN;              // packed weights of a group: 64 byte-rows x 256 columns
+constexpr int X_BYTES = BM * GK * 2;                // x of a group: 64 rows x 128 k, fp16
+constexpr int Q_BYTES = 2048;                       // scales (512 B) at 0, zero points (128 B) at 512; the rest takes the idle lanes
+constexpr int STAGE = W_BYTES + X_BYTES + Q_BYTES;
+constexpr int RLD = BN + 4;                         // floats per row of a result tile in LDS
+constexpr size_t kLdsBytes = (size_t)NS * STAGE;    // 139264; the two result tiles of the epilogue (133120) reuse it
+constexpr int kLoadsPerGroup = 5;                   // LDS-direct loads per wavefront and group: 2 weights, 2 x, 1 scales / zero points
+static_assert(2 * BM * RLD * sizeof(float) <= kLdsBytes, "the result tiles fit the ring");
 
 struct Magic {
   unsigned int mask_lo, mask_hi, bias_lo, bias_hi;   // 0x000F000F 0x00F000F0 0x64006400 0x54005400
 };
 
 __device__ __forceinline__ h2 as_h2(unsigned int v) { return __builtin_bit_cast(h2, v); }
-__device__ __forceinline__ unsigned int as_u32(h2 v) { return __builtin_bit_cast(unsigned int, v); }
 
 // (w & mask) | bias in one v_bitop3_b32 (truth table 0xEA = (a & b) | c).
 __device__ __forceinline__ unsigned int and_or(unsigned int w, unsigned int mask, unsigned int bias) {
   return __builtin_amdgcn_bitop3_b32(w, mask, bias, 0xEA);
 }
 
-// Position p of a staged column <-> column of the matrix: bits 0 and 1 swapped.
-__device__ __forceinline__ int unpermute(int p) { return (p & ~3) | ((p & 1) << 1) | ((p >> 1) & 1); }
+// 8 halves of x in the k order the nibble extraction leaves in a B operand: k0 k4 k1 k5 k2 k6 k3 k7.
+__device__ __forceinline__ h8 permute_k(u32x4 v) {
+  u32x4 o;
+  o[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
+  o[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
+  o[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
+  o[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
+  return __builtin_bit_cast(h8, o);
+}
+
+// 64 lanes x 16 (4) bytes from global memory straight into LDS: lane l's bytes land at lds_dst + 16 l (4 l); the lane
+// chooses its global address freely.  The instruction takes the LDS address from m0, which is put back afterwards.
+// Counted by vmcnt like any load; the compiler does not see these loads, so every wait for them below is written by
+// hand (the compiler's own builtin for this instruction makes it wait for vmcnt(0) before every LDS read).
+__device__ __forceinline__ void load_lds_x4(const void* g, unsigned int lds_dst) {
+  unsigned int keep;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(keep) : "v"(g), "s"(lds_dst) : "memory");
+}
+__device__ __forceinline__ void load_lds_x1(const void* g, unsigned int lds_dst) {
+  unsigned int keep;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %1, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(keep) : "v"(g), "s"(lds_dst) : "memory");
+}
 
 template <int MT>   // MT accumulator tiles of 32 rows: 1 for M <= 32, 2 for M <= 64
-__global__ __launch_bounds__(kThreads, 512 / kThreads) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
-                                                             const _Float16* __restrict__ scales,
-                                                             const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y,
-                                                             float* __restrict__ partial, int M_total, int K, int N, int splits,
-                                                             int col_tiles, int m_blocks, Magic mg,
-                                                             const _Float16* __restrict__ residual) {
-  extern __shared__ __align__(16) _Float16 smem[];
-  _Float16* Ws = smem;                           // [2][SK][W_LD]
-  _Float16* Xs = smem + 2 * W_TILE;              // [2][BM][X_LD]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__global__ __launch_bounds__(kThreads) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
+                                                              const _Float16* __restrict__ scales,
+                                                              const unsigned char* __restrict__ qzeros, _Float16* y,
+                                                              float* __restrict__ partial, int M_total, int K, int N, int splits,
+                                                              int col_tiles, int m_blocks, Magic mg,
+                                                              const _Float16* residual) {       // residual may be y itself
+  extern __shared__ __align__(1024) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int cw = wave & 3, kh = wave >> 2;          // 64-column quarter of the tile, k half of every group
 
   // block -> (column tile, K split, block of 64 rows).  The row blocks of one (tile, split) stream the same weights:
   // they get block ids that are 8 apart, which the dispatcher places on the same XCD at the same time, so that the
@@ -91,213 +114,179 @@ __global__ __launch_bounds__(kThreads, 512 / kThreads) void gemm_w4a16_kernel(co
   if (residual) residual += (size_t)m0 * N;
   const int g_begin = (int)((long long)G * split / splits), g_end = (int)((long long)G * (split + 1) / splits);
   const int groups = g_end - g_begin;
+  const unsigned int lds0 = (unsigned int)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
-  // ---- global -> register staging, one quantisation group (two steps) per stage
-  // weights of a step: 32 packed rows x BN bytes = kThreads chunks of 16 bytes, one per thread
-  constexpr int kChunks = BN / 16;              // 16-column chunks per packed row
-  const int cc = tid % kChunks;                 // 16-column chunk
-  const int pr = tid / kChunks;                 // packed row of the step (kThreads / kChunks = 32 of them)
-  const bool col_ok = n0 + cc * 16 < N;         // N % 16 == 0: a chunk is inside or outside as a whole
-  const int wcol = col_ok ? n0 + cc * 16 : 0;   // columns past N: load valid memory, results are never stored
-  const unsigned char* wp = qweight + (size_t)pr * N + wcol;
-  // x of a step: MT*32 rows x 64 k = MT*256 chunks of 16 bytes, XC per thread; rows past M repeat row M-1
-  constexpr int XC = (MT * 256 + kThreads - 1) / kThreads;     // chunks of x per thread and step
-  const _Float16* xp[XC];
-  int xs_off[XC];
+  // ---- what this lane fetches per group: two 16-byte chunks of packed weights, two of x, one dword of scales or
+  // zero points.  Wavefront w fills LDS bytes [1024 j, 1024 j + 1024), j = w and w + 8, of the weight and the x area:
+  // rows 4 j .. 4 j + 3 of 256 bytes.  Columns past N and rows past M re-read valid memory; nothing of them is stored.
+  const unsigned char* wsrc[2];
+  const _Float16* xsrc[2];
 #pragma unroll
-  for (int i = 0; i < XC; ++i) {
-    const int c = tid + kThreads * i, row = c >> 3, kc = c & 7;
-    xp[i] = x + (size_t)(row < M ? row : M - 1) * K + kc * 8;
-    xs_off[i] = row * X_LD + kc * 8;
+  for (int u = 0; u < 2; ++u) {
+    const int r = 4 * (wave + 8 * u) + (lane >> 4);
+    const int col = n0 + ((lane & 15) ^ (r & 7)) * 16;            // N % 16 == 0: a chunk is inside or outside as a whole
+    wsrc[u] = qweight + ((size_t)g_begin * (GK / 2) + r) * N + (col < N ? col : 0);
+    xsrc[u] = x + (size_t)(r < M ? r : M - 1) * K + (size_t)g_begin * GK + ((lane & 15) ^ (r & 15)) * 8;
   }
-
-  // per-lane constants of the operand reads
-  const int a_row = lane & 31, a_k = (lane >> 5) * 8;
-  const int s16 = lane & 15;
-  const int b_k = (lane >> 5) * 8 + (s16 >> 2);
-  const int b_n = wave * 32 + ((lane & 31) >> 4) * 16 + (s16 & 3) * 4;
-  const int my_col = n0 + unpermute(wave * 32 + (lane & 31));       // the column this lane accumulates
-  const bool my_ok = my_col < N;
-  const int sc_col = my_ok ? my_col : 0;
-
-  // Stages are indexed statically (a run-time index would put the arrays in scratch memory).
-  u32x4 wq[2][2];      // [stage][step of the group]
-  u32x4 xr[2][2][XC];
-  u32x2 zq[2];
-  _Float16 sc16[2];
-  auto load_group = [&](int g, auto tag) {
-    constexpr int S = decltype(tag)::value;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-#pragma unroll
-      for (int i = 0; i < XC; ++i) xr[S][h][i] = *reinterpret_cast<const u32x4*>(xp[i] + (size_t)g * GK + h * SK);
-      wq[S][h] = *reinterpret_cast<const u32x4*>(wp + ((size_t)g * (GK / 2) + h * (SK / 2)) * N);
+  const unsigned char* qsrc;
+  int qstep;                                        // bytes from one group to the next
+  {
+    const int d = wave * 64 + lane;                 // dword of the 2 KiB area
+    if (d < 128) {                                  // scales of columns 2 d, 2 d + 1
+      const int col = n0 + 2 * d;
+      qsrc = reinterpret_cast<const unsigned char*>(scales + (size_t)g_begin * N + (col < N ? col : 0));
+      qstep = 2 * N;
+    } else if (d < 160) {                           // zero points of columns 8 (d - 128) .. + 7
+      const int col = n0 + 8 * (d - 128);
+      qsrc = qzeros + (size_t)g_begin * (N / 2) + ((col < N ? col : 0) >> 1);
+      qstep = N / 2;
+    } else {                                        // idle lanes re-read the first scales into the padding
+      qsrc = reinterpret_cast<const unsigned char*>(scales + (size_t)g_begin * N);
+      qstep = 2 * N;
     }
-    zq[S] = *reinterpret_cast<const u32x2*>(qzeros + (size_t)g * (N / 2) + (wcol >> 1));
-    sc16[S] = scales[(size_t)g * N + sc_col];
-  };
-
-  f16v total[MT], grp[MT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) total[i][r] = 0.f;
-
-  h2 z_lo[8], z_hi[8];   // zero points of this thread's 16 columns, paired (c0,c2) and (c1,c3), on both nibble biases
-  auto prepare_zeros = [&](auto tag) {
-    constexpr int S = decltype(tag)::value;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const unsigned int zw = (zq[S][j >> 1] >> ((j & 1) * 16)) & 0xffffu;   // z0 | z1<<4 | z2<<8 | z3<<12
-      const unsigned int e = zw | (zw << 8);              // z0 at bits 0-3, z2 at bits 16-19
-      const unsigned int o = (zw >> 4) | (zw << 4);       // z1 at bits 0-3, z3 at bits 16-19
-      z_lo[2 * j] = as_h2(and_or(e, mg.mask_lo, mg.bias_lo));
-      z_lo[2 * j + 1] = as_h2(and_or(o, mg.mask_lo, mg.bias_lo));
-      z_hi[2 * j] = as_h2(and_or(e << 4, mg.mask_hi, mg.bias_hi));
-      z_hi[2 * j + 1] = as_h2(and_or(o << 4, mg.mask_hi, mg.bias_hi));
-    }
-  };
-  // Unpack one step (half H of the group in stage S) into LDS buffer `buf`.
-  auto unpack = [&](int buf, auto tag, auto half_tag) {
-    constexpr int S = decltype(tag)::value, H = decltype(half_tag)::value;
-    u32x4 even[2], odd[2];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const unsigned int w = wq[S][H][j], w8 = w >> 8;
-      const h2 e02 = as_h2(and_or(w, mg.mask_lo, mg.bias_lo)) - z_lo[2 * j];
-      const h2 e13 = as_h2(and_or(w8, mg.mask_lo, mg.bias_lo)) - z_lo[2 * j + 1];
-      const h2 o02 = as_h2(and_or(w, mg.mask_hi, mg.bias_hi)) - z_hi[2 * j];
-      const h2 o13 = as_h2(and_or(w8, mg.mask_hi, mg.bias_hi)) - z_hi[2 * j + 1];
-      even[j >> 1][(j & 1) * 2] = as_u32(e02);
-      even[j >> 1][(j & 1) * 2 + 1] = as_u32(e13);
-      odd[j >> 1][(j & 1) * 2] = as_u32(o02);
-      odd[j >> 1][(j & 1) * 2 + 1] = as_u32(o13);
-    }
-    _Float16* row = Ws + buf * W_TILE + (2 * pr) * W_LD + cc * 16;       // packed row pr = k rows 2*pr, 2*pr+1 of the step
-    *reinterpret_cast<u32x4*>(row) = even[0];
-    *reinterpret_cast<u32x4*>(row + 8) = even[1];
-    *reinterpret_cast<u32x4*>(row + W_LD) = odd[0];
-    *reinterpret_cast<u32x4*>(row + W_LD + 8) = odd[1];
-#pragma unroll
-    for (int i = 0; i < XC; ++i) *reinterpret_cast<u32x4*>(Xs + buf * X_TILE + xs_off[i]) = xr[S][H][i];
-  };
-  // Operand fragments of two k-steps of 16 (kk0, kk0 + 1) of the step in LDS buffer `buf`.
-  auto read_frags = [&](h8 (&fa)[2][MT], h8 (&fb)[2], int buf, int kk0) {
-    const _Float16* ws = Ws + buf * W_TILE;
-    const _Float16* xs = Xs + buf * X_TILE;
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      const _Float16* p = ws + ((kk0 + k) * 16 + b_k) * W_LD + b_n;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * W_LD));
-      const h4 l4 = __builtin_bit_cast(h4, lo), h4v = __builtin_bit_cast(h4, hi);
-      fb[k] = h8{l4[0], l4[1], l4[2], l4[3], h4v[0], h4v[1], h4v[2], h4v[3]};
-#pragma unroll
-      for (int t = 0; t < MT; ++t) fa[k][t] = *reinterpret_cast<const h8*>(xs + (a_row + t * 32) * X_LD + (kk0 + k) * 16 + a_k);
-    }
-  };
-  auto mfma2 = [&](const h8 (&fa)[2][MT], const h8 (&fb)[2]) {
-#pragma unroll
-    for (int k = 0; k < 2; ++k)
-#pragma unroll
-      for (int t = 0; t < MT; ++t) grp[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[k][t], fb[k], grp[t], 0, 0, 0);
-  };
-  // Scheduling masks of sched_group_barrier: 0x008 MFMA, 0x002 VALU, 0x100 LDS read, 0x200 LDS write, 0x020 global load.
-  // First half of a step: the MFMAs of k-steps 0,1 with, between them, the operand reads of k-steps 2,3 and the
-  // unpacking of the next step into the other buffer.
-#define ART_FIRST_HALF()                                        \
-  do {                                                          \
-    __builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * MT, 0); \
-    for (int m_ = 0; m_ < 2 * MT; ++m_) {                       \
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
-      __builtin_amdgcn_sched_group_barrier(0x002, 24, 0);       \
-    }                                                           \
-    __builtin_amdgcn_sched_group_barrier(0x200, 4 + XC, 0);     \
-    __builtin_amdgcn_sched_barrier(0);                          \
-  } while (0)
-  // Second half: the MFMAs of k-steps 2,3 with the first operand reads of the next step (and the global loads) between them.
-#define ART_SECOND_HALF()                                       \
-  do {                                                          \
-    __builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * MT, 0); \
-    for (int m_ = 0; m_ < 2 * MT; ++m_) {                       \
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
-      __builtin_amdgcn_sched_group_barrier(0x020, 3, 0);        \
-    }                                                           \
-    __builtin_amdgcn_sched_barrier(0);                          \
-  } while (0)
-
-  using S0 = std::integral_constant<int, 0>;
-  using S1 = std::integral_constant<int, 1>;
-  using H0 = std::integral_constant<int, 0>;
-  using H1 = std::integral_constant<int, 1>;
-  const int last = groups - 1;
-  if (groups > 0) {
-    load_group(g_begin, S0{});
-    load_group(g_begin + (groups > 1 ? 1 : 0), S1{});
-    prepare_zeros(S0{});
-    unpack(0, S0{}, H0{});
   }
-  art_lds_barrier();
-  h8 fa01[2][MT], fb01[2], fa23[2][MT], fb23[2];
-  if (groups > 0) read_frags(fa01, fb01, 0, 0);
-  // Group i (stage S): its first step sits in LDS buffer 0 and the operands of its k-steps 0,1 in registers.
-  // The body has no branches (the scheduling directives work inside one basic block): past the last group it
-  // reloads and unpacks the last group again, which nobody multiplies.
-  auto group_body = [&](int i, auto tag, auto next_tag) {
-    constexpr int S = decltype(tag)::value;
-    const float sc = my_ok ? (float)sc16[S] : 0.f;
+  // batch b (group g_begin + b) goes to stage b % NS: kLoadsPerGroup loads per wavefront
+  auto issue = [&](int b) {
+    const unsigned int st = lds0 + (unsigned int)(b % NS) * STAGE;
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
+    for (int u = 0; u < 2; ++u) load_lds_x4(wsrc[u] + (size_t)b * (GK / 2) * N, st + (wave + 8 * u) * 1024);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) grp[t][r] = 0.f;
-    // step 0 of the group (buffer 0); step 1 is unpacked into buffer 1
-    read_frags(fa23, fb23, 0, 2);
-    unpack(1, tag, H1{});
-    mfma2(fa01, fb01);
-    ART_FIRST_HALF();
-    art_lds_barrier();
-    read_frags(fa01, fb01, 1, 0);
-    load_group(g_begin + (i + 2 < groups ? i + 2 : last), tag);          // stage S is consumed: refill it
-    mfma2(fa23, fb23);
-    ART_SECOND_HALF();
-    // step 1 of the group (buffer 1); step 0 of the next group is unpacked into buffer 0
-    read_frags(fa23, fb23, 1, 2);
-    prepare_zeros(next_tag);
-    unpack(0, next_tag, H0{});
-    mfma2(fa01, fb01);
-    ART_FIRST_HALF();
-    art_lds_barrier();
-    read_frags(fa01, fb01, 0, 0);
-    mfma2(fa23, fb23);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int t = 0; t < MT; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) total[t][r] += grp[t][r] * sc;
+    for (int u = 0; u < 2; ++u) load_lds_x4(xsrc[u] + (size_t)b * GK, st + W_BYTES + (wave + 8 * u) * 1024);
+    load_lds_x1(qsrc + (size_t)b * qstep, st + W_BYTES + X_BYTES + wave * 256);
   };
-  for (int i = 0; i < groups; i += 2) {
-    group_body(i, S0{}, S1{});
-    if (i + 1 < groups) group_body(i + 1, S1{}, S0{});
-  }
-#undef ART_FIRST_HALF
-#undef ART_SECOND_HALF
 
-  // ---- epilogue: accumulator element r of tile t is row t*32 + (r/4)*8 + (lane/32)*4 + r%4, column my_col
-  if (!my_ok || groups == 0) return;
+  // ---- operand roles.  A transposing read takes 8 byte-rows x 16 columns per 16 lanes: lane s16 supplies the
+  // 8-byte piece (row s16 / 2, half s16 % 2) and receives the 8 bytes of column s16.  Lanes 16-31 of a column tile
+  // take the chunk 8 further on, so that the 32 lanes of a pass touch 16 different chunk positions.
+  const int s16 = lane & 15, hi16 = (lane >> 4) & 1, h = lane >> 5;
+  int b_off[2], colpos[2];
+#pragma unroll
+  for (int ct = 0; ct < 2; ++ct) {
+    const int chunk = cw * 2 + ct + 8 * hi16;       // this lane's 16-column chunk of column tile ct
+    b_off[ct] = (kh * 32 + h * 16 + (s16 >> 1)) * 256 + ((chunk ^ (s16 >> 1)) * 16) + (s16 & 1) * 8;
+    colpos[ct] = chunk * 16 + s16;                  // the column (within the tile) this lane accumulates
+  }
+  int a_off[4];                                     // x chunk kh * 8 + h * 4 + e of row lane % 32 (+ 32 per accumulator tile)
+#pragma unroll
+  for (int e = 0; e < 4; ++e) a_off[e] = W_BYTES + (lane & 31) * 256 + (((kh * 8 + h * 4 + e) ^ s16) * 16);
+
+  f16v acc[MT][2];
 #pragma unroll
   for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = t * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-      if (row < M) {
-        if (splits == 1) {
-          _Float16 o = (_Float16)total[t][r];
-          if (residual) o = (_Float16)((float)o + (float)residual[(size_t)row * N + my_col]);      // may alias y: same element
-          y[(size_t)row * N + my_col] = o;
-        }
-        else partial[((size_t)split * M_total + m0 + row) * N + my_col] = total[t][r];
-      }
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[t][c][r] = 0.f;
+
+  for (int b = 0; b < NS - 1; ++b)
+    if (b < groups) issue(b);
+#pragma unroll 1
+  for (int i = 0; i < groups; ++i) {
+    // loads return in order: batch i is complete when at most the batches issued after it are outstanding
+    const int later = groups - 1 - i;
+    if (later >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerGroup) : "memory");
+    else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerGroup) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();                   // batch i is in LDS for everybody; everybody has left stage (i - 1) % NS
+    asm volatile("" ::: "memory");
+    if (i + NS - 1 < groups) issue(i + NS - 1);     // ... which the batch three groups ahead overwrites
+    const unsigned char* st = smem + (size_t)(i % NS) * STAGE;
+    h2 s2[2], zlo[2], zhi[2];                       // scale, zero point on the two nibble biases, of this lane's two columns
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+      const _Float16 sc = *reinterpret_cast<const _Float16*>(st + W_BYTES + X_BYTES + colpos[ct] * 2);
+      const unsigned int zb = st[W_BYTES + X_BYTES + 512 + (colpos[ct] >> 1)];
+      const _Float16 s = (n0 + colpos[ct] < N) ? sc : (_Float16)0.f;
+      s2[ct] = h2{s, s};
+      const unsigned int z = (zb >> ((colpos[ct] & 1) * 4)) & 15u;
+      const unsigned int zz = z | (z << 16);
+      zlo[ct] = as_h2(zz | mg.bias_lo);             // 1024 + z
+      zhi[ct] = as_h2((zz << 4) | mg.bias_hi);      // 64 + z
     }
+    // every LDS operand of the group goes to registers first: 4 transposing reads (q x column tile), 4 MT reads of x
+    i32x2 pk[2][2];
+    u32x4 ax[4][MT];
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct) pk[q][ct] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(st + b_off[ct] + q * 2048));
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) ax[e][t] = *reinterpret_cast<const u32x4*>(st + a_off[e] + t * 32 * 256);
+    // round e = (q, dword of the 8 bytes): 16 values of k for each lane half; its operands are built while the
+    // MFMAs of round e - 1 run
+    h8 fa[2][MT], fb[2][2];
+    auto build = [&](int e, int slot) {
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct) {
+        const unsigned int w = (unsigned int)pk[e >> 1][ct][e & 1], w8 = w >> 8;
+        const h2 p0 = (as_h2(and_or(w, mg.mask_lo, mg.bias_lo)) - zlo[ct]) * s2[ct];      // k0 k4
+        const h2 p1 = (as_h2(and_or(w, mg.mask_hi, mg.bias_hi)) - zhi[ct]) * s2[ct];      // k1 k5
+        const h2 p2 = (as_h2(and_or(w8, mg.mask_lo, mg.bias_lo)) - zlo[ct]) * s2[ct];     // k2 k6
+        const h2 p3 = (as_h2(and_or(w8, mg.mask_hi, mg.bias_hi)) - zhi[ct]) * s2[ct];     // k3 k7
+        fb[slot][ct] = h8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) fa[slot][t] = permute_k(ax[e][t]);
+    };
+    auto multiply = [&](int slot) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+          acc[t][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[slot][t], fb[slot][ct], acc[t][ct], 0, 0, 0);
+    };
+    build(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 3; ++e) {
+      multiply(e & 1);
+      build(e + 1, (e + 1) & 1);
+      // one MFMA (mask 0x008), then a share of the vector work (mask 0x002) of the next round: 26 + 4 MT instructions
+#pragma unroll
+      for (int m = 0; m < 2 * MT; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (26 + 4 * MT + 2 * MT - 1) / (2 * MT), 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    multiply(1);
+  }
+
+  // ---- the two k halves meet in LDS as [k half][row][column]; then every thread owns four neighbouring columns.
+  // Accumulator element r of tile t is row t*32 + (r/4)*8 + (lane/32)*4 + r%4.
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = t * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
+        red[((size_t)kh * BM + row) * RLD + colpos[ct]] = acc[t][ct][r];
+      }
+  __syncthreads();
+  if (groups == 0) return;
+#pragma unroll 1
+  for (int e = tid; e < MT * 32 * (BN / 4); e += kThreads) {
+    const int row = e >> 6, c4 = (e & 63) * 4;
+    if (row >= M || n0 + c4 >= N) continue;         // N % 4 == 0: four columns are inside or outside as a whole
+    const f32x4 v = *reinterpret_cast<const f32x4*>(red + (size_t)row * RLD + c4) +
+                    *reinterpret_cast<const f32x4*>(red + ((size_t)BM + row) * RLD + c4);
+    if (splits == 1) {
+      h4 o = h4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+      if (residual) {                               // y = fp16(fp16(product) + residual); may alias y: same elements
+        const h4 res = *reinterpret_cast<const h4*>(residual + (size_t)row * N + n0 + c4);
+        o = h4{(_Float16)((float)o[0] + (float)res[0]), (_Float16)((float)o[1] + (float)res[1]),
+               (_Float16)((float)o[2] + (float)res[2]), (_Float16)((float)o[3] + (float)res[3])};
+      }
+      *reinterpret_cast<h4*>(y + (size_t)row * N + n0 + c4) = o;
+    } else {
+      *reinterpret_cast<f32x4*>(partial + ((size_t)split * M_total + m0 + row) * N + n0 + c4) = v;
+    }
+  }
 }
 
 // y[m,n] = fp16(sum over splits, in split order); four columns per thread (N % 4 == 0).
@@ -354,8 +343,8 @@ extern "C" int art_gemm_w4a16_residual(const void* x_dev, const void* qweight_de
   ART_REQUIRE(M >= 1, "art_gemm_w4a16: M must be positive (got %d)", M);
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemm_w4a16: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0 && ((uintptr_t)qzeros_dev % 8) == 0 &&
-                  ((uintptr_t)y_dev % 8) == 0,
-              "art_gemm_w4a16: x and qweight must be 16-byte aligned, qzeros and y 8-byte aligned");
+                  ((uintptr_t)y_dev % 8) == 0 && ((uintptr_t)scales_dev % 4) == 0,
+              "art_gemm_w4a16: x and qweight must be 16-byte aligned, qzeros and y 8-byte aligned, scales 4-byte aligned");
   art::Workspace* wsp = art::workspace((hipStream_t)stream);
   if (!wsp) return 1;
   art::Workspace& ws = *wsp;

@@ -172,7 +172,9 @@ def test_w4a16_gemm_matches_oracle(autort, M, K, N):
     m = M - 1
     y1 = f(args[0][m:m + 1].contiguous(), *args[1:])
     assert np.allclose(y1.cpu().numpy().astype(np.float32), want[m:m + 1].astype(np.float32), **FP16_TOL)
-    assert np.allclose(y1.float().cpu().numpy(), y[m:m + 1].float().cpu().numpy(), rtol=2e-3, atol=2e-3)
+    # (the GEMM rounds s * (q - z) to fp16 as the oracle does, the GEMV applies s in fp32: both are inside the oracle
+    # tolerance, and within half of it of each other)
+    assert np.allclose(y1.float().cpu().numpy(), y[m:m + 1].float().cpu().numpy(), rtol=5e-3, atol=5e-3)
 
 
 @pytest.mark.parametrize('M,K,N', [(4, 512, 256), (5, 1024, 144), (6, 4096, 512), (7, 384, 1040), (8, 4096, 4096)])
