@@ -232,6 +232,14 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
 #pragma unroll
     for (int i = 0; i < R / 4; ++i) xv[m][i] = xp[i];
   }
+  // fused RMSNorm: the norm weights of this lane's slice of x go out ahead of the weight stream too - loads return in
+  // order, so behind it they would hold the first multiply-accumulate back until the whole patch has arrived
+  u32x4 n0v = {0, 0, 0, 0}, n1v = {0, 0, 0, 0};
+  if constexpr (norm) {
+    const u32x4* np = reinterpret_cast<const u32x4*>(fused.norm_w + 2 * r0c);
+    n0v = np[0];
+    n1v = np[1];
+  }
   u32x4 w[R];
   {
     const unsigned char* wp = qweight + (size_t)r0c * N + n0c;
@@ -313,8 +321,6 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
     float ss_all = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
     if constexpr (W == 8) ss_all += (s_ss[4] + s_ss[5]) + (s_ss[6] + s_ss[7]);
     const float r = 1.0f / sqrtf(ss_all * fused.inv_n + fused.eps);
-    const u32x4* np = reinterpret_cast<const u32x4*>(fused.norm_w + 2 * r0c);
-    const u32x4 n0v = np[0], n1v = np[1];
     const unsigned int nw[8] = {n0v[0], n0v[1], n0v[2], n0v[3], n1v[0], n1v[1], n1v[2], n1v[3]};
     const unsigned int xw[8] = {xv[0][0][0], xv[0][0][1], xv[0][0][2], xv[0][0][3], xv[0][1][0], xv[0][1][1], xv[0][1][2], xv[0][1][3]};
     unsigned int out[8];
