@@ -232,6 +232,15 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
 #pragma unroll
     for (int i = 0; i < R / 4; ++i) xv[m][i] = xp[i];
   }
+  // fused residual add: the first wavefront finishes the tile's columns, two per lane; their residual values are
+  // fetched now, not behind the returning atomics at the very end of the block, where the round trip would be exposed.
+  // (y may be the residual itself: only the block that arrives last at a column writes it, after every block of the
+  // tile has issued its atomics, i.e. after every one of these loads has completed.)
+  half2_t res2 = {(_Float16)0, (_Float16)0};
+  if (M == 1 && fused.residual != nullptr && tid < 64) {
+    const int rc = tile * CT + 2 * tid;
+    if (rc < N) res2 = *reinterpret_cast<const half2_t*>(fused.residual + rc);
+  }
   // fused RMSNorm: the norm weights of this lane's slice of x go out ahead of the weight stream too - loads return in
   // order, so behind it they would hold the first multiply-accumulate back until the whole patch has arrived
   u32x4 n0v = {0, 0, 0, 0}, n1v = {0, 0, 0, 0};
@@ -402,10 +411,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
 #pragma unroll
     for (int m = 0; m < M; ++m) {
       half2_t o = {(_Float16)r[m][0], (_Float16)r[m][1]};
-      if (M == 1 && fused.residual != nullptr) {
-        const half2_t res = *reinterpret_cast<const half2_t*>(fused.residual + col);
-        o = half2_t{(_Float16)((float)o.x + (float)res.x), (_Float16)((float)o.y + (float)res.y)};
-      }
+      if (M == 1 && fused.residual != nullptr) o = half2_t{(_Float16)((float)o.x + (float)res2.x), (_Float16)((float)o.y + (float)res2.y)};
       *reinterpret_cast<half2_t*>(y + (size_t)m * N + col) = o;
     }
     return;
@@ -428,7 +434,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
       if (((old[m][j] + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
         const long long total = old[m][j] + mine[m][j] - ((long long)splits << 56);
         _Float16 o = (_Float16)from_fixed(total);
-        if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)fused.residual[col + j]);
+        if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)(j == 0 ? res2.x : res2.y));
         y[(size_t)m * N + col + j] = o;
         slots[(size_t)m * N + col + j] = 0ull;            // ready for the next launch (stream order makes this visible)
       }
