@@ -260,6 +260,21 @@ builtin('attention_f32')(lambda: DecodeAttention('attention_f32'))
 builtin('attention_f16')(lambda: DecodeAttention('attention_f16'))
 
 
+SUMSQ_WORDS = 256      # 64-bit words of a sum-of-squares buffer (one per 128 columns of the projection that fills it)
+
+
+def _sumsq_buffers(who, *buffers):
+    given = [b for b in buffers if b is not None]
+    for b in given:
+        if b.dtype != torch.int64 or b.numel() != SUMSQ_WORDS or not b.is_contiguous():
+            raise TypeError(f'{who}: a sum-of-squares buffer is a contiguous int64 tensor of {SUMSQ_WORDS} words')
+    return given
+
+
+def _ptr_or_null(t):
+    return c_void_p(t.data_ptr() if t is not None else 0)
+
+
 class GemvW4Fused:
     """``gemv_w4a16_fused(x[K], qweight, scales, qzeros, out[N], norm_weight=None, residual=None, eps=1e-5)``:
     the packed int4 GEMV with an RMSNorm of its input and/or a residual add of its output folded in
@@ -267,8 +282,11 @@ class GemvW4Fused:
     name = 'gemv_w4a16_fused'
 
     def __call__(self, x, qweight, scales, qzeros, out=None, norm_weight=None, residual=None, eps=RMS_EPS, swiglu=False,
-                 extra=None):
-        """``swiglu=True``: ``x`` holds gate | up (2*K values) and the product is taken with silu(gate) * up."""
+                 extra=None, sumsq_in=None, sumsq_out=None, sumsq_clear=None):
+        """``swiglu=True``: ``x`` holds gate | up (2*K values) and the product is taken with silu(gate) * up.
+        ``sumsq_*``: int64[256] buffers that hand sum(y^2) from the projection that writes a residual stream
+        (``sumsq_out``, which also zeroes ``sumsq_clear`` for the next writer) to the one that normalises it
+        (``sumsq_in`` with ``norm_weight``), see ``art_gemv_w4a16_fused_sumsq``."""
         K, N = qweight.shape[0] * 2, qweight.shape[1]
         if x.numel() != (2 * K if swiglu else K):
             raise ValueError('gemv_w4a16_fused: x has the wrong length')
@@ -284,11 +302,13 @@ class GemvW4Fused:
                 if t.dtype != torch.float16 or t.numel() != (K if what == 'norm_weight' else N):
                     raise TypeError(f'gemv_w4a16_fused: {what} must be float16 of matching length')
                 tensors.append(t)
+        tensors += _sumsq_buffers('gemv_w4a16_fused', sumsq_in, sumsq_out, sumsq_clear)
         _require_cuda(*tensors)
-        capi.check(capi.lib().art_gemv_w4a16_fused(
+        capi.check(capi.lib().art_gemv_w4a16_fused_sumsq(
             c_void_p(x.data_ptr()), c_void_p(qweight.data_ptr()), c_void_p(scales.data_ptr()), c_void_p(qzeros.data_ptr()),
             c_void_p(out.data_ptr()), K, N, c_void_p(norm_weight.data_ptr() if norm_weight is not None else 0), float(eps),
-            c_void_p(residual.data_ptr() if residual is not None else 0), int(bool(swiglu)), c_void_p(current_stream_handle())))
+            c_void_p(residual.data_ptr() if residual is not None else 0), int(bool(swiglu)), _ptr_or_null(sumsq_in),
+            _ptr_or_null(sumsq_out), _ptr_or_null(sumsq_clear), c_void_p(current_stream_handle())))
         return out
 
 
@@ -376,7 +396,7 @@ class GemvW4Attn:
     split attention's output (merged on the fly) with the residual add folded in."""
     name = 'gemv_w4a16_attn'
 
-    def __call__(self, partial, qweight, scales, qzeros, out, residual=None):
+    def __call__(self, partial, qweight, scales, qzeros, out, residual=None, sumsq_out=None, sumsq_clear=None):
         K, N = qweight.shape[0] * 2, qweight.shape[1]
         if partial.dim() != 3 or partial.shape[2] != 132 or partial.dtype != torch.float32 or partial.shape[0] * 128 != K:
             raise TypeError('gemv_w4a16_attn: partial must be float32 [K/128, parts, 132]')
@@ -384,11 +404,13 @@ class GemvW4Attn:
             raise ValueError('gemv_w4a16_attn: operand shapes do not match K, N')
         if scales.dtype != torch.float16 or out.dtype != torch.float16 or (residual is not None and residual.dtype != torch.float16):
             raise TypeError('gemv_w4a16_attn: scales, out and residual must be float16')
-        _require_cuda(*([partial, qweight, scales, qzeros, out] + ([residual] if residual is not None else [])))
-        capi.check(capi.lib().art_gemv_w4a16_attn(
+        _require_cuda(*([partial, qweight, scales, qzeros, out] + ([residual] if residual is not None else []) +
+                        _sumsq_buffers('gemv_w4a16_attn', sumsq_out, sumsq_clear)))
+        capi.check(capi.lib().art_gemv_w4a16_attn_sumsq(
             c_void_p(partial.data_ptr()), partial.shape[1], c_void_p(qweight.data_ptr()), c_void_p(scales.data_ptr()),
             c_void_p(qzeros.data_ptr()), c_void_p(out.data_ptr()), K, N,
-            c_void_p(residual.data_ptr() if residual is not None else 0), c_void_p(current_stream_handle())))
+            c_void_p(residual.data_ptr() if residual is not None else 0), _ptr_or_null(sumsq_out), _ptr_or_null(sumsq_clear),
+            c_void_p(current_stream_handle())))
         return out
 
 

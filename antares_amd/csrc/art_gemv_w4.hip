@@ -152,16 +152,45 @@ struct Fused {
   float inv_n, eps;
   const float* att_partial;   // != NULL: x is merged from the per-part records of a split decode attention (see MODE 3)
   int att_parts;
+  // sum(y^2) handed from the projection that writes a residual stream to the projection that normalises it (M = 1):
+  //   sumsq_out   != NULL : every block adds the squares of the outputs it finishes (after the residual add, as rounded
+  //                         to fp16) to word [column tile] of it, as fixed point in units of 2^-30;
+  //   sumsq_clear != NULL : its kSumsqWords words are set to zero (the buffer the NEXT projection adds into);
+  //   sumsq_in    != NULL : with norm_w, the sum of squares of x is the sum of words [0, K/128) of it, x is not re-read.
+  unsigned long long* sumsq_out;
+  unsigned long long* sumsq_clear;
+  const unsigned long long* sumsq_in;
 };
+constexpr int kSumsqWords = 256;                     // words of a sum-of-squares buffer: projections of up to 32768 columns
+constexpr float kSumsqUnit = 1073741824.f;           // 2^30
+// One square on its way into a word: exact below 2^25 (|y| < 5792), capped there above and for NaN, so that the 128
+// squares of a column tile can never wrap the word.
+__device__ __forceinline__ unsigned long long sumsq_fixed(float y) {
+  const float t = y * y;
+  return t < 33554432.f ? (unsigned long long)(t * kSumsqUnit) : (1ull << 55);
+}
+// sum over the 64 lanes of a wavefront of a value below 2^22; every lane gets the result
+__device__ __forceinline__ unsigned int wave_sum_all_u32(unsigned int v) {
+#define ART_DPP_ADD(ctrl) v += (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, ctrl, 0xf, 0xf, false)
+  ART_DPP_ADD(0xB1);    // quad_perm [1,0,3,2]
+  ART_DPP_ADD(0x4E);    // quad_perm [2,3,0,1]
+  ART_DPP_ADD(0x141);   // row_half_mirror
+  ART_DPP_ADD(0x140);   // row_mirror
+#undef ART_DPP_ADD
+  return ((unsigned int)__builtin_amdgcn_readlane((int)v, 0) + (unsigned int)__builtin_amdgcn_readlane((int)v, 16)) +
+         ((unsigned int)__builtin_amdgcn_readlane((int)v, 32) + (unsigned int)__builtin_amdgcn_readlane((int)v, 48));
+}
 
 // The register allocator is told that four wavefronts per SIMD are plenty (a launch has three): with the default
 // target of eight it postpones two of the eight weight loads until registers free up, a second memory round trip.
-template <int M, int MODE, int R, int W>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused, 3: x = merged split attention
+template <int M, int MODE, int R, int W>   // MODE 0: plain product, 1: RMSNorm of x fused, 2: x = SwiGLU(gate | up) fused, 3: x = merged split attention,
+                                           // 4: RMSNorm of x fused, its sum of squares handed in (sumsq_in)
 __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_w4a16_kernel(
     const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight, const _Float16* __restrict__ scales,
     const unsigned char* __restrict__ qzeros, _Float16* __restrict__ y, int K, int N, int splits,
     unsigned long long* __restrict__ slots, Magic magic, Fused fused) {
   static_assert(R == 8 || (R == 4 && MODE == 0), "the fused prologues are written for 8 rows per lane");
+  static_assert(MODE != 4 || W == 4, "the handed-in sum of squares comes with four wavefronts");
   static_assert(W == 4 || W == 8, "four or eight wavefronts per block");
   constexpr int kThreads = 64 * W, KL = kThreads / CL;  // k lanes per block: 32 or 64
   constexpr int kRowsPerBlock = KL * R;                 // packed rows per block: 256 (512 values of k) at R = 8, W = 4
@@ -184,10 +213,16 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
   // ---- fused RMSNorm, part 1: the loads for the sum of squares go out BEFORE the weight loads.  Loads
   // return in order, so these can be consumed (and the block-wide reduction done) while the weights are
   // still in flight; issued after the weights they would wait for the whole stream.
-  constexpr bool norm = (M == 1) && (MODE == 1);
+  constexpr bool norm = (M == 1) && (MODE == 1 || MODE == 4);      // x is normalised
+  constexpr bool norm_own = (M == 1) && (MODE == 1);                // ... with a sum of squares computed here
   constexpr int kSq = 512 / kThreads;                     // 16-byte chunks of x per thread that cover K = 4096
   u32x4 sq[kSq];
-  if constexpr (norm) {
+  unsigned long long ss_word = 0;
+  if constexpr (MODE == 4) {                              // one word per lane: K / 128 <= 64
+    if (lane < (K >> 7)) ss_word = fused.sumsq_in[lane];
+  }
+  if (M == 1 && fused.sumsq_clear != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && tid < kSumsqWords) fused.sumsq_clear[tid] = 0ull;
+  if constexpr (norm_own) {
 #pragma unroll
     for (int i = 0; i < kSq; ++i) {
       const int c = tid + i * kThreads;
@@ -303,6 +338,11 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
   // ---- fused RMSNorm, part 2 (while the weight loads are in flight): sum of squares over all of x.
   // Every block recomputes it from the 2*K bytes of x (served by L2) rather than waiting for another kernel.
   if constexpr (norm) {
+    float ss_all;
+    if constexpr (MODE == 4) {
+      // words below 2^62 each: split at 2^32 so that both parts convert exactly enough (24 bits each) and sum in a fixed order
+      ss_all = wave_sum_all((float)(unsigned int)(ss_word >> 32) * 4294967296.f + (float)(unsigned int)ss_word) * (1.f / kSumsqUnit);
+    } else {
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < kSq; ++i) {
@@ -327,8 +367,9 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
     ss = wave_sum_all(ss);
     if (lane == 0) s_ss[wave] = ss;
     art_lds_barrier();      // LDS only: the weight loads issued above stay in flight
-    float ss_all = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
+    ss_all = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
     if constexpr (W == 8) ss_all += (s_ss[4] + s_ss[5]) + (s_ss[6] + s_ss[7]);
+    }
     const float r = 1.0f / sqrtf(ss_all * fused.inv_n + fused.eps);
     const unsigned int nw[8] = {n0v[0], n0v[1], n0v[2], n0v[3], n1v[0], n1v[1], n1v[2], n1v[3]};
     const unsigned int xw[8] = {xv[0][0][0], xv[0][0][1], xv[0][0][2], xv[0][0][3], xv[0][1][0], xv[0][1][1], xv[0][1][2], xv[0][1][3]};
@@ -391,7 +432,9 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
   __syncthreads();
   if (tid >= 64) return;
   const int c2 = 2 * tid, col = tile * CT + c2;           // the first wavefront finishes two columns per lane
-  if (col >= N) return;
+  const bool hand_on = (M == 1) && fused.sumsq_out != nullptr;      // the whole wavefront stays for the sum of squares
+  if (col >= N && !hand_on) return;
+  unsigned long long sq_mine = 0;                         // squares of the outputs this lane has finished
 
   float r[M][2];
 #pragma unroll
@@ -407,38 +450,52 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
       r[m][1] += (p4[1] + p5[1]) + (p6[1] + p7[1]);
     }
   }
-  if (splits == 1) {
+  if (col < N) {
+    if (splits == 1) {
 #pragma unroll
-    for (int m = 0; m < M; ++m) {
-      half2_t o = {(_Float16)r[m][0], (_Float16)r[m][1]};
-      if (M == 1 && fused.residual != nullptr) o = half2_t{(_Float16)((float)o.x + (float)res2.x), (_Float16)((float)o.y + (float)res2.y)};
-      *reinterpret_cast<half2_t*>(y + (size_t)m * N + col) = o;
-    }
-    return;
-  }
-  // returning atomics, one per (row, column): [arrival count : 8][fixed-point sum : 56].  All of them go out before
-  // the first result is looked at, so the lane pays one round trip.
-  long long mine[M][2], old[M][2];
-#pragma unroll
-  for (int m = 0; m < M; ++m)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      mine[m][j] = (1LL << 56) + to_fixed(r[m][j], splits);
-      old[m][j] = (long long)__hip_atomic_fetch_add(slots + (size_t)m * N + col + j, (unsigned long long)mine[m][j], __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
-    }
-#pragma unroll
-  for (int m = 0; m < M; ++m)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      if (((old[m][j] + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
-        const long long total = old[m][j] + mine[m][j] - ((long long)splits << 56);
-        _Float16 o = (_Float16)from_fixed(total);
-        if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)(j == 0 ? res2.x : res2.y));
-        y[(size_t)m * N + col + j] = o;
-        slots[(size_t)m * N + col + j] = 0ull;            // ready for the next launch (stream order makes this visible)
+      for (int m = 0; m < M; ++m) {
+        half2_t o = {(_Float16)r[m][0], (_Float16)r[m][1]};
+        if (M == 1 && fused.residual != nullptr) o = half2_t{(_Float16)((float)o.x + (float)res2.x), (_Float16)((float)o.y + (float)res2.y)};
+        *reinterpret_cast<half2_t*>(y + (size_t)m * N + col) = o;
+        if (hand_on) sq_mine = sumsq_fixed((float)o.x) + sumsq_fixed((float)o.y);
       }
+    } else {
+      // returning atomics, one per (row, column): [arrival count : 8][fixed-point sum : 56].  All of them go out
+      // before the first result is looked at, so the lane pays one round trip.
+      long long mine[M][2], old[M][2];
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          mine[m][j] = (1LL << 56) + to_fixed(r[m][j], splits);
+          old[m][j] = (long long)__hip_atomic_fetch_add(slots + (size_t)m * N + col + j, (unsigned long long)mine[m][j], __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if (((old[m][j] + (1LL << 55)) >> 56) == (long long)(splits - 1)) {
+            const long long total = old[m][j] + mine[m][j] - ((long long)splits << 56);
+            _Float16 o = (_Float16)from_fixed(total);
+            if (M == 1 && fused.residual != nullptr) o = (_Float16)((float)o + (float)(j == 0 ? res2.x : res2.y));
+            y[(size_t)m * N + col + j] = o;
+            slots[(size_t)m * N + col + j] = 0ull;            // ready for the next launch (stream order makes this visible)
+            if (hand_on) sq_mine += sumsq_fixed((float)o);
+          }
+        }
     }
+  }
+  if (hand_on) {
+    // Which block finishes a column depends on timing, the sum of the integers does not.  Three 21-bit limbs, each
+    // summed over the wavefront (two squares per lane: below 2^28), one atomic per block that finished anything.
+    const unsigned int l0 = wave_sum_all_u32((unsigned int)sq_mine & 0x1fffffu);
+    const unsigned int l1 = wave_sum_all_u32((unsigned int)(sq_mine >> 21) & 0x1fffffu);
+    const unsigned int l2 = wave_sum_all_u32((unsigned int)(sq_mine >> 42));
+    const unsigned long long total = (unsigned long long)l0 + ((unsigned long long)l1 << 21) + ((unsigned long long)l2 << 42);
+    if (tid == 0 && total != 0ull)
+      __hip_atomic_fetch_add(fused.sumsq_out + tile, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 // Split-K accumulators of the entry point that allocates nothing (art_gemv_w4a16_noalloc): 64-bit slots, one per
@@ -451,7 +508,7 @@ unsigned long long* g_scratch_ptr[kMaxDevices];          // device address of `s
 
 template <int M>
 int launch(const void* x, const void* qw, const void* sc, const void* qz, void* y, int K, int N, hipStream_t stream,
-           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0}, unsigned long long* slots = nullptr,
+           Fused fused = Fused{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0, nullptr, nullptr, nullptr}, unsigned long long* slots = nullptr,
            int rows_per_lane = 8, int waves = 0) {
   const int rows = K / 2;
   const int tiles = (N + CT - 1) / CT;
@@ -481,7 +538,8 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
       else if (fused.att_partial != nullptr) ART_GEMV_LAUNCH(3, 8, 8);
       else ART_GEMV_LAUNCH(0, 8, 8);
     } else {
-      if (fused.norm_w != nullptr) ART_GEMV_LAUNCH(1, 8, 4);
+      if (fused.norm_w != nullptr && fused.sumsq_in != nullptr) ART_GEMV_LAUNCH(4, 8, 4);
+      else if (fused.norm_w != nullptr) ART_GEMV_LAUNCH(1, 8, 4);
       else if (fused.gate_up != nullptr) ART_GEMV_LAUNCH(2, 8, 4);
       else if (fused.att_partial != nullptr) ART_GEMV_LAUNCH(3, 8, 4);
       else if (rows_per_lane == 4) ART_GEMV_LAUNCH(0, 4, 4);
@@ -524,7 +582,7 @@ extern "C" int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, 
     const int step = (M - m >= 4) ? 4 : (M - m);
     const _Float16* xs = (const _Float16*)x_dev + (size_t)m * K;
     _Float16* ys = (_Float16*)y_dev + (size_t)m * N;
-    const Fused none{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0};
+    const Fused none{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0, nullptr, nullptr, nullptr};
     int rc = step == 4 ? launch<4>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl, 4)
            : step == 3 ? launch<3>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl, 4)
            : step == 2 ? launch<2>(xs, qweight_dev, scales_dev, qzeros_dev, ys, K, N, st, none, nullptr, rpl, 4)
@@ -561,7 +619,7 @@ extern "C" int art_gemv_w4a16_noalloc(const void* x_dev, const void* qweight_dev
   ART_HIP(hipGetDevice(&dev));
   ART_REQUIRE(dev >= 0 && dev < kMaxDevices && g_scratch_ptr[dev] != nullptr, "art_gemv_w4a16_noalloc: call art_init(%d) first", dev);
   unsigned long long* slots = g_scratch_ptr[dev];
-  const Fused none{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0};
+  const Fused none{nullptr, nullptr, nullptr, 0.f, 0.f, nullptr, 0, nullptr, nullptr, nullptr};
   hipStream_t st = (hipStream_t)stream;
   return M == 4 ? launch<4>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, st, none, slots)
        : M == 3 ? launch<3>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, st, none, slots)
@@ -572,6 +630,28 @@ extern "C" int art_gemv_w4a16_noalloc(const void* x_dev, const void* qweight_dev
 extern "C" int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                                     void* y_dev, int K, int N, const void* norm_weight_dev, float eps, const void* residual_dev,
                                     int swiglu_input, void* stream) {
+  return art_gemv_w4a16_fused_sumsq(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, norm_weight_dev, eps, residual_dev,
+                                    swiglu_input, nullptr, nullptr, nullptr, stream);
+}
+
+namespace {
+// the checks the two entry points with sum-of-squares buffers share
+int check_sumsq(const char* who, const void* in, const void* out, const void* clear, int K, int N, const void* norm_w) {
+  ART_REQUIRE(((uintptr_t)in % 8) == 0 && ((uintptr_t)out % 8) == 0 && ((uintptr_t)clear % 8) == 0,
+              "%s: the sum-of-squares buffers must be 8-byte aligned", who);
+  ART_REQUIRE(in == nullptr || (norm_w != nullptr && K <= 64 * 128),
+              "%s: a handed-in sum of squares needs a norm weight and K <= 8192 (K=%d)", who, K);
+  ART_REQUIRE(out == nullptr || N <= kSumsqWords * CT, "%s: a sum-of-squares buffer covers %d columns (N=%d)", who, kSumsqWords * CT, N);
+  ART_REQUIRE(out == nullptr || out != clear, "%s: the buffer that is cleared cannot be the one that is added to", who);
+  ART_REQUIRE(in == nullptr || (in != clear && in != out), "%s: the buffer that is read cannot be cleared or added to by the same call", who);
+  return 0;
+}
+}  // namespace
+
+extern "C" int art_gemv_w4a16_fused_sumsq(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                                          void* y_dev, int K, int N, const void* norm_weight_dev, float eps,
+                                          const void* residual_dev, int swiglu_input, const void* sumsq_in_dev,
+                                          void* sumsq_out_dev, void* sumsq_clear_dev, void* stream) {
   ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16_fused: null pointer");
   ART_REQUIRE(!(swiglu_input && norm_weight_dev), "art_gemv_w4a16_fused: SwiGLU input and RMSNorm cannot be combined");
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_fused: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
@@ -582,13 +662,22 @@ extern "C" int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, 
   // blocks of one column tile write y while blocks of other tiles still read x: only the residual may alias y
   ART_REQUIRE(!art::overlaps(x_dev, (size_t)(swiglu_input ? 2 : 1) * K * 2, y_dev, (size_t)N * 2),
               "art_gemv_w4a16_fused: y must not overlap x (it may alias the residual)");
+  if (check_sumsq("art_gemv_w4a16_fused_sumsq", sumsq_in_dev, sumsq_out_dev, sumsq_clear_dev, K, N, norm_weight_dev)) return 1;
   Fused f{(const _Float16*)norm_weight_dev, (const _Float16*)residual_dev, swiglu_input ? (const _Float16*)x_dev : nullptr,
-          1.0f / (float)K, eps, nullptr, 0};
+          1.0f / (float)K, eps, nullptr, 0, (unsigned long long*)sumsq_out_dev, (unsigned long long*)sumsq_clear_dev,
+          (const unsigned long long*)sumsq_in_dev};
   return launch<1>(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, (hipStream_t)stream, f);
 }
 
 extern "C" int art_gemv_w4a16_attn(const void* partial_dev, int parts, const void* qweight_dev, const void* scales_dev,
                                    const void* qzeros_dev, void* y_dev, int K, int N, const void* residual_dev, void* stream) {
+  return art_gemv_w4a16_attn_sumsq(partial_dev, parts, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, residual_dev, nullptr, nullptr,
+                                   stream);
+}
+
+extern "C" int art_gemv_w4a16_attn_sumsq(const void* partial_dev, int parts, const void* qweight_dev, const void* scales_dev,
+                                         const void* qzeros_dev, void* y_dev, int K, int N, const void* residual_dev,
+                                         void* sumsq_out_dev, void* sumsq_clear_dev, void* stream) {
   ART_REQUIRE(partial_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16_attn: null pointer");
   ART_REQUIRE(parts >= 2 && parts <= art::kMaxAttnParts, "art_gemv_w4a16_attn: parts must be in 2..%d (got %d)", art::kMaxAttnParts, parts);
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16_attn: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
@@ -598,6 +687,8 @@ extern "C" int art_gemv_w4a16_attn(const void* partial_dev, int parts, const voi
               "art_gemv_w4a16_attn: y, scales and the residual must be 4-byte aligned");
   ART_REQUIRE(!art::overlaps(partial_dev, (size_t)(K / 128) * parts * 132 * 4, y_dev, (size_t)N * 2),
               "art_gemv_w4a16_attn: y must not overlap the partial records");
-  Fused f{nullptr, (const _Float16*)residual_dev, nullptr, 0.f, 0.f, (const float*)partial_dev, parts};
+  if (check_sumsq("art_gemv_w4a16_attn_sumsq", nullptr, sumsq_out_dev, sumsq_clear_dev, K, N, nullptr)) return 1;
+  Fused f{nullptr, (const _Float16*)residual_dev, nullptr, 0.f, 0.f, (const float*)partial_dev, parts,
+          (unsigned long long*)sumsq_out_dev, (unsigned long long*)sumsq_clear_dev, nullptr};
   return launch<1>(partial_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, K, N, (hipStream_t)stream, f);
 }

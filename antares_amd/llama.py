@@ -109,6 +109,9 @@ class LlamaInt4Decoder:
         inv = (1.0 / (cfg.rope_base ** (torch.arange(0, D, 2).float() / D))).to(torch.float16)
         self.inv_freq = torch.cat([inv, inv]).view(D).to(self.dev)
         self.att_f = torch.tensor([1 / math.sqrt(D)], dtype=torch.float32, device=self.dev)
+        # sum(x^2) of the residual stream, handed from the projection that writes it to the one that normalises it
+        self.hand_sumsq = fused and d <= 8192
+        self.sumsq = torch.zeros(2, 256, dtype=torch.int64, device=self.dev)
         # device-side step state
         self.token = torch.zeros(1, dtype=torch.int32, device=self.dev)
         self.pos = torch.zeros(1, dtype=torch.int32, device=self.dev)
@@ -156,21 +159,32 @@ class LlamaInt4Decoder:
         gemv = ops.gemv_w4a16_fused
         if embed:
             self.embed(self.w['embed'], self.token, out=self.x)
+        # The projections that write the residual stream (o, down) leave sum(x^2) of what they wrote in a buffer, and the
+        # projection that normalises the stream next reads it there instead of re-reading x in every block.  Two
+        # buffers alternate: a writer adds into one and zeroes the other for the writer after it.  Only the first
+        # projection of a step computes its own sum (its x is an embedding row).
+        after_o, after_down = self.sumsq if self.hand_sumsq else (None, None)
         for l, lw in enumerate(self.w['layers']):
             a, o, gu, dn = lw['qkv'], lw['o'], lw['gate_up'], lw['down']
-            gemv(self.x, a['qweight'], a['scales'], a['qzeros'], self.qkv, norm_weight=lw['att_norm'], eps=cfg.rms_eps)
+            gemv(self.x, a['qweight'], a['scales'], a['qzeros'], self.qkv, norm_weight=lw['att_norm'], eps=cfg.rms_eps,
+                 sumsq_in=after_down if l > 0 else None)
             if self.att_parts > 1:      # attention over several blocks per head, merged by the o-projection as it loads x
                 ops.attention_rope_split_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f,
                                              self.att_partial, extra=[self.pos])
-                ops.gemv_w4a16_attn(self.att_partial, o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
+                ops.gemv_w4a16_attn(self.att_partial, o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x,
+                                    sumsq_out=after_o, sumsq_clear=after_down)
             else:
                 ops.attention_rope_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f, self.att,
                                        extra=[self.pos])
-                gemv(self.att.view(-1), o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
-            gemv(self.x, gu['qweight'], gu['scales'], gu['qzeros'], self.gu, norm_weight=lw['ffn_norm'], eps=cfg.rms_eps)
-            gemv(self.gu, dn['qweight'], dn['scales'], dn['qzeros'], self.x, residual=self.x, swiglu=True)
+                gemv(self.att.view(-1), o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x,
+                     sumsq_out=after_o, sumsq_clear=after_down)
+            gemv(self.x, gu['qweight'], gu['scales'], gu['qzeros'], self.gu, norm_weight=lw['ffn_norm'], eps=cfg.rms_eps,
+                 sumsq_in=after_o)
+            gemv(self.gu, dn['qweight'], dn['scales'], dn['qzeros'], self.x, residual=self.x, swiglu=True,
+                 sumsq_out=after_down, sumsq_clear=after_o)
         h = self.w['lm_head']
-        gemv(self.x, h['qweight'], h['scales'], h['qzeros'], self.logits, norm_weight=self.w['final_norm'], eps=cfg.rms_eps)
+        gemv(self.x, h['qweight'], h['scales'], h['qzeros'], self.logits, norm_weight=self.w['final_norm'], eps=cfg.rms_eps,
+             sumsq_in=after_down)
         return self.logits
 
     def step_plain(self) -> torch.Tensor:

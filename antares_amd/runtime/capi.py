@@ -60,6 +60,8 @@ _SIGNATURES = {
     'art_gemv_w4a16_noalloc': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_decode_attention_rope_split': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p]),
     'art_gemv_w4a16_attn': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
+    'art_gemv_w4a16_attn_sumsq': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p,
+                                          c_void_p, c_void_p]),
     'art_rope_qkv_store_rows': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     'art_prefill_attention': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_longlong, c_void_p]),
     'art_greedy_next': (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
@@ -68,6 +70,8 @@ _SIGNATURES = {
     'art_partition_even_first_i32': (c_int, [c_void_p, c_void_p, c_longlong, c_void_p]),
     'art_gemv_w4a16_fused': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p,
                                      c_int, c_void_p]),
+    'art_gemv_w4a16_fused_sumsq': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_float,
+                                           c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     'art_decode_attention_rope': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]),
     'art_rope_qkv_store': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_gemm_f16': (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),

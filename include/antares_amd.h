@@ -184,6 +184,22 @@ int art_gemv_w4a16_fused(const void* x_dev, const void* qweight_dev, const void*
                          void* y_dev, int K, int N, const void* norm_weight_dev, float eps, const void* residual_dev,
                          int swiglu_input, void* stream);
 
+/* art_gemv_w4a16_fused with the sum of squares of a residual stream handed from the projection that writes the
+ * stream to the projection that normalises it, so that the RMSNorm of lines :128-131 of the sample does not re-read
+ * its input in every block.  A sum-of-squares buffer is 256 64-bit words of device memory, zero before its first use:
+ *   sumsq_out_dev   != NULL: word [n / 128] receives, added up over the call, the squares of the y[n] written (as
+ *                            rounded to fp16, after the residual add) in units of 2^-30; a square of 2^25 or more
+ *                            (|y| >= 5793) or of a NaN counts as 2^25.  Integer sums: independent of timing.
+ *   sumsq_clear_dev != NULL: that buffer is set to zero (the one the NEXT writer of a stream adds into).
+ *   sumsq_in_dev    != NULL: needs norm_weight_dev and K <= 8192; sum(x^2) is taken as the sum of words
+ *                            [0, K/128) of it instead of being computed from x.
+ * The three must be different buffers.  With all three NULL this is art_gemv_w4a16_fused.  No counterpart in the
+ * reference, which normalises in a separate operator. */
+int art_gemv_w4a16_fused_sumsq(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                               void* y_dev, int K, int N, const void* norm_weight_dev, float eps, const void* residual_dev,
+                               int swiglu_input, const void* sumsq_in_dev, void* sumsq_out_dev, void* sumsq_clear_dev,
+                               void* stream);
+
 /* The reference's own weight format (samples/05_llama2_7b_int4.py:135-139):
  * qweight int32 [K/8,N], eight nibbles per word along K (least significant
  * first), zero point fixed at 8, scales fp32 or fp16 [K/128,N], x and y fp32
@@ -269,6 +285,11 @@ int art_decode_attention_rope_split(const void* qkv_dev, const void* inv_freq_de
  * art_decode_attention_rope_split with the same `parts` (2..8), K = heads * 128. */
 int art_gemv_w4a16_attn(const void* partial_dev, int parts, const void* qweight_dev, const void* scales_dev,
                         const void* qzeros_dev, void* y_dev, int K, int N, const void* residual_dev, void* stream);
+/* art_gemv_w4a16_attn that also adds the squares of its outputs to sumsq_out_dev and clears sumsq_clear_dev (see
+ * art_gemv_w4a16_fused_sumsq; either may be NULL). */
+int art_gemv_w4a16_attn_sumsq(const void* partial_dev, int parts, const void* qweight_dev, const void* scales_dev,
+                              const void* qzeros_dev, void* y_dev, int K, int N, const void* residual_dev,
+                              void* sumsq_out_dev, void* sumsq_clear_dev, void* stream);
 int art_decode_attention(const void* q_dev, const void* k_dev, const void* v_dev, const void* att_f_dev, void* out_dev,
                          int seq_len, int heads, int head_dim, const void* pos_dev, int q_dtype, int kv_dtype, int out_dtype,
                          void* stream);

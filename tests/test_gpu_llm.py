@@ -351,3 +351,100 @@ def test_rope_qkv_store_rows_against_the_oracle():
     # positions that do not fit the caches are refused on the host
     with pytest.raises(Exception, match='do not fit'):
         autort.ops.rope_qkv_store_rows_f16(qkv.to(dev), inv_freq.to(dev), q_out, kd, vd, extra=[S - T + 1])
+
+
+def _tile_sums_of_squares(y: torch.Tensor) -> np.ndarray:
+    """What a projection leaves in its sum-of-squares buffer for the fp16 outputs y: per tile of 128 columns the sum of
+    floor(y^2 * 2^30), each square capped at 2^25 (integer arithmetic)."""
+    sq = y.double().cpu().numpy() ** 2
+    fixed = np.where(sq < 2.0 ** 25, np.floor(sq * 2.0 ** 30), 2.0 ** 55).astype(np.uint64)
+    pad = (-fixed.size) % 128
+    return np.concatenate([fixed, np.zeros(pad, dtype=np.uint64)]).reshape(-1, 128).sum(axis=1)
+
+
+@pytest.mark.parametrize('K,N,scale', [(1024, 512, 1.0), (4096, 4096, 1.0), (11008, 4096, 0.02), (512, 272, 300.0)])
+def test_sum_of_squares_handed_from_one_projection_to_the_next(autort, K, N, scale):
+    """The projection that writes a residual stream (with residual add, plain or SwiGLU input) leaves sum(y^2) per
+    column tile as exact integers and zeroes the other buffer; the projection that normalises the stream and takes the
+    sum from the buffer agrees with the one that computes it from x, and with the oracle."""
+    from oracle import hot_ops
+    from antares_amd import workloads
+    dev = autort.device()
+    note(f'sum of squares K={K} N={N} scale={scale}')
+    g = gen(K + N)
+    p = workloads.w4_problem(K + 3 * N, 1, K, N)
+    qw, sc, qz = (p[k].to(dev) for k in ('qweight', 'scales', 'qzeros'))
+    x = (torch.randn(K, generator=g) * scale).half().to(dev)
+    res = (torch.randn(N, generator=g) * scale).half().to(dev)
+    a = torch.zeros(256, dtype=torch.int64, device=dev)
+    b = torch.full((256,), 12345, dtype=torch.int64, device=dev)
+    y = autort.ops.gemv_w4a16_fused(x, qw, sc, qz, residual=res, sumsq_out=a, sumsq_clear=b)
+    y_plain = autort.ops.gemv_w4a16_fused(x, qw, sc, qz, residual=res)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_plain)
+    assert int(b.abs().max()) == 0
+    want = _tile_sums_of_squares(y)
+    got = a.cpu().numpy().astype(np.uint64)
+    assert np.array_equal(got[:want.size], want) and not got[want.size:].any()
+    # a second writer adds on top (the decoder clears in between)
+    autort.ops.gemv_w4a16_fused(x, qw, sc, qz, residual=res, sumsq_out=a)
+    torch.cuda.synchronize()
+    assert np.array_equal(a.cpu().numpy().astype(np.uint64)[:want.size], 2 * want)
+    a.zero_()
+    a[:want.size] = torch.from_numpy(want.astype(np.int64)).to(dev)
+    # the consumer: y is the stream (N must be a K of its own: a multiple of 128 here except in the ragged case)
+    if N % 128:
+        return
+    p2 = workloads.w4_problem(N + 5, 1, N, 528)
+    qw2, sc2, qz2 = (p2[k].to(dev) for k in ('qweight', 'scales', 'qzeros'))
+    nw = (torch.rand(N, generator=g) + 0.5).half().to(dev)
+    handed = autort.ops.gemv_w4a16_fused(y, qw2, sc2, qz2, norm_weight=nw, eps=1e-5, sumsq_in=a)
+    own = autort.ops.gemv_w4a16_fused(y, qw2, sc2, qz2, norm_weight=nw, eps=1e-5)
+    torch.cuda.synchronize()
+    assert torch.allclose(handed.float(), own.float(), rtol=2e-3, atol=2e-3)
+    xn = hot_ops.rmsnorm(y.cpu().numpy(), None, nw.cpu().numpy(), 1.0 / N, 1e-5, np.float16)
+    ref = hot_ops.gemm_w4a16(xn.reshape(1, -1), p2['qweight'].numpy(), p2['scales'].numpy(), p2['qzeros'].numpy())
+    assert np.allclose(handed.cpu().numpy().astype(np.float32).reshape(1, -1), ref.astype(np.float32), **FP16_TOL)
+
+
+def test_sum_of_squares_through_the_attention_merge(autort):
+    """gemv_w4a16_attn leaves the same sums as the fused projection on the merged attention output."""
+    from antares_amd import workloads
+    dev = autort.device()
+    H, D, S, parts, pos = 32, 128, 384, 8, 200
+    g = gen(77)
+    qkv = torch.randn(3 * H * D, generator=g).half().to(dev)
+    inv = (1.0 / (10000 ** (torch.arange(0, D, 2).float() / D))).half()
+    inv_freq = torch.cat([inv, inv]).to(dev)
+    kc = (torch.randn(S, H * D, generator=g) * 0.5).half().to(dev)
+    vc = torch.randn(S, H * D, generator=g).half().to(dev)
+    att_f = torch.tensor([1 / math.sqrt(D)], dtype=torch.float32, device=dev)
+    pos_t = torch.tensor([pos], dtype=torch.int32, device=dev)
+    p = workloads.w4_problem(9, 1, H * D, 4096)
+    qw, sc, qz = (p[k].to(dev) for k in ('qweight', 'scales', 'qzeros'))
+    res = torch.randn(4096, generator=g).half().to(dev)
+    partial = torch.full((H, parts, 132), float('nan'), dtype=torch.float32, device=dev)
+    autort.ops.attention_rope_split_f16(qkv, inv_freq, kc, vc, att_f, partial, extra=[pos_t])
+    a = torch.zeros(256, dtype=torch.int64, device=dev)
+    b = torch.ones(256, dtype=torch.int64, device=dev)
+    y = torch.empty(4096, dtype=torch.float16, device=dev)
+    autort.ops.gemv_w4a16_attn(partial, qw, sc, qz, y, residual=res, sumsq_out=a, sumsq_clear=b)
+    torch.cuda.synchronize()
+    want = _tile_sums_of_squares(y)
+    assert np.array_equal(a.cpu().numpy().astype(np.uint64)[:32], want) and int(b.abs().max()) == 0
+
+
+def test_sum_of_squares_buffers_are_checked(autort):
+    from antares_amd.runtime import capi
+    from antares_amd import workloads
+    dev = autort.device()
+    p = workloads.w4_problem(3, 1, 256, 256)
+    qw, sc, qz = (p[k].to(dev) for k in ('qweight', 'scales', 'qzeros'))
+    x = torch.randn(256).half().to(dev)
+    a = torch.zeros(256, dtype=torch.int64, device=dev)
+    with pytest.raises(capi.ArtError, match='norm weight'):
+        autort.ops.gemv_w4a16_fused(x, qw, sc, qz, sumsq_in=a)
+    with pytest.raises(capi.ArtError, match='cannot be the one'):
+        autort.ops.gemv_w4a16_fused(x, qw, sc, qz, sumsq_out=a, sumsq_clear=a)
+    with pytest.raises(TypeError, match='sum-of-squares buffer'):
+        autort.ops.gemv_w4a16_fused(x, qw, sc, qz, sumsq_out=torch.zeros(8, dtype=torch.int64, device=dev))
