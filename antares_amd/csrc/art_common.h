@@ -40,10 +40,10 @@ inline bool overlaps(const void* a, size_t an, const void* b, size_t bn) {
   return a0 < b0 + bn && b0 < a0 + an;
 }
 
-// Workspace layout.  Ticket words must read zero whenever no kernel is running,
+// Workspace layout.  The exchange words and the accumulators keep their meaning between launches,
 // so they never share bytes with scratch data.
-constexpr size_t kGemvTicketOffset = 0;                 // 16384 ticket words of the split-K kernels
-constexpr size_t kGemvTicketBytes = 64 * 1024;
+constexpr size_t kExchangeOffset = 0;                    // launch tag + one word per block of the phase-chain probe (tagged, never zeroed again)
+constexpr size_t kExchangeBytes = 64 * 1024;
 constexpr size_t kSlotOffset = 64 * 1024;                // 64-bit split-K accumulators (zero between launches)
 constexpr size_t kScratchOffset = 4 * 1024 * 1024;       // partial sums, tile counts (any content)
 

@@ -323,6 +323,124 @@ extern "C" int art_read_bytes(const void* src_dev, size_t bytes, void* sink_dev,
   return 0;
 }
 
+// ------------------------------------------------------------ store-only kernel
+// The counterpart of the read-only launch for writes: every thread stores 16-byte vectors of a constant with
+// non-temporal stores, nothing is read.  What it takes is the floor of a launch that has to write these bytes.
+__global__ __launch_bounds__(256) void art_fill_kernel(u32x4* __restrict__ dst, size_t nvec, unsigned int value) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  const u32x4 v = {value, value, value, value};
+  for (; i < nvec; i += stride) __builtin_nontemporal_store(v, &dst[i]);
+}
+
+extern "C" int art_fill_bytes(void* dst_dev, size_t bytes, unsigned int value, void* stream) {
+  ART_REQUIRE(dst_dev && ((uintptr_t)dst_dev % 16) == 0 && bytes % 16 == 0, "art_fill_bytes: pointer and size must be multiples of 16");
+  const size_t nvec = bytes / 16;
+  if (nvec == 0) return 0;
+  size_t blocks = (nvec + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  art_fill_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>((u32x4*)dst_dev, nvec, value);
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ phases inside one launch
+// What a grid-wide barrier inside a kernel costs on this part, and whether a persistent kernel can keep the weight
+// stream going across it: 256 resident blocks run `phases` phases; in a phase every block fetches its share of
+// `phase_bytes` with the read-only launch's pattern (three 32 KiB units per block at most) and then all blocks meet.
+// The meeting uses no atomics and no fences: a block's thirteenth wavefront stores (phase, launch tag) into the
+// block's own word with an agent-scope store and polls everybody's words with agent-scope loads, a bounded number
+// of times; the twelve worker wavefronts wait at an LDS-only barrier, so loads they have in flight stay in flight.
+//   mode 0: no loads at all (the barrier by itself);  mode 1: a phase's loads are issued after the previous barrier;
+//   mode 2: the NEXT phase's loads are issued before the barrier (what a persistent decode kernel would do).
+constexpr int kChainBlocks = 256, kChainWorkers = 768, kChainThreads = 832, kChainSpinLimit = 1 << 18;
+
+__global__ __launch_bounds__(kChainThreads) void art_phase_chain_kernel(const unsigned char* __restrict__ src, size_t phase_bytes,
+                                                                        int phases, size_t pitch, int tiles, int mode,
+                                                                        unsigned long long* __restrict__ exchange,
+                                                                        unsigned int* __restrict__ sink,
+                                                                        unsigned int* __restrict__ status) {
+  __shared__ int s_ok;
+  __shared__ unsigned long long s_tag;
+  const int tid = threadIdx.x, lane = tid & 63, q = tid >> 8, t = tid & 255, cl = t & 7, kl = t >> 3;
+  const bool control = tid >= kChainWorkers;
+  unsigned long long* launches = exchange;
+  unsigned long long* words = exchange + 8;
+  if (tid == kChainWorkers) s_tag = __hip_atomic_load(launches, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+  const int units = (int)(phase_bytes / 32768);
+  const int unit = (int)blockIdx.x + kChainBlocks * q;
+  const bool has = !control && unit < units;
+  const int tile = unit % tiles, split = unit / tiles;
+  const size_t off = has ? ((size_t)split * 256 + (size_t)kl * 8) * pitch + (size_t)tile * 128 + cl * 16 : 0;
+  __syncthreads();
+  const unsigned long long tag = s_tag;
+  unsigned int acc = 0;
+  u32x4 w[8];
+  if (mode == 2 && has) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + off + (size_t)i * pitch));
+  }
+  for (int ph = 0; ph < phases; ++ph) {
+    if (mode == 1 && has) {
+      const unsigned char* p = src + (size_t)ph * phase_bytes + off;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)i * pitch));
+    }
+    if (mode != 0 && has) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc ^= w[i][0] ^ w[i][1] ^ w[i][2] ^ w[i][3];
+    }
+    if (mode == 2 && has && ph + 1 < phases) {
+      const unsigned char* p = src + (size_t)(ph + 1) * phase_bytes + off;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)i * pitch));
+    }
+    // ---- all blocks meet
+    art_lds_barrier();                       // every wavefront of the block has finished the phase
+    if (control) {
+      const unsigned long long want = (tag << 16) | (unsigned long long)(ph + 1);
+      if (lane == 0) __hip_atomic_store(words + blockIdx.x, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      bool done = false;
+      for (int spin = 0; spin < kChainSpinLimit && !done; ++spin) {
+        bool ok = true;
+#pragma unroll
+        for (int k = 0; k < kChainBlocks / 64; ++k)
+          ok = ok && __hip_atomic_load(words + lane + 64 * k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= want;
+        done = __all(ok);
+      }
+      if (lane == 0) {
+        s_ok = done ? 1 : 0;
+        if (!done) __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    art_lds_barrier();
+    if (!s_ok) break;                        // a block that gave up stops meeting; the others give up in turn and exit
+  }
+  if (blockIdx.x == 0 && tid == kChainWorkers)   // the next launch on this workspace gets a new tag
+    __hip_atomic_store(launches, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (acc == 0x9E3779B9u) sink[blockIdx.x] = acc;
+}
+
+extern "C" int art_phase_chain_probe(const void* src_dev, size_t src_bytes, size_t phase_bytes, int phases, int mode, void* sink_dev,
+                                     void* status_dev, void* stream) {
+  ART_REQUIRE(src_dev && sink_dev && status_dev && ((uintptr_t)src_dev % 16) == 0, "art_phase_chain_probe: null or misaligned pointer");
+  ART_REQUIRE(mode >= 0 && mode <= 2 && phases >= 1 && phases <= 65535, "art_phase_chain_probe: mode 0..2, 1..65535 phases");
+  ART_REQUIRE(phase_bytes > 0 && phase_bytes % 32768 == 0 && phase_bytes / 32768 <= 3 * (size_t)kChainBlocks,
+              "art_phase_chain_probe: a phase is a multiple of 32768 bytes, at most %d", 3 * kChainBlocks * 32768);
+  ART_REQUIRE((size_t)phases * phase_bytes <= src_bytes, "art_phase_chain_probe: %d phases of %zu bytes do not fit the %zu bytes of src", phases,
+              phase_bytes, src_bytes);
+  ART_REQUIRE(art::compute_units() >= kChainBlocks, "art_phase_chain_probe: needs %d compute units (all blocks must be resident)", kChainBlocks);
+  art::Workspace* wsp = art::workspace((hipStream_t)stream);
+  if (!wsp) return 1;
+  const size_t pitch = (phase_bytes % (11008u * 256u) == 0) ? 11008 : 128;
+  art_phase_chain_kernel<<<dim3(kChainBlocks), dim3(kChainThreads), 0, (hipStream_t)stream>>>(
+      (const unsigned char*)src_dev, phase_bytes, phases, pitch, (int)(pitch / 128), mode,
+      reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(wsp->base) + art::kExchangeOffset), (unsigned int*)sink_dev,
+      (unsigned int*)status_dev);
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---- device memory for callers that own no allocator (the reference's evaluator; the torch plugin uses torch's)
 extern "C" int art_alloc(size_t bytes, void** out_dev) {
   ART_REQUIRE(out_dev != nullptr, "art_alloc: null output");

@@ -52,6 +52,8 @@ _SIGNATURES = {
     'art_memcpy_dtoh': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     'art_memcpy_dtod': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     'art_read_bytes': (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
+    'art_fill_bytes': (c_int, [c_void_p, c_size_t, c_uint, c_void_p]),
+    'art_phase_chain_probe': (c_int, [c_void_p, c_size_t, c_size_t, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     'art_gemv_w4a16': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     'art_gemv_w4a16_tuned': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     'art_gemm_w4a16_tuned': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),

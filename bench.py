@@ -4,6 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra] [--no-decode]
     python bench.py --calibrate-copy MIB LAUNCHES     # plain copy of known size, for scaling memory-traffic counters
     python bench.py --read-floor                      # only the read-only launch over the headline's weight bytes
+    python bench.py --stream-floors                   # read-only, store-only and copy launches over 22.5 / 67 MB
+    python bench.py --phase-chain                     # phases that meet inside ONE launch against dependent launches
 
 Headline workload (BASELINE.json: "int4-GEMV HBM GB/s"): the int4 group-128
 GEMV y[1,11008] = x[1,4096] @ dequant(W), through ``autort.export`` and the
@@ -66,6 +68,10 @@ def parse_args():
                     help='run only the plain copy kernel on MIB MiB, LAUNCHES times (counter calibration), and exit')
     ap.add_argument('--read-floor', action='store_true',
                     help='run only the read-only launch over 32 distinct buffers of the headline weight size, and exit')
+    ap.add_argument('--stream-floors', action='store_true',
+                    help='run only the read-only, store-only and copy launches (what one launch needs to move bytes), and exit')
+    ap.add_argument('--phase-chain', action='store_true',
+                    help='run only the probe of phases meeting inside one launch (a persistent kernel against dependent launches), and exit')
     return ap.parse_args()
 
 
@@ -109,6 +115,75 @@ def bench_read_floor(torch, capi, steps, warmup, nbytes=2048 * 11008, layers=LAY
     return {'kernel': 'art_read_kernel', 'bytes_per_launch': nbytes, 'us_per_launch': round(sec * 1e6, 3),
             'gbps': round(nbytes / sec / 1e9, 1), 'frac_of_peak': round(nbytes / sec / 1e9 / HBM_PEAK_GBPS, 4),
             'us_per_launch_of_one_block': round(tiny * 1e6, 3)}
+
+
+def bench_stream_floors(torch, capi, steps, warmup, layers=16):
+    """What one dependent launch needs to read, to write, and to read and write bytes with nothing else to do:
+    `art_read_bytes`, `art_fill_bytes` and `art_copy_bytes` over `layers` distinct buffers in one HIP graph."""
+    from ctypes import c_void_p
+    lib = capi.lib()
+    out = []
+    sink = torch.zeros(4096, dtype=torch.int32, device='cuda')
+    for nbytes in (2048 * 11008, 6144 * 11008):
+        bufs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device='cuda') for _ in range(layers)]
+        dsts = [torch.empty_like(b) for b in bufs]
+
+        def reads():
+            st = torch.cuda.current_stream().cuda_stream
+            for b in bufs:
+                capi.check(lib.art_read_bytes(c_void_p(b.data_ptr()), nbytes, c_void_p(sink.data_ptr()), c_void_p(st)))
+
+        def fills():
+            st = torch.cuda.current_stream().cuda_stream
+            for d in dsts:
+                capi.check(lib.art_fill_bytes(c_void_p(d.data_ptr()), nbytes, 7, c_void_p(st)))
+
+        def copies():
+            st = torch.cuda.current_stream().cuda_stream
+            for b, d in zip(bufs, dsts):
+                capi.check(lib.art_copy_bytes(c_void_p(d.data_ptr()), c_void_p(b.data_ptr()), nbytes, c_void_p(st)))
+        row = {'bytes': nbytes}
+        for name, fn, moved in (('read_only', reads, nbytes), ('store_only', fills, nbytes), ('copy', copies, 2 * nbytes)):
+            sec = time_graph(torch, capi, fn, steps, warmup) / layers
+            row[name] = {'us_per_launch': round(sec * 1e6, 3), 'gbps_moved': round(moved / sec / 1e9, 1)}
+        assert bool((dsts[0] == bufs[0]).all())
+        out.append(row)
+        del bufs, dsts
+    return out
+
+
+def bench_phase_chain(torch, capi, phases=32, nbytes=2048 * 11008, runs=5):
+    """`phases` phases of `nbytes` each inside ONE launch, all blocks meeting after every phase
+    (`art_phase_chain_probe`), against the same reads as `phases` dependent launches."""
+    from ctypes import c_void_p
+    lib = capi.lib()
+    src = torch.randint(0, 256, (phases * nbytes,), dtype=torch.uint8, device='cuda')
+    sink = torch.zeros(4096, dtype=torch.int32, device='cuda')
+    status = torch.zeros(1, dtype=torch.int32, device='cuda')
+    stream = side_stream(torch)
+    out = {'phases': phases, 'bytes_per_phase': nbytes}
+    with torch.cuda.stream(stream):
+        for mode, name in ((0, 'meeting_only'), (1, 'loads_after_the_meeting'), (2, 'next_loads_before_the_meeting')):
+            best = None
+            for _ in range(runs + 1):
+                start, stop = capi.Event(), capi.Event()
+                start.record(stream.cuda_stream)
+                capi.check(lib.art_phase_chain_probe(c_void_p(src.data_ptr()), src.numel(), nbytes, phases, mode, c_void_p(sink.data_ptr()),
+                                                     c_void_p(status.data_ptr()), c_void_p(stream.cuda_stream)))
+                stop.record(stream.cuda_stream)
+                us = start.elapsed_ms(stop) * 1e3 / phases
+                best = us if best is None else min(best, us)
+            stream.synchronize()
+            if int(status.item()) != 0:
+                raise RuntimeError('art_phase_chain_probe: a block gave up waiting (the chip was not free)')
+            out[name + '_us_per_phase'] = round(best, 3)
+
+    def launches():
+        st = torch.cuda.current_stream().cuda_stream
+        for i in range(phases):
+            capi.check(lib.art_read_bytes(c_void_p(src.data_ptr() + i * nbytes), nbytes, c_void_p(sink.data_ptr()), c_void_p(st)))
+    out['dependent_launches_us_per_phase'] = round(time_graph(torch, capi, launches, 20, 3) / phases * 1e6, 3)
+    return out
 
 
 _SIDE_STREAM = None
@@ -383,6 +458,12 @@ def main():
         return
     if args.read_floor:
         print(json.dumps(bench_read_floor(torch, capi, args.steps, args.warmup)), flush=True)
+        return
+    if args.stream_floors:
+        print(json.dumps(bench_stream_floors(torch, capi, args.steps, args.warmup)), flush=True)
+        return
+    if args.phase_chain:
+        print(json.dumps(bench_phase_chain(torch, capi)), flush=True)
         return
     K, N, M = 4096, 11008, 1
     head = bench_gemv(torch, autort, capi, workloads, K, N, M, args.steps, args.warmup, args.seed)

@@ -120,6 +120,21 @@ int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* strea
  * written in practice). */
 int art_read_bytes(const void* src_dev, size_t bytes, void* sink_dev, void* stream);
 
+/* Store-only counterpart: one launch that writes `bytes` (a multiple of 16, 16-byte aligned) of the 32-bit `value`
+ * with non-temporal 16-byte stores and reads nothing: the floor of a launch that has to write these bytes. */
+int art_fill_bytes(void* dst_dev, size_t bytes, unsigned int value, void* stream);
+
+/* Measurement only, no counterpart in the reference: what a grid-wide meeting inside ONE launch costs on this part,
+ * i.e. what a persistent whole-token kernel would pay instead of a dependent launch.  256 resident blocks run `phases`
+ * phases over src_dev (phases * phase_bytes bytes, at most src_bytes; phase_bytes a multiple of 32768, at most
+ * 24 MiB); in every phase a block fetches its share with the access pattern of art_read_bytes, then all blocks meet
+ * through one word per block in the stream's workspace (agent-scope stores and loads, no atomics, no fences, every
+ * wait bounded).  mode 0: no loads; 1: a phase's loads follow the previous meeting; 2: the next phase's loads are
+ * issued before the meeting.  status_dev: one 32-bit word, zero before the call, 1 afterwards if a block gave up
+ * waiting (the chip was not free to hold all 256 blocks).  sink_dev: 256 words of scratch. */
+int art_phase_chain_probe(const void* src_dev, size_t src_bytes, size_t phase_bytes, int phases, int mode, void* sink_dev,
+                          void* status_dev, void* stream);
+
 /* ---------------------------------------------------- hand-written kernels */
 
 /* Weight-only int4 GEMV / skinny GEMM, group size 128 along K:

@@ -93,3 +93,36 @@ def test_device_copies_and_the_read_only_launch():
     torch.cuda.synchronize()
     assert torch.equal(buf, before) and int(sink.abs().sum()) == 0
     assert l.art_read_bytes(c_void_p(buf.data_ptr()), 1000, c_void_p(sink.data_ptr()), None) != 0
+
+
+@pytest.mark.gpu
+def test_store_only_launch_and_phases_meeting_inside_one_launch():
+    """art_fill_bytes writes the constant and nothing else; art_phase_chain_probe runs its phases to the end in every
+    mode (no block gives up waiting on a free chip), twice in a row on one workspace, and rejects sizes it cannot take."""
+    import torch
+    from ctypes import c_void_p
+    from antares_amd.runtime import capi
+    capi.init(0)
+    l = capi.lib()
+    buf = torch.zeros(1 << 20, dtype=torch.int32, device='cuda')
+    capi.check(l.art_fill_bytes(c_void_p(buf.data_ptr()), (1 << 20) * 4 - 64, 0x01020304, None))
+    torch.cuda.synchronize()
+    assert bool((buf[:-16] == 0x01020304).all()) and int(buf[-16:].abs().sum()) == 0
+    assert l.art_fill_bytes(c_void_p(buf.data_ptr()), 24, 1, None) != 0
+    phases, nbytes = 6, 32768 * 40
+    src = torch.randint(0, 256, (phases * nbytes,), dtype=torch.uint8, device='cuda')
+    before = src.clone()
+    sink = torch.zeros(4096, dtype=torch.int32, device='cuda')
+    status = torch.zeros(1, dtype=torch.int32, device='cuda')
+    for rep in range(2):
+        for mode in (0, 1, 2):
+            print(f'[case] phase chain mode {mode} rep {rep}', flush=True)
+            capi.check(l.art_phase_chain_probe(c_void_p(src.data_ptr()), src.numel(), nbytes, phases, mode, c_void_p(sink.data_ptr()),
+                                               c_void_p(status.data_ptr()), None))
+            torch.cuda.synchronize()
+            assert int(status.item()) == 0
+    assert torch.equal(src, before) and int(sink.abs().sum()) == 0
+    assert l.art_phase_chain_probe(c_void_p(src.data_ptr()), src.numel(), nbytes, phases + 1, 1, c_void_p(sink.data_ptr()),
+                                   c_void_p(status.data_ptr()), None) != 0
+    assert l.art_phase_chain_probe(c_void_p(src.data_ptr()), src.numel(), 1000, 1, 1, c_void_p(sink.data_ptr()),
+                                   c_void_p(status.data_ptr()), None) != 0
