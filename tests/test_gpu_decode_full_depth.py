@@ -69,3 +69,46 @@ def test_32_layer_decode_matches_the_oracle():
         if top2[1] - top2[0] > 0.15 * spread:
             assert int(dec.token.item()) == int(np.argmax(want))
         token = int(dec.token.item())          # both sides continue with the device's choice
+
+
+@pytest.mark.timeout(300)
+def test_full_width_prefill_matches_the_oracle_token_by_token():
+    """Whole-prompt ingestion at the benchmark model's widths (dim 4096, 32 heads, ffn 11008, vocab 32000; two layers so
+    that the oracle's token-by-token pass stays short): the int4 GEMMs at their real shapes with 12 rows, the causal
+    attention with 32 heads, rotary and cache writes of all rows - logits of the last position and every cache row
+    against the oracle, which takes the prompt one token at a time."""
+    from antares_amd.autort import patterns
+    from antares_amd.ir import parse_program
+    from antares_amd.llama import LlamaConfig, LlamaInt4Decoder, random_weights
+    from oracle.cpu_backend import CpuModule
+    from oracle.llama_ref import LlamaRef
+    cfg = LlamaConfig(n_layers=2)
+    T = 12
+    w = random_weights(cfg, seed=21)
+    mod = CpuModule(parse_program(patterns.W4A16_IR, patterns.W4A16_INPUTS), nranks=256, fast_math=False)
+
+    def linear(x, lin):
+        return mod(x=np.ascontiguousarray(x), qweight=lin['qweight'].numpy().view('int8'), scales=lin['scales'].numpy(),
+                   qzeros=lin['qzeros'].numpy().view('int8'))['y']
+    ref = LlamaRef(cfg, w, linear=linear)
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, cfg.vocab, (T,), generator=g, dtype=torch.int32)
+    t0 = time.time()
+    for pos in range(T):
+        want = ref.forward(int(prompt[pos]), pos).astype(np.float32)
+    print(f'[case] full-width prefill T={T}: oracle took {time.time() - t0:.1f} s', flush=True)
+    dec = LlamaInt4Decoder(cfg, w, fused=True, att_parts=8)
+    got = dec.prefill(prompt.to(dec.dev)).float().cpu().numpy()
+    spread = float(want.std())
+    err = float(np.abs(got - want).max())
+    print(f'[case] full-width prefill: spread {spread:.3f}, max |diff| {err:.4f}', flush=True)
+    # as in the full-width decode test: a logit is a sum of 4096 products of spread about 5, reached by the operators'
+    # fp16 roundings scaled by that spread
+    assert 2.0 < spread < 10.0 and np.allclose(got, want, rtol=2e-2, atol=2e-2 * spread), (err, spread)
+    assert int(dec.pos.item()) == T - 1
+    for l in range(cfg.n_layers):
+        for got_c, want_c in ((dec.key_cache[l, :T], ref.key_cache[l, :T]), (dec.val_cache[l, :T], ref.val_cache[l, :T])):
+            want_c = want_c.astype(np.float32)
+            assert np.allclose(got_c.float().cpu().numpy(), want_c, rtol=2e-2, atol=2e-2 * max(1.0, float(want_c.std()))), \
+                (l, np.abs(got_c.float().cpu().numpy() - want_c).max(), float(want_c.std()))
+    assert not dec.key_cache[:, T:].any() and not dec.val_cache[:, T:].any()
