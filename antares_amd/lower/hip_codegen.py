@@ -7,8 +7,10 @@ templates:
 
 * elementwise / gather statements: one flat grid-stride loop; when every tensor
   is read and written at the same flat position the kernel moves 16-byte
-  vectors per lane (the reference's untuned default is one scalar element per
-  block, antares/common.py:81-100);
+  vectors per lane, and so it does when every load is a run along the last
+  axis or constant along it (bias rows, gathered rows: `table[ids[N], C]`)
+  (the reference's untuned default is one scalar element per block,
+  antares/common.py:81-100);
 * reduce statements: three variants compiled together — one wavefront per
   output (DPP / readlane reduction), one 256-thread block per output, one
   thread per output — and the launcher picks by extents and by which axis is
@@ -132,6 +134,9 @@ class KernelPlan:
     reduce_axes: List[Tuple[str, object]]
     vec: int = 1                   # elements per lane in the vector variant
     vec_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for it
+    row_vec: int = 1               # elements per lane in the row-vector variant (vectors along the last data axis)
+    row_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for it
+    row_dims: List[object] = field(default_factory=list)    # extents (int or dimension name) that must be multiples of row_vec
     reduce_contiguous: Optional[bool] = None   # True: a reduce axis is fastest in the biggest operand
     tile_axes: Optional[Tuple[str, str]] = None   # permutation copies: last axis of the load, last axis of the store
 
@@ -150,6 +155,16 @@ class KernelPlan:
                 n *= v
         return n
 
+    def _row_vectors(self, env: Dict[str, int], pointers: Dict[str, int], total: int) -> int:
+        """Vectors of the row-vector variant for these extents and addresses, 0 when it does not apply."""
+        if 'rowvec' not in self.variants or total < self.row_vec:
+            return 0
+        if any(pointers[t] % 16 for t in self.row_tensors):
+            return 0
+        if any((d if isinstance(d, int) else env[d]) % self.row_vec for d in self.row_dims):
+            return 0
+        return total // self.row_vec
+
     def choose(self, env: Dict[str, int], pointers: Dict[str, int]) -> Tuple[str, int, int]:
         """-> (kernel symbol, grid.x, block.x) for these extents and addresses."""
         total = 1
@@ -164,6 +179,9 @@ class KernelPlan:
             if 'vec' in self.variants and all(pointers[t] % 16 == 0 for t in self.vec_tensors) and total >= self.vec:
                 work = (total + self.vec - 1) // self.vec
                 return self.variants['vec'], min((work + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
+            rows = self._row_vectors(env, pointers, total)
+            if rows:
+                return self.variants['rowvec'], min((rows + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
             tiles = self._tiles(env)
             if tiles:
                 return self.variants['tile'], min(tiles, MAX_GRID), BLOCK
@@ -193,6 +211,8 @@ class KernelPlan:
         if self.kind == 'map':
             if 'vec' in self.variants and all(pointers[t] % 16 == 0 for t in self.vec_tensors) and total >= self.vec:
                 tags.append(('vec', (total + self.vec - 1) // self.vec))
+            if self._row_vectors(env, pointers, total):
+                tags.append(('rowvec', self._row_vectors(env, pointers, total)))
             if self._tiles(env):
                 tags.append(('tile', self._tiles(env) * BLOCK))
             tags.append(('scalar', total))
@@ -263,6 +283,35 @@ def _transpose_axes(st, tensors):
         return None
     a_ax, b_ax = idx[-1].name, axes[-1]
     return None if a_ax == b_ax else (a_ax, b_ax)
+
+
+def _row_vector_loads(st, tensors):
+    """Loads that walk memory along the statement's last data axis L, for a statement that stores densely along L:
+    every load either does not mention L at all (one value for the whole vector) or has the bare axis L as its last
+    index and L nowhere else (a contiguous run: bias rows, gathered rows, `table[ids[N], C]`).  Returns (L, those
+    loads) or None when the statement is not of that shape."""
+    axes = [a for a, _ in st.data_axes]
+    exts = [e for _, e in st.data_axes]
+    if not axes or st.scatter or st.reduce_axes or [i.name for i in st.out_index if i.kind == 'axis'] != axes:
+        return None
+    if len(st.out_index) != len(axes) or list(tensors[st.output].shape) != exts:
+        return None
+    if st.root.kind == 'when' and len(st.root.args) == 1:
+        return None
+    L = axes[-1]
+    runs = []
+    for n in walk(st.root):
+        if n.kind != 'load':
+            continue
+        if n.name == st.output:
+            return None
+        uses = [any(m.kind == 'axis' and m.name == L for m in walk(a)) for a in n.args]
+        if not any(uses):
+            continue
+        if any(uses[:-1]) or n.args[-1].kind != 'axis':
+            return None
+        runs.append(n)
+    return (L, runs) if runs else None
 
 
 def _is_flat_map(st, tensors) -> bool:
@@ -379,6 +428,50 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
                 src.append('\n'.join(body))
                 variants['vec'] = sym
                 plan.vec, plan.vec_tensors = V, names
+        rv = _row_vector_loads(st, tensors) if 'vec' not in variants and cond is None else None
+        if rv is not None:
+            L, runs = rv
+            names = sorted({n.name for n in runs} | {st.output})
+            V = max(1, 16 // max(ITEMSIZE[tensors[n].dtype] for n in names))
+            if V > 1:
+                sym = name + '_r'
+                body = header(sym)
+                for n in names:
+                    body.append(f'  typedef {HIP_TYPE[tensors[n].dtype]} __vec_{n} __attribute__((ext_vector_type({V})));')
+                body.append(f'  const long long __lv = __ext_{L} / {V};')
+                body.append(f'  const long long __nvec = __total / {V};')
+                body.append('  for (long long __v = __tid; __v < __nvec; __v += __nthr) {')
+                body.append('    long long __r = __v;')
+                body.append(f'    const int __l0 = (int)(__r % __lv) * {V}; __r /= __lv;')
+                for ax, _ in reversed(st.data_axes[:-1]):
+                    body.append(f'    const int {ax} = (int)(__r % __ext_{ax}); __r /= __ext_{ax};')
+                def streamed(n):
+                    return sum(1 for s_ in graph.statements if n in s_.reads or n == s_.output) == 1
+                for k, n in enumerate(runs):
+                    off = plain.offset(n.name, [plain.expr(a) for a in n.args[:-1]] + ['__l0'])
+                    ref = f'*(const __vec_{n.name}*)&{n.name}[{off}]'
+                    once = one_touch(n) is not None
+                    body.append(f'    const __vec_{n.name} __run_{k} = ' + (f'__builtin_nontemporal_load(&({ref}));' if once else f'{ref};'))
+                def run_lane(n):
+                    for k, m in enumerate(runs):
+                        if m is n:
+                            return f'__run_{k}[__e]'
+                    return None
+                rem = ExprEmitter(tensors, load_override=run_lane)
+                body.append(f'    __vec_{st.output} __out;')
+                body.append('    #pragma unroll')
+                body.append(f'    for (int __e = 0; __e < {V}; ++__e) {{')
+                body.append(f'      const int {L} = __l0 + __e; (void){L};')
+                body.append(f'      __out[__e] = ({oct_})({rem.expr(root)});')
+                body.append('    }')
+                dst_ = f'((__vec_{st.output}*){st.output})[__v]'
+                body.append(f'    __builtin_nontemporal_store(__out, &{dst_});' if streamed(st.output) else f'    {dst_} = __out;')
+                body += ['  }', '}']
+                src.append('\n'.join(body))
+                variants['rowvec'] = sym
+                plan.row_vec = V
+                plan.row_tensors = names
+                plan.row_dims = [st.data_axes[-1][1]] + [tensors[n.name].shape[-1] for n in runs]
         tr = _transpose_axes(st, tensors)
         if tr is not None:
             a_ax, b_ax = tr

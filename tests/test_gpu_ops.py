@@ -485,3 +485,61 @@ def test_w4a16_gemm_with_the_residual_folded_in(autort, M, K, N):
     plain = torch.empty_like(acc)
     autort.ops.gemm_w4a16_residual(*d, plain)
     assert np.allclose(plain.float().cpu().numpy(), prod.astype(np.float32), **FP16_TOL)
+
+
+ROW_VECTOR_CASES = [
+    # program, inputs, shapes of the inputs, does the row-vector variant apply to these extents
+    ('output0[N, C] = input0[N, C] + input1[C]', ['input0=float32[N:300, C:1024]', 'input1=float32[C:1024]'], [(300, 1024), (1024,)], True),
+    ('output0[N, C] = input0[input1[N], C]', ['input0=float32[V:500, C:256]', 'input1=int32[N:1000]'], [(500, 256), (1000,)], True),
+    ('emb[T, D] = table[tok[T], D]', ['table=float16[V:320, D:4096]', 'tok=int32[T:37]'], [(320, 4096), (37,)], True),
+    ('output0[B, N, C] = (input0[B, N, C].to(`float32`) * input1[B, C] + input2[N]).to(`float16`)',
+     ['input0=float16[B:3, N:50, C:72]', 'input1=float32[B:3, C:72]', 'input2=float32[N:50]'], [(3, 50, 72), (3, 72), (50,)], True),
+    ('output0[N, C] = input0[N, C] * C + input1[N]', ['input0=int32[N:33, C:64]', 'input1=int32[N:33]'], [(33, 64), (33,)], True),
+    # a last extent that is no multiple of the vector: the scalar kernel runs
+    ('output0[N, C] = input0[N, C] + input1[C]', ['input0=float32[N:30, C:1023]', 'input1=float32[C:1023]'], [(30, 1023), (1023,)], False),
+]
+
+
+@pytest.mark.parametrize('ir,inputs,shapes,applies', ROW_VECTOR_CASES)
+def test_row_vector_maps_match_the_oracle(autort, ir, inputs, shapes, applies):
+    """Maps whose loads are runs along the last axis or constant along it (bias rows, gathered rows) move 16-byte
+    vectors per lane; results are the oracle's, and the scalar kernel takes over where the extents do not fit."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'row-vector map {ir} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='rowvec_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    plan = op.plans[0]
+    assert 'rowvec' in plan.variants and 'vec' not in plan.variants
+    g = torch.Generator().manual_seed(len(ir))
+    tensors, names = [], []
+    for spec, shape in zip(inputs, shapes):
+        name, rest = spec.split('=')
+        names.append(name)
+        if rest.startswith('int32'):
+            hi = 320 if 'tok' in name else (500 if name == 'input1' and 'input0[input1' in ir else 1000)
+            tensors.append(torch.randint(0, hi, shape, generator=g, dtype=torch.int32))
+        else:
+            tensors.append(torch.randn(shape, generator=g).to(torch.float16 if rest.startswith('float16') else torch.float32))
+    env = {}
+    for spec, shape in zip(inputs, shapes):
+        dims = spec.split('[', 1)[1].rstrip(']').split(',')
+        for d, v in zip(dims, shape):
+            env[d.split(':')[0].strip()] = v
+    ptrs = {n: 0 for n in plan.args}
+    assert (plan.choose(env, ptrs)[0] == plan.variants['rowvec']) == applies
+    got = op(*[t.to(dev) for t in tensors]).cpu().numpy()
+    out_name = ir.split('[', 1)[0].strip()
+    want = CpuModule(parse_program(ir, inputs), fast_math=False)(**{n: t.numpy() for n, t in zip(names, tensors)})[out_name]
+    if got.dtype.kind == 'i':
+        assert np.array_equal(got, want)
+    else:
+        assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=1e-2 if got.dtype == np.float16 else 1e-5,
+                           atol=1e-2 if got.dtype == np.float16 else 1e-5)
+    # an operand that is not 16-byte aligned falls back to the scalar kernel, same result
+    if applies and tensors[0].dtype != torch.int32:
+        base = torch.empty(tensors[0].numel() + 1, dtype=tensors[0].dtype, device=dev)
+        view = base[1:].view(tensors[0].shape)
+        view.copy_(tensors[0])
+        got2 = op(view, *[t.to(dev) for t in tensors[1:]]).cpu().numpy()
+        assert np.array_equal(got2, got)
