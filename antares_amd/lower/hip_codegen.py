@@ -11,10 +11,12 @@ templates:
   axis or constant along it (bias rows, gathered rows: `table[ids[N], C]`)
   (the reference's untuned default is one scalar element per block,
   antares/common.py:81-100);
-* reduce statements: three variants compiled together — one wavefront per
+* reduce statements: variants compiled together — one wavefront per
   output (DPP / readlane reduction), one 256-thread block per output, one
-  thread per output — and the launcher picks by extents and by which axis is
-  contiguous in memory (the reference reduces through LDS because its TVM patch
+  thread per output, and for contractions one thread per 4 x 4 patch of
+  outputs (register tiling: operands that are constant along one of the two
+  tiled axes are loaded once per patch) — and the launcher picks by extents
+  and by which axis is contiguous in memory (the reference reduces through LDS because its TVM patch
   disables wavefront shuffles off CUDA, engine/device-stub/tvm_v0.8.0.patch:186-191);
 * scatter statements: one thread per point of the iteration space, atomics for
   ``+=.  <=.  >=.``.
@@ -138,6 +140,8 @@ class KernelPlan:
     row_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for it
     row_dims: List[object] = field(default_factory=list)    # extents (int or dimension name) that must be multiples of row_vec
     reduce_contiguous: Optional[bool] = None   # True: a reduce axis is fastest in the biggest operand
+    patch: Optional[Tuple[int, int]] = None    # outputs per thread of the register-tiled reduce variant, along patch_dims
+    patch_dims: List[object] = field(default_factory=list)   # the two extents (int or dimension name) it tiles
     tile_axes: Optional[Tuple[str, str]] = None   # permutation copies: last axis of the load, last axis of the store
 
     def _tiles(self, env: Dict[str, int]) -> int:
@@ -165,6 +169,15 @@ class KernelPlan:
             return 0
         return total // self.row_vec
 
+    def _patches(self, env: Dict[str, int], total: int) -> int:
+        """Threads of the register-tiled reduce variant for these extents, 0 when it does not apply."""
+        if 'patch' not in self.variants or self.patch is None:
+            return 0
+        for d, t in zip(self.patch_dims, self.patch):
+            if (d if isinstance(d, int) else env[d]) % t:
+                return 0
+        return total // (self.patch[0] * self.patch[1])
+
     def choose(self, env: Dict[str, int], pointers: Dict[str, int]) -> Tuple[str, int, int]:
         """-> (kernel symbol, grid.x, block.x) for these extents and addresses."""
         total = 1
@@ -189,6 +202,9 @@ class KernelPlan:
         if self.kind == 'scatter':
             return self.variants['scalar'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
         # reduce
+        patches = self._patches(env, total)
+        if patches >= 131072 and red >= 8:           # two wavefronts per SIMD and more: below that one output per thread hides latency better
+            return self.variants['patch'], min((patches + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
         lanes_ok = self.reduce_contiguous is not False
         if red >= 2048 and total <= 1024 and lanes_ok:
             return self.variants['block'], min(total, MAX_GRID), BLOCK
@@ -221,6 +237,8 @@ class KernelPlan:
         else:
             waves_per_block = BLOCK // 64
             tags += [('thread', total), ('wave', (total + waves_per_block - 1) // waves_per_block * BLOCK), ('block', total * BLOCK)]
+            if self._patches(env, total):
+                tags.append(('patch', self._patches(env, total)))
         out = []
         for tag, work in tags:
             if tag not in self.variants:
@@ -547,8 +565,86 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
                                [f'    __acc = art_block_reduce(__acc, {op}, __smem);', f'    if (threadIdx.x == 0) {{ {store} }}']))
         variants.update({'thread': name + '_t', 'wave': name + '_w', 'block': name + '_b'})
         plan.reduce_contiguous = _reduce_axis_contiguous(st, tensors)
+        pa = _patch_axes(st)
+        if pa is not None:
+            # Register tiling for contractions (the reference's tiled schedule, backends/c-rocm/schedule/standard/
+            # algo_tiling.py:35-98): a thread owns TX x TY neighbouring outputs along two data axes chosen so that every
+            # operand is constant along one of them; the statement's expression is written out for each of the 16
+            # outputs and the compiler keeps one copy of every load they share.  Each output still accumulates its terms
+            # in the reference's order.
+            xa, ya = pa
+            ext = dict(st.data_axes)
+
+            def tile(e):                 # 4 outputs along an axis, 2 where a static extent only divides by 2
+                return 4 if not isinstance(e, int) or e % 4 == 0 else (2 if e % 2 == 0 else 0)
+            TX, TY = tile(ext[xa]), tile(ext[ya])
+        if pa is not None and TX and TY:
+            sym = name + '_p'
+            b = header(sym)
+            b.append(f'  const long long __red = {red_total};')
+            b.append(f'  const long long __px = __ext_{xa} / {TX}, __py = __ext_{ya} / {TY};')
+            b.append(f'  const long long __patches = __total / {TX * TY};')
+            b.append('  for (long long __o = __tid; __o < __patches; __o += __nthr) {')
+            b.append('    long long __r = __o;')
+            for ax, _ in reversed(st.data_axes):
+                if ax == ya:
+                    b.append(f'    const int __y0 = (int)(__r % __py) * {TY}; __r /= __py;')
+                elif ax == xa:
+                    b.append(f'    const int __x0 = (int)(__r % __px) * {TX}; __r /= __px;')
+                else:
+                    b.append(f'    const int {ax} = (int)(__r % __ext_{ax}); __r /= __ext_{ax};')
+            b.append(f'    {act} __acc[{TX}][{TY}];')
+            b.append('    #pragma unroll')
+            b.append(f'    for (int __i = 0; __i < {TX}; ++__i)')
+            b.append('      #pragma unroll')
+            b.append(f'      for (int __j = 0; __j < {TY}; ++__j) __acc[__i][__j] = {ident};')
+            b.append('    for (long long __k = 0; __k < __red; ++__k) {')
+            b += [l.replace('__r', '__q') for l in _decompose('__k', st.reduce_axes, '      ')]
+            b.append('      #pragma unroll')
+            b.append(f'      for (int __i = 0; __i < {TX}; ++__i) {{')
+            b.append('        #pragma unroll')
+            b.append(f'        for (int __j = 0; __j < {TY}; ++__j) {{')
+            b.append(f'          const int {xa} = __x0 + __i, {ya} = __y0 + __j; (void){xa}; (void){ya};')
+            b.append(f'          __acc[__i][__j] = {op}(__acc[__i][__j], ({act})({plain.expr(root)}));')
+            b += ['        }', '      }', '    }']
+            b.append('    #pragma unroll')
+            b.append(f'    for (int __i = 0; __i < {TX}; ++__i) {{')
+            b.append('      #pragma unroll')
+            b.append(f'      for (int __j = 0; __j < {TY}; ++__j) {{')
+            b.append(f'        const int {xa} = __x0 + __i, {ya} = __y0 + __j; (void){xa}; (void){ya};')
+            b.append(f'        const {act} __acc_ = __acc[__i][__j];')
+            pstore = f'{dst} = ({oct_})__acc_;'
+            b.append(f'        if ({cond}) {{ {pstore} }}' if cond else f'        {pstore}')
+            b += ['      }', '    }', '  }', '}']
+            src.append('\n'.join(b))
+            variants['patch'] = sym
+            plan.patch, plan.patch_dims = (TX, TY), [ext[xa], ext[ya]]
 
     return '\n\n'.join(src), plan
+
+
+def _patch_axes(st):
+    """(X, Y) for the register-tiled reduce variant: Y is the last data axis (lanes of a wavefront stay neighbours in
+    memory), X the data axis that leaves the most loads constant along X or Y - all of them in a matrix product or a
+    convolution.  None when the store is not indexed by the bare data axes, or no load is constant along either."""
+    axes = [a for a, _ in st.data_axes]
+    if len(axes) < 2 or st.scatter or [i.name for i in st.out_index if i.kind == 'axis'] != axes or len(st.out_index) != len(axes):
+        return None
+    loads = [n for n in walk(st.root) if n.kind == 'load']
+    if not loads or any(n.name == st.output for n in loads):
+        return None
+    def mentions(n, ax):
+        return any(m.kind == 'axis' and m.name == ax for a in n.args for m in walk(a))
+    ya = axes[-1]
+    best, best_score = None, 0
+    for xa in axes[:-1]:
+        score = sum(1 for n in loads if not mentions(n, xa) or not mentions(n, ya))
+        shared_x = sum(1 for n in loads if not mentions(n, xa))
+        if shared_x and score >= best_score:          # later axes win ties: their neighbours are closer in memory
+            best, best_score = xa, score
+    if best is None or not any(not mentions(n, ya) for n in loads):
+        return None
+    return best, ya
 
 
 def _reduce_axis_contiguous(st, tensors) -> Optional[bool]:

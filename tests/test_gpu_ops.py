@@ -543,3 +543,66 @@ def test_row_vector_maps_match_the_oracle(autort, ir, inputs, shapes, applies):
         view.copy_(tensors[0])
         got2 = op(view, *[t.to(dev) for t in tensors[1:]]).cpu().numpy()
         assert np.array_equal(got2, got)
+
+
+PATCH_CASES = [
+    ('output0[N, M] +=! input0[N, K] * input1[K, M]', ['input0=float32[N:64, K:96]', 'input1=float32[K:96, M:128]'], [(64, 96), (96, 128)]),
+    ('output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]', ['input0=float32[B:3, N:32, K:40]', 'input1=float32[B:3, K:40, M:64]'],
+     [(3, 32, 40), (3, 40, 64)]),
+    ('output0[N, M] +=! input0[N, K] * input1[M, K]', ['input0=float16[N:32, K:64]', 'input1=float16[M:48, K:64]'], [(32, 64), (48, 64)]),
+    ('output0[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[F, C, KH, KW] where HO in 10, WO in 12',
+     ['input0=float32[N:2, C:5, H:12, W:14]', 'input1=float32[F:8, C:5, KH:3, KW:3]'], [(2, 5, 12, 14), (8, 5, 3, 3)]),
+    ('output0[N, M] >=! input0[N, K] + input1[K, M]', ['input0=int32[N:16, K:33]', 'input1=int32[K:33, M:20]'], [(16, 33), (33, 20)]),
+]
+
+
+@pytest.mark.parametrize('ir,inputs,shapes', PATCH_CASES)
+def test_register_tiled_contractions_match_the_oracle(autort, ir, inputs, shapes, monkeypatch):
+    """The reduce variant in which a thread owns 4 x 4 neighbouring outputs (what large contractions get) gives the
+    oracle's results, and the bits of the one-output-per-thread variant, whose order of accumulation it keeps."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'register-tiled reduce {ir} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='patch_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    plan = op.plans[0]
+    assert 'patch' in plan.variants
+    g = torch.Generator().manual_seed(len(ir))
+    names = [spec.split('=')[0] for spec in inputs]
+    tensors = [torch.randint(-1000, 1000, shp, generator=g, dtype=torch.int32) if 'int32' in spec else
+               (torch.randn(shp, generator=g) * 0.5).to(torch.float16 if 'float16' in spec else torch.float32)
+               for spec, shp in zip(inputs, shapes)]
+    total = op(*[t.to(dev) for t in tensors]).numel()
+    results = {}
+    for tag in ('patch', 'thread'):
+        work = total // 16 if tag == 'patch' else total
+        monkeypatch.setattr(plan, 'choose', lambda env, ptrs, tag=tag, work=work: (plan.variants[tag], (work + 255) // 256, 256))
+        results[tag] = op(*[t.to(dev) for t in tensors]).cpu()
+    assert torch.equal(results['patch'], results['thread'])
+    out_name = ir.split('[', 1)[0].strip()
+    want = CpuModule(parse_program(ir, inputs), fast_math=False)(**{n: t.numpy() for n, t in zip(names, tensors)})[out_name]
+    got = results['patch'].numpy()
+    if got.dtype.kind == 'i':
+        assert np.array_equal(got, want)
+    else:
+        tol = 1e-2 if got.dtype == np.float16 else 1e-4
+        assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=tol, atol=tol)
+
+
+def test_large_contractions_take_the_register_tiled_variant(autort):
+    """A 2048 x 2048 x 256 fp32 matrix product is large enough for it (a 1024 x 1024 one is not); the result is the
+    float64 product's."""
+    note('register-tiled reduce picked for a 2048x2048x256 fp32 matmul')
+    dev = autort.device()
+    op = autort.export(ir='output0[N, M] +=! input0[N, K] * input1[K, M]', inputs=['input0=float32[N:2048, K:256]', 'input1=float32[K:256, M:2048]'],
+                       name='patch_matmul_2048')
+    plan = op.plans[0]
+    zero = {n: 0 for n in plan.args}
+    assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['patch']
+    assert plan.choose({'N': 2046, 'K': 256, 'M': 2048}, zero)[0] != plan.variants['patch']
+    assert plan.choose({'N': 1024, 'K': 256, 'M': 1024}, zero)[0] != plan.variants['patch']
+    g = torch.Generator().manual_seed(2)
+    a, b = torch.randn(2048, 256, generator=g), torch.randn(256, 2048, generator=g)
+    got = op(a.to(dev), b.to(dev)).cpu()
+    want = (a.double() @ b.double()).float()
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-3)
