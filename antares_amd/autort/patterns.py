@@ -172,3 +172,34 @@ def _gemm_f16_handler(op, bound, env, stream) -> bool:
 
 
 register(GEMM_F16_IR, GEMM_F16_INPUTS, _gemm_f16_handler)
+
+
+# ---------------------------------------------------------------------------
+# fp32 GEMM: C[M,N] = A[M,K] @ B[K,N] (AntaresIR.md:115 as written; the README's `gemm_f32`)
+# ---------------------------------------------------------------------------
+GEMM_F32_IR = 'c[M, N] +=! a[M, K] * b[K, N]'
+GEMM_F32_INPUTS = ['a=float32[M:4096, K:4096]', 'b=float32[K:4096, N:4096]']
+
+
+def _gemm_f32_handler(op, bound, env, stream) -> bool:
+    r = op.fast_roles
+    a, b, c = bound[r['a']], bound[r['b']], bound[r['c']]
+    M, K = a.shape
+    N = b.shape[1]
+    # small products are left to the generic lowering: a launch of the tiled kernel needs a few hundred tiles to pay
+    if N % 4 or K % 32 or N < 4 or M * N < 128 * 128 * 32 or a.data_ptr() % 16 or b.data_ptr() % 16:
+        return False
+
+    def run(_, t, st=None):
+        capi.check(capi.lib().art_gemm_f32(c_void_p(t[0].data_ptr()), c_void_p(t[1].data_ptr()), c_void_p(t[2].data_ptr()), M, N, K,
+                                          c_void_p(stream if st is None else st)))
+    # the kernel has no launch parameter to search; a tuning run records its time for the shape in the module file
+    key = f'gemm_f32|{M},{K},{N}'
+    trials = op.config.get('tune')
+    if key not in op.tuned and isinstance(trials, int) and trials > 0 and not torch.cuda.is_current_stream_capturing():
+        tune_hand_kernel(op, key, [0], lambda v, t: run(v, t, torch.cuda.current_stream().cuda_stream), 1, [(a, b, torch.empty_like(c))])
+    run(0, (a, b, c))
+    return True
+
+
+register(GEMM_F32_IR, GEMM_F32_INPUTS, _gemm_f32_handler)

@@ -234,6 +234,13 @@ int art_gemv_gptq(const void* x_dev, const void* qweight_dev, const void* scales
  * (AntaresIR.md:115; tiled schedule backends/c-rocm/schedule/standard/algo_tiling.py:35-98). */
 int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream);
 
+/* fp32 GEMM on the matrix cores (v_mfma_f32_32x32x2_f32): C[M,N] = A[M,K] @ B[K,N], all fp32, row-major; any M,
+ * N % 4 == 0, K % 32 == 0; A and B 16-byte aligned, C must not overlap them.
+ * Replaces the kernel the reference generates for `output0[N, M] +=! input0[N, K] * input1[K, M]` in float32
+ * (AntaresIR.md:115), the `gemm_f32` operator its README tunes (README.md:128-150; tiled schedule
+ * backends/c-rocm/schedule/standard/algo_tiling.py:35-98). */
+int art_gemm_f32(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream);
+
 /* Stable even-first partition of int32 values: all even values in input order,
  * then all odd values in input order.  Two launches (count, then rank + scatter),
  * 12 bytes of traffic per element, no atomics; at most 1024 blocks, each walking its span tile by tile

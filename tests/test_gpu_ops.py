@@ -596,6 +596,7 @@ def test_large_contractions_take_the_register_tiled_variant(autort):
     dev = autort.device()
     op = autort.export(ir='output0[N, M] +=! input0[N, K] * input1[K, M]', inputs=['input0=float32[N:2048, K:256]', 'input1=float32[K:256, M:2048]'],
                        name='patch_matmul_2048')
+    op.fast_path = None               # this shape would go to the matrix-core kernel: the generic lowering is what is tested here
     plan = op.plans[0]
     zero = {n: 0 for n in plan.args}
     assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['patch']
@@ -606,3 +607,27 @@ def test_large_contractions_take_the_register_tiled_variant(autort):
     got = op(a.to(dev), b.to(dev)).cpu()
     want = (a.double() @ b.double()).float()
     assert torch.allclose(got, want, rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize('M,N,K', [(512, 1024, 32), (1000, 1028, 96), (4096, 4096, 512), (129, 8192, 64), (2048, 2048, 2048)])
+def test_fp32_gemm_on_the_matrix_cores_matches_the_float64_product(autort, M, N, K):
+    """`C[M,N] +=! A[M,K] * B[K,N]` in float32 goes to art_gemm_f32 (edge tiles in M and N included); the result is
+    the float64 product's to fp32 accuracy, and identity / one-hot operands pin operand order and transposition."""
+    note(f'gemm_f32 {M}x{N}x{K}')
+    dev = autort.device()
+    op = autort.export(ir='c[M, N] +=! a[M, K] * b[K, N]', inputs=[f'a=float32[M:{M}, K:{K}]', f'b=float32[K:{K}, N:{N}]'], name=f'gemm_f32_{M}_{N}_{K}')
+    assert op.fast_path is not None
+    g = torch.Generator().manual_seed(M + N + K)
+    a, b = torch.randn(M, K, generator=g), torch.randn(K, N, generator=g)
+    got = op(a.to(dev), b.to(dev)).cpu()
+    want = a.double() @ b.double()
+    # fp32 sums of K products of N(0,1) values: error about sqrt(K) * 2^-24 * |terms|
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5 * max(1.0, K ** 0.5)), (got.double() - want).abs().max()
+    if M == 512:
+        sel = torch.zeros(M, K)
+        sel[torch.arange(M), torch.arange(M) % K] = 1.0              # row m of the result = row m % K of b
+        assert torch.equal(op(sel.to(dev), b.to(dev)).cpu(), b[torch.arange(M) % K])
+    # shapes the kernel does not take run through the generic lowering, same operator
+    small = autort.export(ir='c[M, N] +=! a[M, K] * b[K, N]', inputs=['a=float32[M:40, K:24]', 'b=float32[K:24, N:36]'], name='gemm_f32_small')
+    a2, b2 = torch.randn(40, 24, generator=g), torch.randn(24, 36, generator=g)
+    assert torch.allclose(small(a2.to(dev), b2.to(dev)).cpu().double(), a2.double() @ b2.double(), rtol=1e-5, atol=1e-5)
