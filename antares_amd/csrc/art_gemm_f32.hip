@@ -15,9 +15,14 @@
 //     rows of 32 k are full 128-byte lines of A, kept in LDS as [m][k] (row pitch 36 floats: 16-byte aligned and the
 //     eight rows of a quarter wavefront on distinct banks); B stays as it lies in memory, [k][n] (512 contiguous bytes
 //     per wavefront on the way in, 16-byte LDS stores), and a lane picks its four values of k with four 4-byte reads
-//     that 32 lanes spread over 32 banks - transposing B on the way into LDS costs 16-way bank conflicts instead;
+//     that the two halves of a wavefront (rows 4 k apart, row pitch 136 floats) spread over all 64 banks -
+//     transposing B on the way into LDS costs 16-way bank conflicts instead;
 //   * global -> registers -> LDS with one tile in flight in registers while the previous one is multiplied, two LDS
-//     buffers, one barrier per tile;
+//     buffers, one barrier per tile; inside a tile the issue order is pinned (sched_group_barrier): the LDS reads of
+//     the next 8 values of k, the 16-byte global reads and the LDS writes each go out one at a time between matrix
+//     instructions - issued in bursts they fill the LDS queues and the matrix pipe waits (measured at 4096^3:
+//     126 -> 141 TFLOP/s);
+//   * block -> tile mapping is XCD aware (a contiguous run of tiles per XCD, walked in 4 x 8 super-tiles);
 //   * C leaves straight from the accumulators: 32 lanes write 128 contiguous bytes of a row.
 #include "art_common.h"
 
@@ -26,10 +31,10 @@ namespace {
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int BM = 128, BN = 128, BK = 32, LD = BK + 4, LDB = BN + 4;
+constexpr int BM = 128, BN = 128, BK = 32, LD = BK + 4, LDB = BN + 8;
 constexpr int kThreads = 256;
 constexpr int TILE = BM * LD, TILE_B = BK * LDB;    // floats per operand tile in LDS
-constexpr size_t kLdsBytes = (size_t)2 * (TILE + TILE_B) * sizeof(float);     // A and B, two buffers each: 70656
+constexpr size_t kLdsBytes = (size_t)2 * (TILE + TILE_B) * sizeof(float);     // A and B, two buffers each: 71680
 
 __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
                                                              float* __restrict__ C, int M, int N, int K, int tiles_n) {
@@ -38,7 +43,23 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
   float* Bs = smem32 + 2 * TILE;                    // [2][BK][LDB]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+  // block -> tile, XCD aware: workgroups go to the eight XCDs round robin, so the blocks of one XCD get a contiguous
+  // run of tiles, and a run is walked in 4 x 8 super-tiles (4 A panels and 8 B panels shared through that XCD's L2)
+  int tm, tn;
+  {
+    const int nb = (int)gridDim.x, b = (int)blockIdx.x;
+    const int q = nb >> 3, r = nb & 7, xcd = b & 7, idx = b >> 3;
+    const int tile = xcd < r ? xcd * (q + 1) + idx : r * (q + 1) + (xcd - r) * q + idx;
+    const int tiles_m = nb / tiles_n;
+    if ((tiles_m % 4 == 0) && (tiles_n % 8 == 0)) {
+      const int super = tile >> 5, in = tile & 31, sn = tiles_n >> 3;
+      tm = (super / sn) * 4 + (in >> 3);
+      tn = (super % sn) * 8 + (in & 7);
+    } else {
+      tm = tile / tiles_n;
+      tn = tile % tiles_n;
+    }
+  }
 
   // global -> registers: four 16-byte chunks of each operand per thread and tile.  Rows past M and columns past N
   // repeat the last valid ones; their products are never stored.
@@ -80,30 +101,84 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
   load_tiles(0);
   store_tiles(0);
   __syncthreads();
+  // Tile t is multiplied out of LDS buffer t % 2 while tile t + 1 travels global memory -> registers -> the other
+  // buffer (past the last tile the last one is loaded and stored again, which nobody reads: no branch splits the
+  // tile's scheduling region).  The loop is rotated by one group of 8 k: the last group of a tile is multiplied after
+  // the barrier, out of registers, while the first group of the next tile is read - the wait at the barrier and the
+  // first LDS reads behind it cost the matrix pipe nothing.  Before the first tile that group is all zeros.
+  f32x4 a[2][2], b[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) a[1][i][m] = b[1][i][m] = 0.f;
+  auto multiply = [&](int s) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s][i][m], b[s][j][m], acc[i][j], 0, 0, 0);
+  };
   for (int t = 0; t < T; ++t) {
     const int buf = t & 1;
-    if (t + 1 < T) load_tiles(t + 1);               // in flight while this tile is multiplied
     const float* as = As + buf * TILE;
     const float* bs = Bs + buf * TILE_B;
+    auto load_group = [&](int g, int s) {
 #pragma unroll
-    for (int g = 0; g < BK / 8; ++g) {
-      f32x4 a[2], b[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const f32x4*>(as + (row_a + 32 * i) * LD + g * 8 + k_half);
+      for (int i = 0; i < 2; ++i) a[s][i] = *reinterpret_cast<const f32x4*>(as + (row_a + 32 * i) * LD + g * 8 + k_half);
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int m = 0; m < 4; ++m) b[j][m] = bs[(g * 8 + k_half + m) * LDB + col_b + 32 * j];
+        for (int m = 0; m < 4; ++m) b[s][j][m] = bs[(g * 8 + k_half + m) * LDB + col_b + 32 * j];
+    };
+    multiply(1);                                    // group 3 of the previous tile
+    load_group(0, 0);
+    load_tiles(t + 1 < T ? t + 1 : T - 1);
+    load_group(1, 1);
+    multiply(0);
+    load_group(2, 0);
+    multiply(1);
+    load_group(3, 1);
+    store_tiles(buf ^ 1);                           // the other buffer: everybody left it at the last barrier
+    multiply(0);
+    // Issue order of the tile (one scheduling region): memory instructions are spread between the matrix
+    // instructions one at a time, so that neither the LDS queues nor the matrix pipe run dry or full.
+    // masks: 0x008 matrix, 0x020 global read, 0x100 LDS read, 0x200 LDS write
 #pragma unroll
-      for (int m = 0; m < 4; ++m)
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][m], b[j][m], acc[i][j], 0, 0, 0);
+    for (int n = 0; n < 6; ++n) {                                            // previous group 3 multiplies, group 0 is read
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
-    if (t + 1 < T) store_tiles(buf ^ 1);            // the other buffer: everybody left it at the last barrier
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {                                            // ... and the next tile is asked for
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {                                            // groups 0 and 1 multiply, 1 and 2 are read
+#pragma unroll
+      for (int n = 0; n < 6; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 10, 0);
+    }
+#pragma unroll
+    for (int n = 0; n < 6; ++n) {                                            // group 2 multiplies, group 3 is read
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {                                            // ... and the next tile goes to LDS
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
     __syncthreads();
   }
+  multiply(1);                                      // group 3 of the last tile
 
   // accumulator element r of tile (i, j): row i*32 + (r/4)*8 + (lane/32)*4 + r%4, column j*32 + lane%32
 #pragma unroll
