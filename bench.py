@@ -35,6 +35,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+MFMA_F32_PEAK_TFLOPS = 157.3
 LAYERS = 32
 # HBM bytes per launch of the headline GEMV kernel come from the committed counter summary (FETCH_SIZE / WRITE_SIZE
 # scaled by the copy-kernel calibration), which states them on a line `traffic_bytes_per_launch: <integer>`.
@@ -262,6 +263,20 @@ def bench_gemm_f16(torch, autort, capi, workloads, steps, warmup, seed, n):
     tflops = 2.0 * n * n * n / sec / 1e12
     return {'workload': f'fp16 GEMM M=N=K={n} (fp32 accumulate)', 'us_per_launch': sec * 1e6, 'tflops': tflops,
             'roofline_bound': 'mfma', 'roofline_frac': tflops / MFMA_F16_PEAK_TFLOPS}
+
+
+def bench_gemm_f32(torch, autort, capi, steps, warmup, seed, n):
+    """The float32 matrix product as AntaresIR.md:115 writes it (the README's `gemm_f32`), on the fp32 matrix instructions."""
+    from antares_amd.autort import patterns
+    dev = autort.device()
+    op = autort.export(ir=patterns.GEMM_F32_IR, inputs=patterns.GEMM_F32_INPUTS, name='gemm_f32')
+    g = torch.Generator('cpu').manual_seed(seed)
+    a, b = (torch.randn(n, n, generator=g).to(dev) for _ in range(2))
+    c = torch.empty(n, n, dtype=torch.float32, device=dev)
+    sec = time_graph(torch, capi, lambda: op(a, b, out=c), steps, warmup, warm_ms=40.0)
+    tflops = 2.0 * n * n * n / sec / 1e12
+    return {'workload': f'fp32 GEMM M=N=K={n}', 'us_per_launch': sec * 1e6, 'tflops': tflops,
+            'roofline_bound': 'mfma', 'roofline_frac': tflops / MFMA_F32_PEAK_TFLOPS}
 
 
 def bench_sigmoid(torch, autort, capi, workloads, steps, warmup, seed, n=4_096_000, copies=16):
@@ -497,6 +512,8 @@ def main():
         for n in (4096, 8192):
             r = bench_gemm_f16(torch, autort, capi, workloads, max(5, args.steps // 4), args.warmup, args.seed, n)
             extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
+        r = bench_gemm_f32(torch, autort, capi, max(5, args.steps // 4), args.warmup, args.seed, 4096)
+        extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
         for fn in (bench_sigmoid, bench_partition):
             r = fn(torch, autort, capi, workloads, args.steps, args.warmup, args.seed)
             extra.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
