@@ -138,7 +138,12 @@ def _w4a16_handler(op, bound, env, stream) -> bool:
         per_set = q.numel() + 2 * s.numel() + z.numel()
         copies = max(1, min(8, (256 << 20) // max(per_set, 1)))
         clones = [(x, q.clone(), s.clone(), z.clone(), torch.empty_like(y)) for _ in range(copies)]
-        cands = ([512, 256, 1024] if M == 1 else [512, 256]) if gemv else [0] + [v for v in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32) if v <= K // 128]
+        if gemv:
+            cands = [512, 256, 1024] if M == 1 else [512, 256]
+        else:
+            counts = [v for v in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32) if v <= K // 128]
+            # 512 + v: v K-splits over blocks of 64 rows; 256 + v: over blocks of 32 rows (twice the blocks)
+            cands = [0] + [512 + v for v in counts] + ([256 + v for v in counts] if M > 32 else [])
         saved = tune_hand_kernel(op, key, cands, lambda v, t: run(v, t, torch.cuda.current_stream().cuda_stream), trials, clones)
         del clones
     run(saved['value'] if saved is not None else 0, (x, q, s, z, y))

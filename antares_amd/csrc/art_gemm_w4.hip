@@ -48,7 +48,6 @@ constexpr int Q_BYTES = 2048;                       // scales (512 B) at 0, zero
 constexpr int STAGE = W_BYTES + X_BYTES + Q_BYTES;
 constexpr int RLD = BN + 4;                         // floats per row of a result tile in LDS
 constexpr size_t kLdsBytes = (size_t)NS * STAGE;    // 139264; the two result tiles of the epilogue (133120) reuse it
-constexpr int kLoadsPerGroup = 5;                   // LDS-direct loads per wavefront and group: 2 weights, 2 x, 1 scales / zero points
 static_assert(2 * BM * RLD * sizeof(float) <= kLdsBytes, "the result tiles fit the ring");
 
 struct Magic {
@@ -87,7 +86,7 @@ __device__ __forceinline__ void load_lds_x1(const void* g, unsigned int lds_dst)
                : "=&s"(keep) : "v"(g), "s"(lds_dst) : "memory");
 }
 
-template <int MT>   // MT accumulator tiles of 32 rows: 1 for M <= 32, 2 for M <= 64
+template <int MT>   // MT accumulator tiles of 32 rows: a block owns 32 MT rows
 __global__ __launch_bounds__(kThreads) void gemm_w4a16_kernel(const _Float16* __restrict__ x, const unsigned char* __restrict__ qweight,
                                                               const _Float16* __restrict__ scales,
                                                               const unsigned char* __restrict__ qzeros, _Float16* y,
@@ -107,8 +106,10 @@ __global__ __launch_bounds__(kThreads) void gemm_w4a16_kernel(const _Float16* __
   if (unit >= col_tiles * splits) return;
   const int split = unit / col_tiles;
   const int n0 = (unit % col_tiles) * BN;
-  const int m0 = m_block * BM;
-  const int M = M_total - m0 < BM ? M_total - m0 : BM;          // rows of this block
+  constexpr int RB = 32 * MT;                       // rows of a block
+  constexpr int kLoadsPerGroup = 3 + MT;            // LDS-direct loads per wavefront and group: 2 weights, MT x, 1 scales / zero points
+  const int m0 = m_block * RB;
+  const int M = M_total - m0 < RB ? M_total - m0 : RB;          // rows of this block
   x += (size_t)m0 * K;
   y += (size_t)m0 * N;
   if (residual) residual += (size_t)m0 * N;
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(kThreads) void gemm_w4a16_kernel(const _Float16* __
 #pragma unroll
     for (int u = 0; u < 2; ++u) load_lds_x4(wsrc[u] + (size_t)b * (GK / 2) * N, st + (wave + 8 * u) * 1024);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) load_lds_x4(xsrc[u] + (size_t)b * GK, st + W_BYTES + (wave + 8 * u) * 1024);
+    for (int u = 0; u < MT; ++u) load_lds_x4(xsrc[u] + (size_t)b * GK, st + W_BYTES + (wave + 8 * u) * 1024);    // 32 rows each
     load_lds_x1(qsrc + (size_t)b * qstep, st + W_BYTES + X_BYTES + wave * 256);
   };
 
@@ -336,9 +337,9 @@ extern "C" int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, 
 
 extern "C" int art_gemm_w4a16_residual(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                                        void* y_dev, const void* residual_dev, int M, int K, int N, int k_splits, void* stream) {
+  ART_REQUIRE(k_splits >= 0 && k_splits < 0x300, "art_gemm_w4a16: k_splits must be 0 (library's choice) or 1..255, plus 256 x the rows-per-block code (got %d)", k_splits);
   ART_REQUIRE(((uintptr_t)residual_dev % 8) == 0, "art_gemm_w4a16: the residual must be 8-byte aligned");
   ART_REQUIRE(!art::overlaps(x_dev, (size_t)M * K * 2, y_dev, (size_t)M * N * 2), "art_gemm_w4a16: y must not overlap x");
-  ART_REQUIRE(k_splits >= 0, "art_gemm_w4a16: k_splits must be 0 (library's choice) or positive (got %d)", k_splits);
   ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemm_w4a16: null pointer");
   ART_REQUIRE(M >= 1, "art_gemm_w4a16: M must be positive (got %d)", M);
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemm_w4a16: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
@@ -363,12 +364,25 @@ extern "C" int art_gemm_w4a16_residual(const void* x_dev, const void* qweight_de
   const Magic mg{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
   hipStream_t st = (hipStream_t)stream;
   const int G = K / GK, col_tiles = (N + BN - 1) / BN;
-  // Up to kMaxRowBlocks blocks of 64 rows go into one launch (they share the weight stream through L2, and the K-splits
+  // Up to kMaxRowBlocks row blocks go into one launch (they share the weight stream through L2, and the K-splits
   // are combined once); longer batches take several passes over the weights.
+  // Rows per block: 64, or 32 where twice the blocks fill the chip better than twice the K-splits do - a block of 32
+  // rows unpacks the same weights for half the matrix instructions, but every K-split it saves is an fp32 copy of
+  // the output less to write and read back.  The caller's choice arrives in the upper bits of k_splits.
   constexpr int kMaxRowBlocks = 8;
-  for (int m0 = 0; m0 < M; m0 += BM * kMaxRowBlocks) {
-    const int rows = M - m0 < BM * kMaxRowBlocks ? M - m0 : BM * kMaxRowBlocks;
-    const int m_blocks = (rows + BM - 1) / BM;
+  const int want_rows = k_splits >> 8;              // 0: library's choice, 1: 32-row blocks, 2: 64-row blocks
+  k_splits &= 0xff;
+  ART_REQUIRE(want_rows <= 2, "art_gemm_w4a16: rows-per-block code must be 0, 1 or 2 (got %d)", want_rows);
+  int block_rows = BM;
+  if (want_rows == 1 || M <= 32) block_rows = 32;
+  else if (want_rows == 0 && M <= 64) {
+    // measured at M = 64 on MI355X: 32-row blocks win where one block per compute unit then covers at least four
+    // K-splits' worth of column tiles (4096 columns), and lose where they would need a second round of blocks
+    if (col_tiles * 2 * 4 <= compute_units) block_rows = 32;
+  }
+  for (int m0 = 0; m0 < M; m0 += block_rows * kMaxRowBlocks) {
+    const int rows = M - m0 < block_rows * kMaxRowBlocks ? M - m0 : block_rows * kMaxRowBlocks;
+    const int m_blocks = (rows + block_rows - 1) / block_rows;
     int splits = choose_splits(rows, N, K, scratch_bytes, compute_units / m_blocks);
     if (k_splits > 0) {           // the caller's choice, within what the kernel and the scratch space take
       const int cap = (int)(scratch_bytes / ((size_t)rows * N * sizeof(float)));
@@ -379,7 +393,7 @@ extern "C" int art_gemm_w4a16_residual(const void* x_dev, const void* qweight_de
     _Float16* ys = (_Float16*)y_dev + (size_t)m0 * N;
     const _Float16* rs = residual_dev ? (const _Float16*)residual_dev + (size_t)m0 * N : nullptr;
     const dim3 grid((unsigned)((col_tiles * splits + 7) / 8 * 8 * m_blocks));
-    if (rows <= 32)
+    if (block_rows == 32)
       gemm_w4a16_kernel<1><<<grid, kThreads, kLdsBytes, st>>>(xs, (const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                          (const unsigned char*)qzeros_dev, ys, scratch, rows, K, N, splits,
                                                          col_tiles, m_blocks, mg, rs);

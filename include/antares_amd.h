@@ -157,7 +157,10 @@ int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scale
  *   k_per_block:   256, 512 or 1024 values of k per block of the int4 GEMV (4 or 8 packed rows per lane in four
  *                  wavefronts, or 8 rows in eight wavefronts; 1024 needs M = 1): fewer k per block = more blocks and
  *                  more returning atomics per column;
- *   k_splits:      number of K-splits of the int4 GEMM (clamped to K/128 and to what the workspace holds);
+ *   k_splits:      number of K-splits of the int4 GEMM, 1..255 (clamped to K/128 and to what the workspace holds),
+ *                  plus 256 for blocks of 32 rows or 512 for blocks of 64 rows (neither: the library picks; batches of
+ *                  up to 32 rows always take 32-row blocks): 32-row blocks are twice as many and need fewer K-splits,
+ *                  i.e. fewer fp32 copies of the output written and read back, but unpack every weight twice;
  *   max_blocks:    cap on the blocks of the partition, 64..16384 (each walks its span tile by tile). */
 int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                          void* y_dev, int M, int K, int N, int k_per_block, void* stream);

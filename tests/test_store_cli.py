@@ -142,7 +142,7 @@ def test_tune_config_times_candidates_and_keeps_the_winner(ops_dir):
 @pytest.mark.gpu
 def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
     """config="tune:N" on a program that runs on a hand-written kernel searches that kernel's launch parameter (rows
-    per lane of the int4 GEMV, K-splits of the int4 GEMM) for the shape of the call, keeps the winner in the module
+    per lane of the int4 GEMV, K-splits and rows per block of the int4 GEMM) for the shape of the call, keeps the winner in the module
     file, and the tuned operator - like every value of the parameter - matches the oracle."""
     import subprocess
     from ctypes import c_void_p
@@ -159,7 +159,7 @@ def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
             (1, 4096, 4096, 'gemv_w4a16.k_per_block|1,4096,4096', lib.art_gemv_w4a16_tuned, (0, 256, 512, 1024)),
             (1, 11008, 528, 'gemv_w4a16.k_per_block|1,11008,528', lib.art_gemv_w4a16_tuned, (256, 512, 1024)),
             (2, 1024, 1040, 'gemv_w4a16.k_per_block|2,1024,1040', lib.art_gemv_w4a16_tuned, (256, 512)),
-            (64, 4096, 4096, 'gemm_w4a16.k_splits|64,4096,4096', lib.art_gemm_w4a16_tuned, (0, 1, 3, 8, 32, 1000))]:
+            (64, 4096, 4096, 'gemm_w4a16.k_splits|64,4096,4096', lib.art_gemm_w4a16_tuned, (0, 1, 3, 8, 32, 255, 256 + 2, 256 + 8, 256, 512 + 3))]:
         print(f'[case] tuned int4 product M={M} K={K} N={N}', flush=True)
         p = workloads.w4_problem(M + K + N, M, K, N)
         want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy()).astype(np.float32)
@@ -167,7 +167,8 @@ def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
         got = f(*d)
         assert np.allclose(got.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
         choice = f.tuned[key]
-        assert choice['us'] > 0 and (choice['value'] in (256, 512, 1024) if 'gemv' in key else 0 <= choice['value'] <= K // 128)
+        assert choice['us'] > 0 and (choice['value'] in (256, 512, 1024) if 'gemv' in key
+                                    else (choice['value'] & 255) <= K // 128 and choice['value'] >> 8 in (0, 1, 2))
         assert store.load('w4a16_tuned')['tuned'][key] == choice
         assert torch.equal(f(*d), got)                              # the stored choice is used again, no new search
         for v in values:                                            # every value of the parameter gives the oracle's result
@@ -182,6 +183,8 @@ def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
     # a value outside the parameter's range is refused
     assert lib.art_gemv_w4a16_tuned(None, None, None, None, None, 1, 4096, 4096, 5, None) != 0
     assert b'k_per_block' in lib.art_last_error()
+    assert lib.art_gemm_w4a16_tuned(None, None, None, None, None, 64, 4096, 4096, 0x300, None) != 0
+    assert b'rows-per-block' in lib.art_last_error()
 
 
 @pytest.mark.gpu
