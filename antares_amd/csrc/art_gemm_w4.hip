@@ -296,8 +296,21 @@ __global__ __launch_bounds__(256) void gemm_w4a16_combine_kernel(const float* __
                                                                   const _Float16* residual) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i >= count4) return;
+  // eight splits at a time: all eight loads are issued before the first is added (a loop of load-then-add runs one
+  // memory round trip per split); the additions keep the split order.  Past the last split a load repeats split 0
+  // and is not added.
   f32x4 t = *reinterpret_cast<const f32x4*>(partial + i * 4);
-  for (int s = 1; s < splits; ++s) t += *reinterpret_cast<const f32x4*>(partial + s * split_stride + i * 4);
+  for (int s0 = 1; s0 < splits; s0 += 8) {
+    f32x4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int s = s0 + j < splits ? s0 + j : 0;
+      v[j] = *reinterpret_cast<const f32x4*>(partial + s * split_stride + i * 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (s0 + j < splits) t += v[j];
+  }
   h4 out = h4{(_Float16)t[0], (_Float16)t[1], (_Float16)t[2], (_Float16)t[3]};
   if (residual) {                    // y = fp16(fp16(product) + residual); residual may be y itself
     const h4 res = *reinterpret_cast<const h4*>(residual + i * 4);
@@ -310,7 +323,8 @@ __global__ __launch_bounds__(256) void gemm_w4a16_combine_kernel(const float* __
 // Number of K-splits: as many blocks as the chip holds at once (one per compute unit), but at least
 // two groups per block, no more partial-tile bytes than weight bytes (every split adds an fp32 copy of
 // the output to the traffic), and no more than the scratch space allows.  The rule lands on the measured
-// optimum at M = 64 on MI355X: 8 splits for 4096x4096, 5 for 4096x11008, 16 for 11008x4096, 2 for 4096x32000.
+// optimum at M = 64 on MI355X: 8 splits for 4096x4096 and 11008x4096 (two 32-row blocks each), 5 for 4096x11008,
+// 2 for 4096x32000.
 int choose_splits(int rows, int N, int K, size_t scratch_bytes, int compute_units) {
   const int col_tiles = (N + BN - 1) / BN, G = K / GK;
   int s = (512 / kThreads) * compute_units / col_tiles;      // blocks that are resident at once
