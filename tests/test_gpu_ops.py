@@ -395,6 +395,44 @@ def test_permutation_copies_go_through_lds_tiles(autort, ir, spec, shape, perm):
     assert torch.equal(op(x.to(dev)).cpu(), want)
 
 
+@pytest.mark.parametrize('ir,spec,shape,perm', [
+    ('output0[C, N] = input0[N, C]', 'input0=float32[N:1024, C:448]', (1024, 448), (1, 0)),
+    ('output0[N, H, W, C] = input0[N, C, H, W]', 'input0=float16[N:2, C:128, H:3, W:64]', (2, 128, 3, 64), (0, 2, 3, 1)),
+    ('output0[B, C, N] = input0[N, B, C] * 2', 'input0=float32[N:192, B:3, C:64]', (192, 3, 64), (1, 2, 0)),
+    ('output0[C, N] = input0[N, C].cast(`float32`)', 'input0=int32[N:64, C:4096]', (64, 4096), (1, 0)),
+])
+def test_permutation_copies_of_whole_tiles_move_16_byte_vectors(autort, ir, spec, shape, perm):
+    """With whole 64 x 64 tiles and aligned tensors the transposing variant reads and writes 16-byte vectors; a view
+    that is not 16-byte aligned takes the scalar tiles, with the same result."""
+    note(f'vector-tiled permutation {ir} {shape}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=[spec], name='permv_' + str(abs(hash((ir, spec))) % 10 ** 8))
+    plan = op.plans[0]
+    assert 'tilevec' in plan.variants
+    g = torch.Generator().manual_seed(5)
+    if 'int32' in spec:
+        x = torch.randint(-10 ** 6, 10 ** 6, shape, generator=g, dtype=torch.int32)
+    else:
+        x = torch.randn(shape, generator=g).to(torch.float16 if 'float16' in spec else torch.float32)
+    want = x.permute(*perm).contiguous()
+    if '* 2' in ir:
+        want = want * 2
+    if 'cast' in ir:
+        want = want.float()
+    xd = x.to(dev)
+    env = {k: v for k, v in zip([d.split(':')[0] for d in spec[spec.index('[') + 1:-1].split(', ')], shape)}
+    out = torch.empty(want.shape, dtype=want.dtype, device=dev)
+    assert plan.choose(env, {'input0': xd.data_ptr(), 'output0': out.data_ptr()})[0] == plan.variants['tilevec']
+    assert torch.equal(op(xd).cpu(), want)
+    # the same values 4 bytes further on: not aligned for vectors
+    flat = torch.empty(x.numel() + 4, dtype=x.dtype, device=dev)
+    skip = 4 // x.element_size()
+    shifted = flat[skip:skip + x.numel()].view(shape)
+    shifted.copy_(xd)
+    assert plan.choose(env, {'input0': shifted.data_ptr(), 'output0': out.data_ptr()})[0] == plan.variants['tile']
+    assert torch.equal(op(shifted).cpu(), want)
+
+
 def test_split_k_launches_on_two_streams_do_not_disturb_each_other(autort):
     """Every stream has a workspace of its own: GEMVs with K-splits enqueued on two streams at the same time give
     the bits they give alone, and an aliasing y is refused."""
