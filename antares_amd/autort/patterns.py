@@ -208,3 +208,27 @@ def _gemm_f32_handler(op, bound, env, stream) -> bool:
 
 
 register(GEMM_F32_IR, GEMM_F32_INPUTS, _gemm_f32_handler)
+
+
+# ---------------------------------------------------------------------------
+# batched fp32 GEMM: C[B,M,N] = A[B,M,K] @ B[B,K,N] (AntaresIR.md:121)
+# ---------------------------------------------------------------------------
+BATCH_GEMM_F32_IR = 'c[B, M, N] +=! a[B, M, K] * b[B, K, N]'
+BATCH_GEMM_F32_INPUTS = ['a=float32[B:3, M:1024, K:512]', 'b=float32[B:3, K:512, N:512]']
+
+
+def _batch_gemm_f32_handler(op, bound, env, stream) -> bool:
+    r = op.fast_roles
+    a, b, c = bound[r['a']], bound[r['b']], bound[r['c']]
+    batch, M, K = a.shape
+    N = b.shape[2]
+    # as for the single product: the tiled kernel needs a few hundred tiles to pay
+    if N % 4 or K % 32 or N < 4 or batch > 65535 or batch * M * N < 128 * 128 * 32 or a.data_ptr() % 16 or b.data_ptr() % 16 \
+            or (M * K) % 4 or (K * N) % 4:
+        return False
+    capi.check(capi.lib().art_gemm_f32_batched(c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()), batch, M, N, K,
+                                              c_void_p(stream)))
+    return True
+
+
+register(BATCH_GEMM_F32_IR, BATCH_GEMM_F32_INPUTS, _batch_gemm_f32_handler)

@@ -43,6 +43,9 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
   float* Bs = smem32 + 2 * TILE;                    // [2][BK][LDB]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
+  A += (size_t)blockIdx.y * M * K;                  // one product of the batch per grid row
+  B += (size_t)blockIdx.y * K * N;
+  C += (size_t)blockIdx.y * M * N;
   // block -> tile, XCD aware: workgroups go to the eight XCDs round robin, so the blocks of one XCD get a contiguous
   // run of tiles, and a run is walked in 4 x 8 super-tiles (4 A panels and 8 B panels shared through that XCD's L2)
   int tm, tn;
@@ -196,13 +199,15 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
 
 }  // namespace
 
-extern "C" int art_gemm_f32(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream) {
+extern "C" int art_gemm_f32_batched(const void* a_dev, const void* b_dev, void* c_dev, int batch, int M, int N, int K, void* stream) {
   ART_REQUIRE(a_dev && b_dev && c_dev, "art_gemm_f32: null pointer");
+  ART_REQUIRE(batch > 0 && batch <= 65535, "art_gemm_f32: batch must be 1..65535 (got %d)", batch);
   ART_REQUIRE(M > 0 && N >= 4 && K > 0 && N % 4 == 0 && K % 32 == 0,
               "art_gemm_f32: N must be a multiple of 4 and K of 32 (M=%d N=%d K=%d)", M, N, K);
   ART_REQUIRE(((uintptr_t)a_dev % 16) == 0 && ((uintptr_t)b_dev % 16) == 0 && ((uintptr_t)c_dev % 4) == 0,
               "art_gemm_f32: A and B must be 16-byte aligned");
-  ART_REQUIRE(!art::overlaps(a_dev, (size_t)M * K * 4, c_dev, (size_t)M * N * 4) && !art::overlaps(b_dev, (size_t)K * N * 4, c_dev, (size_t)M * N * 4),
+  const size_t nb = (size_t)batch;
+  ART_REQUIRE(!art::overlaps(a_dev, nb * M * K * 4, c_dev, nb * M * N * 4) && !art::overlaps(b_dev, nb * K * N * 4, c_dev, nb * M * N * 4),
               "art_gemm_f32: C must not overlap A or B");
   static bool configured = false;
   if (!configured) {
@@ -211,8 +216,12 @@ extern "C" int art_gemm_f32(const void* a_dev, const void* b_dev, void* c_dev, i
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   ART_REQUIRE((long long)tiles_m * tiles_n <= 0x7fffffffLL, "art_gemm_f32: too many tiles");
-  gemm_f32_kernel<<<dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, (hipStream_t)stream>>>(
+  gemm_f32_kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(kThreads), kLdsBytes, (hipStream_t)stream>>>(
       (const float*)a_dev, (const float*)b_dev, (float*)c_dev, M, N, K, tiles_n);
   ART_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int art_gemm_f32(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream) {
+  return art_gemm_f32_batched(a_dev, b_dev, c_dev, 1, M, N, K, stream);
 }

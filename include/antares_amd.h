@@ -243,6 +243,10 @@ int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, int M, int N
  * (AntaresIR.md:115), the `gemm_f32` operator its README tunes (README.md:128-150; tiled schedule
  * backends/c-rocm/schedule/standard/algo_tiling.py:35-98). */
 int art_gemm_f32(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream);
+/* `batch` such products in one launch, operands and results stored one after the other: C[b] = A[b] @ B[b].
+ * Replaces the kernel the reference generates for `output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]`
+ * (AntaresIR.md:121). */
+int art_gemm_f32_batched(const void* a_dev, const void* b_dev, void* c_dev, int batch, int M, int N, int K, void* stream);
 
 /* Stable even-first partition of int32 values: all even values in input order,
  * then all odd values in input order.  Two launches (count, then rank + scatter),

@@ -669,3 +669,22 @@ def test_fp32_gemm_on_the_matrix_cores_matches_the_float64_product(autort, M, N,
     small = autort.export(ir='c[M, N] +=! a[M, K] * b[K, N]', inputs=['a=float32[M:40, K:24]', 'b=float32[K:24, N:36]'], name='gemm_f32_small')
     a2, b2 = torch.randn(40, 24, generator=g), torch.randn(24, 36, generator=g)
     assert torch.allclose(small(a2.to(dev), b2.to(dev)).cpu().double(), a2.double() @ b2.double(), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize('B,M,N,K', [(3, 1024, 512, 512), (5, 130, 1028, 64), (16, 256, 256, 128)])
+def test_batched_fp32_gemm_on_the_matrix_cores_matches_the_float64_products(autort, B, M, N, K):
+    """`C[B,M,N] +=! A[B,M,K] * B[B,K,N]` (AntaresIR.md:121, written there with other names) goes to
+    art_gemm_f32_batched: every product of the batch is the float64 product's to fp32 accuracy, and one batch with
+    all-zero operands stays zero (no product reads its neighbour's operands)."""
+    note(f'batched gemm_f32 {B}x{M}x{N}x{K}')
+    dev = autort.device()
+    op = autort.export(ir='output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]',
+                       inputs=[f'input0=float32[B:{B}, N:{M}, K:{K}]', f'input1=float32[B:{B}, K:{K}, M:{N}]'], name=f'bmm_f32_{B}_{M}_{N}_{K}')
+    assert op.fast_path is not None
+    g = torch.Generator().manual_seed(B + M + N + K)
+    a, b = torch.randn(B, M, K, generator=g), torch.randn(B, K, N, generator=g)
+    a[1].zero_()
+    got = op(a.to(dev), b.to(dev)).cpu()
+    want = a.double() @ b.double()
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5 * max(1.0, K ** 0.5)), (got.double() - want).abs().max()
+    assert not got[1].any() and got[0].any() and got[2].any()
