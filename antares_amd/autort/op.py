@@ -189,7 +189,9 @@ class ExportedOp:
         key = tuple(env[d] for d in self.fused.dim_names)
         v = self._variants.get(key)
         if v is None:
-            g = split_wide_reductions(self.lowered, env) if self.fused.dims else self.lowered
+            # rows that one row kernel reduces and maps in a single launch are not sliced
+            in_rows = any(p.row_group is not None and p.row_group.grid(env) for p in self.plans)
+            g = split_wide_reductions(self.lowered, env) if self.fused.dims and not in_rows else self.lowered
             if g is self.lowered:
                 v = {'graph': self.lowered, 'plans': self.plans, 'module': None, 'source': None}
             else:
@@ -207,7 +209,20 @@ class ExportedOp:
         dims = [env[d] for d in g.dim_names]
         trials = self.config.get('tune')
         trials = trials if isinstance(trials, int) and trials > 0 else 0
+        skip = 0
         for plan in plans_:
+            if skip:                       # computed by the row kernel of an earlier statement
+                skip -= 1
+                continue
+            group = plan.row_group
+            if group is not None and not trials and group.grid(env):
+                for n in group.args:
+                    if n not in bound:
+                        bound[n] = torch.empty(g.shape_of(n, env), dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)
+                capi.launch(module.function(group.kernel(env)), (group.grid(env), 1, 1), (256, 1, 1), stream,
+                            [bound[n].data_ptr() for n in group.args] + dims)
+                skip = group.count - 1
+                continue
             for n in plan.args:
                 if n not in bound:         # intermediate (reduce result) of a multi-kernel program
                     bound[n] = torch.empty(g.shape_of(n, env), dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)

@@ -21,7 +21,10 @@ templates:
   and by which axis is contiguous in memory (the reference reduces through LDS because its TVM patch
   disables wavefront shuffles off CUDA, engine/device-stub/tvm_v0.8.0.patch:186-191);
 * scatter statements: one thread per point of the iteration space, atomics for
-  ``+=.  <=.  >=.``.
+  ``+=.  <=.  >=.``;
+* runs of statements that reduce over the last axis of a row and then map over
+  the row with the results (softmax, layer normalisation) get, besides their
+  own kernels, one kernel that does the whole run with a block per row.
 
 Kernel signatures follow the reference's HIP kernel ABI
 (backends/c-rocm/config.py:25-85): tensor pointers first, in the order given by
@@ -126,6 +129,39 @@ class ExprEmitter:
 
 
 @dataclass
+class RowGroup:
+    """A run of statements that one kernel computes row by row: reductions over the last axis of a row followed by
+    the map that uses their results (softmax, layer normalisation, AntaresIR.md:226-232)."""
+    symbol: str
+    args: List[str]                # inputs (sorted), then the reduce results in statement order, then the map's output
+    count: int                     # statements covered, starting with the one that carries the group
+    row_axes: List[Tuple[str, object]]
+    red_axis: Tuple[str, object]
+    cached: Dict[int, str] = field(default_factory=dict)   # elements per thread -> kernel that keeps the row in registers
+
+    def kernel(self, env: Dict[str, int]) -> str:
+        """The kernel for these extents: the row in registers when it fits (read from memory once), else a walk
+        over the row per statement."""
+        e = self.red_axis[1]
+        n = e if isinstance(e, int) else env[e]
+        for per_thread in sorted(self.cached):
+            if n <= per_thread * BLOCK:
+                return self.cached[per_thread]
+        return self.symbol
+
+    def grid(self, env: Dict[str, int]) -> int:
+        """Blocks to launch for these extents (one per row, capped), 0 when the per-statement kernels do better:
+        rows shorter than half a block would leave most lanes idle."""
+        e = self.red_axis[1]
+        if (e if isinstance(e, int) else env[e]) < 128:
+            return 0
+        rows = 1
+        for _, e in self.row_axes:
+            rows *= e if isinstance(e, int) else env[e]
+        return min(rows, MAX_GRID)
+
+
+@dataclass
 class KernelPlan:
     """Everything the runtime needs to launch one statement."""
     name: str                      # base kernel name
@@ -146,6 +182,7 @@ class KernelPlan:
     patch_dims: List[object] = field(default_factory=list)   # the two extents (int or dimension name) it tiles
     tile_axes: Optional[Tuple[str, str]] = None   # permutation copies: last axis of the load, last axis of the store
     tile_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for the vector form of it
+    row_group: Optional[RowGroup] = None          # set on the first statement of a run that one row kernel can compute
 
     def _tiles(self, env: Dict[str, int]) -> int:
         """64 x 64 tiles of the transposing variant, 0 when it does not apply or an axis is too short to pay."""
@@ -746,6 +783,117 @@ def _reduce_axis_contiguous(st, tensors) -> Optional[bool]:
     return score > 0
 
 
+
+def _row_group_at(graph, i: int) -> int:
+    """Number of statements, starting at statement i, that form a row group (0: none): one or more reductions over
+    the same single axis R with the same data axes D, each result indexed by D, then a map over D + [R].  Later
+    statements of the group may read earlier results only at the row's own position."""
+    sts, tensors = graph.statements, graph.tensors
+    first = sts[i]
+    if first.scatter or len(first.reduce_axes) != 1 or not first.data_axes:
+        return 0
+    D, R = list(first.data_axes), first.reduce_axes[0]
+    d_names = [a for a, _ in D]
+    j, temps = i, []
+    while j < len(sts):
+        st = sts[j]
+        if st.scatter or list(st.reduce_axes) != [R] or list(st.data_axes) != D:
+            break
+        if [ix.name if ix.kind == 'axis' else None for ix in st.out_index] != d_names or st.output in temps:
+            return 0
+        if st.root.kind == 'when' and len(st.root.args) == 1:
+            return 0
+        temps.append(st.output)
+        j += 1
+    if not temps or j >= len(sts):
+        return 0
+    m = sts[j]
+    if m.scatter or m.reduce_axes or list(m.data_axes) != D + [R] or m.output in temps:
+        return 0
+    if [ix.name if ix.kind == 'axis' else None for ix in m.out_index] != d_names + [R[0]]:
+        return 0
+    if m.root.kind == 'when' and len(m.root.args) == 1:
+        return 0
+    if list(tensors[m.output].shape) != [e for _, e in D + [R]]:
+        return 0
+    for k in range(i, j + 1):
+        st = sts[k]
+        for n in walk(st.root):
+            if n.kind != 'load':
+                continue
+            if n.name == m.output or n.name == st.output:
+                return 0
+            if n.name in temps:
+                if temps.index(n.name) >= k - i or [a.name if a.kind == 'axis' else None for a in n.args] != d_names:
+                    return 0
+    return j + 1 - i
+
+
+def _lower_row_group(graph, i: int, count: int, sym: str) -> Tuple[str, RowGroup]:
+    """One block of 256 threads per row: every reduction meets in the block and its result stays in a register for
+    the statements that follow; reduce results are also stored, as the per-statement kernels would.  Rows of up to
+    1024 / 4096 elements are read once, all loads in flight together, and kept in registers (4 / 16 per thread);
+    longer rows are walked once per statement (the first walk brings the row from memory, the later ones find it
+    in cache)."""
+    sts, tensors, dims = graph.statements[i:i + count], graph.tensors, graph.dim_names
+    m = sts[-1]
+    D, (r_ax, r_ext) = list(sts[0].data_axes), sts[0].reduce_axes[0]
+    temps = [st.output for st in sts[:-1]]
+    written = temps + [m.output]
+    inputs = sorted({r for st in sts for r in st.reads} - set(written))
+    args = inputs + written
+    d_idx = [a for a, _ in D]
+
+    def is_row_load(n):
+        return n.name not in written and [a.name if a.kind == 'axis' else None for a in n.args] == d_idx + [r_ax]
+    row_tensors = sorted({n.name for st in sts for n in walk(st.root) if n.kind == 'load' and is_row_load(n)})
+
+    def emit(symbol: str, per_thread: int) -> str:
+        def override(n):
+            if n.name in temps:
+                return f'__t_{n.name}'
+            if per_thread and is_row_load(n):
+                return f'__c_{n.name}[__e]'
+            return None
+        em = ExprEmitter(tensors, load_override=override)
+        plain = ExprEmitter(tensors)
+        if per_thread:
+            walk_row = ['    #pragma unroll', f'    for (int __e = 0; __e < {per_thread}; ++__e) {{',
+                        f'      const int {r_ax} = threadIdx.x + {BLOCK} * __e;', f'      if ({r_ax} < __ext_{r_ax})']
+            close = ['    }']
+        else:
+            walk_row = ['    #pragma unroll 4', f'    for (int {r_ax} = threadIdx.x; {r_ax} < __ext_{r_ax}; {r_ax} += {BLOCK})']
+            close = []
+        body = [_signature(symbol, args, tensors, dims, written) + ' {'] + _extents(m)
+        body.append('  const long long __rows = ' + (' * '.join(f'(long long)__ext_{ax}' for ax, _ in D) or '1LL') + ';')
+        for st in sts[:-1]:
+            body.append(f'  __shared__ {HIP_TYPE[st.root.dtype]} __smem_{st.output}[4];')
+        body.append('  for (long long __o = blockIdx.x; __o < __rows; __o += gridDim.x) {')
+        body += _decompose('__o', D, '    ')
+        if per_thread:
+            for t in row_tensors:
+                body.append(f'    {HIP_TYPE[tensors[t].dtype]} __c_{t}[{per_thread}];')
+            body += walk_row + ['      {'] + [f'        __c_{t}[__e] = {t}[{plain.offset(t, d_idx + [r_ax])}];' for t in row_tensors] + ['      }'] + close
+        for st in sts[:-1]:
+            act, oct_ = HIP_TYPE[st.root.dtype], HIP_TYPE[st.out_dtype]
+            op = _REDUCE_OP[st.reduce] + '()'
+            body.append(f'    {act} __acc_{st.output} = {reduce_identity(st.reduce, st.root.dtype)};')
+            body += walk_row + [f'        __acc_{st.output} = {op}(__acc_{st.output}, ({act})({em.expr(st.root)}));'] + close
+            body += [f'    const {oct_} __t_{st.output} = ({oct_})art_block_reduce(__acc_{st.output}, {op}, __smem_{st.output});',
+                     f'    if (threadIdx.x == 0) {st.output}[{em.offset(st.output, d_idx)}] = __t_{st.output};']
+        body += walk_row + [f'        {m.output}[{em.offset(m.output, d_idx + [r_ax])}] = ({HIP_TYPE[m.out_dtype]})({em.expr(m.root)});'] + close
+        body += ['  }', '}']
+        return '\n'.join(body)
+
+    group = RowGroup(symbol=sym, args=args, count=count, row_axes=D, red_axis=(r_ax, r_ext))
+    code = [emit(sym, 0)]
+    if row_tensors:
+        for per_thread in (4, 16):
+            group.cached[per_thread] = f'{sym}_c{per_thread}'
+            code.append(emit(group.cached[per_thread], per_thread))
+    return '\n\n'.join(code), group
+
+
 def lower_graph(graph, prefix: str = 'autort') -> Tuple[str, List[KernelPlan]]:
     """Fused graph -> (HIP source text with container-format headers, plans).
 
@@ -762,8 +910,16 @@ def lower_graph(graph, prefix: str = 'autort') -> Tuple[str, List[KernelPlan]]:
         head += '// VAMAP: ' + ','.join(f'{d}:{v if v is not None else "?"}' for d, v in sorted(graph.dims.items())) + '\n'
     head += '// COMPUTE_V1: - einstein_v2(' + repr(' '.join(graph.source.split())) + ')\n'
     parts, plans = [head + PRELUDE], []
+    grouped_until = 0
     for i, st in enumerate(graph.statements):
         code, plan = lower_statement(st, graph, f'{prefix}_k{i}')
+        count = _row_group_at(graph, i) if i >= grouped_until else 0
+        if count:
+            # the row kernel travels with the first statement's kernels; the per-statement kernels stay for the
+            # extents it is not launched at
+            row_code, plan.row_group = _lower_row_group(graph, i, count, f'{prefix}_k{i}_rows')
+            code += '\n\n' + row_code
+            grouped_until = i + count
         ins = ', '.join(disp(n) for n in plan.args[:-1])
         parts.append(f'// LOCAL: {plan.name} -- {ins} -> {disp(plan.output)}\n\n{code}\n')
         plans.append(plan)

@@ -688,3 +688,67 @@ def test_batched_fp32_gemm_on_the_matrix_cores_matches_the_float64_products(auto
     want = a.double() @ b.double()
     assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5 * max(1.0, K ** 0.5)), (got.double() - want).abs().max()
     assert not got[1].any() and got[0].any() and got[2].any()
+
+
+ROW_GROUP_CASES = [
+    # program, inputs, shapes, does the row kernel run at these extents
+    ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
+     'output0[N, C] = (input0[N, C] - temp0[N]).call(`exp`) / temp1[N]', ['input0=float32[N:37, C:1000]'], [(37, 1000)], True),
+    ('temp0[N] +=! input0[N, C]; temp1[N] +=! input0[N, C] * input0[N, C]; '
+     'output0[N, C] = (input0[N, C] * C.val() - temp0[N]) * (temp1[N] * C.val() - temp0[N] * temp0[N] + 1e-5).call(`rsqrt`)',
+     ['input0=float32[N:32, C:1024]'], [(32, 1024)], True),
+    # rows of a 3-D tensor, a per-column weight and a per-row shift besides the row itself, fp16 storage
+    ('ss[B, N] +=! x[B, N, C].to(`float32`) * x[B, N, C].to(`float32`); '
+     'y[B, N, C] = (x[B, N, C].to(`float32`) * (ss[B, N] / C.val() + 1e-5).call(`rsqrt`) * w[C].to(`float32`) + shift[B, N]).to(`float16`)',
+     ['x=float16[B:3, N:17, C:520]', 'w=float16[C:520]', 'shift=float32[B:3, N:17]'], [(3, 17, 520), (520,), (3, 17)], True),
+    # integer rows: maximum and count of the maxima, exact
+    ('top[N] >=! v[N, C]; hits[N] +=! (v[N, C] == top[N]).to(`int32`); out[N, C] = (top[N] - v[N, C]) * hits[N]',
+     ['v=int32[N:50, C:300]'], [(50, 300)], True),
+    # short rows: the per-statement kernels run, same result
+    ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
+     'output0[N, C] = (input0[N, C] - temp0[N]).call(`exp`) / temp1[N]', ['input0=float32[N:300, C:64]'], [(300, 64)], False),
+]
+
+
+@pytest.mark.parametrize('ir,inputs,shapes,applies', ROW_GROUP_CASES)
+def test_row_reductions_and_their_map_run_as_one_kernel(autort, ir, inputs, shapes, applies):
+    """Reductions over the last axis followed by the map that uses them (softmax, layer normalisation,
+    AntaresIR.md:226-232) are computed by one kernel, a block per row; results are the oracle's, and they equal
+    what the per-statement kernels give to the rounding of the reductions."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'row group {ir[:40]} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='rows_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    group = op.plans[0].row_group
+    assert group is not None and group.count == len(op.plans) == ir.count(';') + 1
+    env = {}
+    for spec, shape in zip(inputs, shapes):
+        for d, v in zip(spec.split('[', 1)[1].rstrip(']').split(','), shape):
+            env[d.split(':')[0].strip()] = v
+    assert (group.grid(env) > 0) == applies
+    g = torch.Generator().manual_seed(len(ir))
+    tensors, names = [], []
+    for spec, shape in zip(inputs, shapes):
+        name, rest = spec.split('=')
+        names.append(name)
+        if rest.startswith('int32'):
+            tensors.append(torch.randint(-40, 40, shape, generator=g, dtype=torch.int32))
+        else:
+            tensors.append(torch.randn(shape, generator=g).to(torch.float16 if rest.startswith('float16') else torch.float32))
+    got = op(*[t.to(dev) for t in tensors]).cpu().numpy()
+    out_name = ir.rsplit(';', 1)[1].split('[', 1)[0].strip()
+    want = CpuModule(parse_program(ir, inputs), fast_math=False)(**{n: t.numpy() for n, t in zip(names, tensors)})[out_name]
+    if got.dtype.kind == 'i':
+        assert np.array_equal(got, want)
+    else:
+        tol = 2e-2 if got.dtype == np.float16 else 2e-5
+        assert np.allclose(got.astype(np.float64), want.astype(np.float64), rtol=tol, atol=tol), np.abs(got.astype(np.float64) - want).max()
+    # statement by statement (the row kernel switched off): same values up to the order of the sums
+    for p in op.plans:
+        p.row_group = None
+    apart = op(*[t.to(dev) for t in tensors]).cpu().numpy()
+    if got.dtype.kind == 'i':
+        assert np.array_equal(got, apart)
+    else:
+        assert np.allclose(got.astype(np.float64), apart.astype(np.float64), rtol=tol, atol=tol)
