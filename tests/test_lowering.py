@@ -1,0 +1,59 @@
+"""Decisions the generic lowering takes from the text of a program alone (no GPU): which statements one row kernel
+may cover, and that the generated source compiles for gfx950."""
+import pytest
+
+from antares_amd.ir import parse_program
+from antares_amd.ir.graph import fuse_elementwise
+from antares_amd.lower import hip_codegen
+
+SOFTMAX = ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
+           'output0[N, C] = (input0[N, C] - temp0[N]).call(`exp`) / temp1[N]')
+
+
+def lowered(ir, inputs):
+    return hip_codegen.lower_graph(fuse_elementwise(parse_program(ir, inputs)))
+
+
+def test_softmax_is_one_row_group_with_kernels_for_short_and_long_rows():
+    src, plans = lowered(SOFTMAX, ['input0=float32[N:32, C:1024]'])
+    group = plans[0].row_group
+    assert group is not None and group.count == 3 and plans[1].row_group is None and plans[2].row_group is None
+    assert group.args == ['input0', 'temp0', 'temp1', 'output0']
+    assert group.red_axis[0] == 'C' and [a for a, _ in group.row_axes] == ['N']
+    # rows of up to 1024 / 4096 elements stay in registers, longer ones are walked; short rows are left alone
+    assert group.kernel({'N': 32, 'C': 1024}) == group.cached[4]
+    assert group.kernel({'N': 32, 'C': 1025}) == group.cached[16]
+    assert group.kernel({'N': 32, 'C': 4097}) == group.symbol
+    assert group.grid({'N': 32, 'C': 1024}) == 32 and group.grid({'N': 32, 'C': 127}) == 0
+    assert group.grid({'N': 10 ** 6, 'C': 1024}) == hip_codegen.MAX_GRID
+    for sym in [group.symbol] + list(group.cached.values()):
+        assert f'void {sym}(' in src
+
+
+@pytest.mark.parametrize('ir,inputs', [
+    # the map reads a result at another row's position
+    ('t[N] +=! x[N, C]; y[N, C] = x[N, C] - t[(N + 1) % 8]', ['x=float32[N:8, C:256]']),
+    # the reduction runs over the first axis: rows are not contiguous runs of its operand's last axis, and the map's
+    # axes are not (data axes + reduce axis) in that order
+    ('t[C] +=! x[N, C]; y[N, C] = x[N, C] - t[C]', ['x=float32[N:8, C:256]']),
+    # the map is over other axes than the reductions
+    ('t[N] +=! x[N, C]; y[N, K] = z[N, K] - t[N]', ['x=float32[N:8, C:256]', 'z=float32[N:8, K:256]']),
+    # a map that stores only where a condition holds
+    ('t[N] +=! x[N, C]; y[N, C] = (x[N, C] - t[N]).when([x[N, C] > 0])', ['x=float32[N:8, C:256]', 'y=float32[N:8, C:256]']),
+    # a reduction alone, and a map alone
+    ('t[N] +=! x[N, C]', ['x=float32[N:8, C:256]']),
+    ('y[N, C] = x[N, C] * 2', ['x=float32[N:8, C:256]']),
+])
+def test_programs_that_are_no_row_group(ir, inputs):
+    _, plans = lowered(ir, inputs)
+    assert all(p.row_group is None for p in plans)
+
+
+def test_row_kernels_compile_for_gfx950(tmp_path, monkeypatch):
+    monkeypatch.setenv('AUTORT_CACHE_DIR', str(tmp_path / 'cache'))
+    from antares_amd.autort.op import compile_cached
+    ir = ('ss[B, N] +=! x[B, N, C].to(`float32`) * x[B, N, C].to(`float32`); '
+          'y[B, N, C] = (x[B, N, C].to(`float32`) * (ss[B, N] / C.val() + 1e-5).call(`rsqrt`) * w[C].to(`float32`)).to(`float16`)')
+    src, plans = lowered(ir, ['x=float16[B:3, N:17, C:520]', 'w=float16[C:520]'])
+    assert plans[0].row_group is not None and plans[0].row_group.count == 2
+    assert len(compile_cached(src)) > 1000
