@@ -190,7 +190,7 @@ class ExportedOp:
         v = self._variants.get(key)
         if v is None:
             # rows that one row kernel reduces and maps in a single launch are not sliced
-            in_rows = any(p.row_group is not None and p.row_group.grid(env) for p in self.plans)
+            in_rows = any(p.row_group is not None and p.row_group.choose(env, {n: 0 for n in p.row_group.args})[1] for p in self.plans)
             g = split_wide_reductions(self.lowered, env) if self.fused.dims and not in_rows else self.lowered
             if g is self.lowered:
                 v = {'graph': self.lowered, 'plans': self.plans, 'module': None, 'source': None}
@@ -215,14 +215,15 @@ class ExportedOp:
                 skip -= 1
                 continue
             group = plan.row_group
-            if group is not None and not trials and group.grid(env):
+            if group is not None and not trials:
                 for n in group.args:
                     if n not in bound:
                         bound[n] = torch.empty(g.shape_of(n, env), dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)
-                capi.launch(module.function(group.kernel(env)), (group.grid(env), 1, 1), (256, 1, 1), stream,
-                            [bound[n].data_ptr() for n in group.args] + dims)
-                skip = group.count - 1
-                continue
+                sym, grid = group.choose(env, {n: bound[n].data_ptr() for n in group.args})
+                if grid:
+                    capi.launch(module.function(sym), (grid, 1, 1), (256, 1, 1), stream, [bound[n].data_ptr() for n in group.args] + dims)
+                    skip = group.count - 1
+                    continue
             for n in plan.args:
                 if n not in bound:         # intermediate (reduce result) of a multi-kernel program
                     bound[n] = torch.empty(g.shape_of(n, env), dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)

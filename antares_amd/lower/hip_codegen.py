@@ -132,33 +132,46 @@ class ExprEmitter:
 class RowGroup:
     """A run of statements that one kernel computes row by row: reductions over the last axis of a row followed by
     the map that uses their results (softmax, layer normalisation, AntaresIR.md:226-232)."""
-    symbol: str
+    symbol: str                    # the kernel for rows of any length: a block per row, the row walked per statement
     args: List[str]                # inputs (sorted), then the reduce results in statement order, then the map's output
     count: int                     # statements covered, starting with the one that carries the group
     row_axes: List[Tuple[str, object]]
     red_axis: Tuple[str, object]
-    cached: Dict[int, str] = field(default_factory=dict)   # elements per thread -> kernel that keeps the row in registers
+    # kernels that keep the row in registers: (lanes per row: 64 or 256, elements per vector, vectors per lane, symbol)
+    cached: List[Tuple[int, int, int, str]] = field(default_factory=list)
+    vec_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for the vector kernels
 
-    def kernel(self, env: Dict[str, int]) -> str:
-        """The kernel for these extents: the row in registers when it fits (read from memory once), else a walk
-        over the row per statement."""
+    def _extents(self, env: Dict[str, int]) -> Tuple[int, int]:
         e = self.red_axis[1]
         n = e if isinstance(e, int) else env[e]
-        for per_thread in sorted(self.cached):
-            if n <= per_thread * BLOCK:
-                return self.cached[per_thread]
-        return self.symbol
-
-    def grid(self, env: Dict[str, int]) -> int:
-        """Blocks to launch for these extents (one per row, capped), 0 when the per-statement kernels do better:
-        rows shorter than half a block would leave most lanes idle."""
-        e = self.red_axis[1]
-        if (e if isinstance(e, int) else env[e]) < 128:
-            return 0
         rows = 1
         for _, e in self.row_axes:
             rows *= e if isinstance(e, int) else env[e]
-        return min(rows, MAX_GRID)
+        return rows, n
+
+    def choose(self, env: Dict[str, int], pointers: Dict[str, int]) -> Tuple[str, int]:
+        """-> (kernel symbol, grid.x) for these extents and addresses; grid 0 when the per-statement kernels do
+        better (rows shorter than two wavefronts leave most lanes idle).  Among the kernels that hold a row of this
+        length in registers: 16-byte vectors when the row length and the addresses allow, a wavefront per row when
+        there are enough rows to fill the chip that way (no barriers), else a block per row."""
+        rows, n = self._extents(env)
+        if n < 128 or rows == 0:
+            return self.symbol, 0
+        aligned = all(pointers[t] % 16 == 0 for t in self.vec_tensors)
+        fits = [(team, v, e, sym) for team, v, e, sym in self.cached
+                if n <= team * v * e and (v == 1 or (aligned and n % v == 0))]
+        if not fits:
+            return self.symbol, min(rows, MAX_GRID)
+        vmax = max(v for _, v, _, _ in fits)
+        fits = [f for f in fits if f[1] == vmax]
+        waves = [f for f in fits if f[0] == 64]
+        if waves and rows >= 8192:
+            pick = min(waves, key=lambda f: f[2])
+        else:
+            blocks = [f for f in fits if f[0] == BLOCK] or fits
+            pick = min(blocks, key=lambda f: f[2])
+        per_block = BLOCK // pick[0]
+        return pick[3], min((rows + per_block - 1) // per_block, MAX_GRID)
 
 
 @dataclass
@@ -830,11 +843,11 @@ def _row_group_at(graph, i: int) -> int:
 
 
 def _lower_row_group(graph, i: int, count: int, sym: str) -> Tuple[str, RowGroup]:
-    """One block of 256 threads per row: every reduction meets in the block and its result stays in a register for
-    the statements that follow; reduce results are also stored, as the per-statement kernels would.  Rows of up to
-    1024 / 4096 elements are read once, all loads in flight together, and kept in registers (4 / 16 per thread);
-    longer rows are walked once per statement (the first walk brings the row from memory, the later ones find it
-    in cache)."""
+    """Kernels that compute the whole run row by row.  Every reduction meets in the row's team of lanes (a block of
+    256 or one wavefront) and its result stays in a register for the statements that follow; reduce results are
+    also stored, as the per-statement kernels would.  Where a row fits, it is read once, all loads in flight
+    together, and kept in registers (4 or 16 vectors of 1 or 16 bytes per lane); longer rows are walked once per
+    statement by a block (the first walk brings the row from memory, the later ones find it in cache)."""
     sts, tensors, dims = graph.statements[i:i + count], graph.tensors, graph.dim_names
     m = sts[-1]
     D, (r_ax, r_ext) = list(sts[0].data_axes), sts[0].reduce_axes[0]
@@ -843,54 +856,96 @@ def _lower_row_group(graph, i: int, count: int, sym: str) -> Tuple[str, RowGroup
     inputs = sorted({r for st in sts for r in st.reads} - set(written))
     args = inputs + written
     d_idx = [a for a, _ in D]
+    oct_m = HIP_TYPE[m.out_dtype]
 
     def is_row_load(n):
         return n.name not in written and [a.name if a.kind == 'axis' else None for a in n.args] == d_idx + [r_ax]
     row_tensors = sorted({n.name for st in sts for n in walk(st.root) if n.kind == 'load' and is_row_load(n)})
+    vmax = 16 // max(ITEMSIZE[tensors[t].dtype] for t in row_tensors + [m.output])
+    plain = ExprEmitter(tensors)
 
-    def emit(symbol: str, per_thread: int) -> str:
+    def emit(symbol: str, team: int, V: int, E: int) -> str:
+        """team lanes per row, E vectors of V elements per lane held in registers (E == 0: the row is walked)."""
         def override(n):
             if n.name in temps:
                 return f'__t_{n.name}'
-            if per_thread and is_row_load(n):
-                return f'__c_{n.name}[__e]'
+            if E and is_row_load(n):
+                return f'__c_{n.name}[__e]' + ('[__k]' if V > 1 else '')
             return None
         em = ExprEmitter(tensors, load_override=override)
-        plain = ExprEmitter(tensors)
-        if per_thread:
-            walk_row = ['    #pragma unroll', f'    for (int __e = 0; __e < {per_thread}; ++__e) {{',
-                        f'      const int {r_ax} = threadIdx.x + {BLOCK} * __e;', f'      if ({r_ax} < __ext_{r_ax})']
-            close = ['    }']
-        else:
-            walk_row = ['    #pragma unroll 4', f'    for (int {r_ax} = threadIdx.x; {r_ax} < __ext_{r_ax}; {r_ax} += {BLOCK})']
-            close = []
+        lane = 'threadIdx.x' if team == BLOCK else '(threadIdx.x & 63)'
+
+        def over_row(per_chunk_before, per_element, per_chunk_after):
+            """Loop over this lane's share of the row: chunk-level lines, then element-level lines inside."""
+            out = []
+            if E:
+                out += ['    #pragma unroll', f'    for (int __e = 0; __e < {E}; ++__e) {{',
+                        f'      const int __r0 = ({lane} + {team} * __e) * {V};', f'      if (__r0 < __ext_{r_ax}) {{']
+                ind = '        '
+            else:
+                out += ['    #pragma unroll 4', f'    for (int __r0 = {lane}; __r0 < __ext_{r_ax}; __r0 += {team}) {{', '      {']
+                ind = '        '
+            out += [ind + l for l in per_chunk_before]
+            if per_element:
+                if V > 1:
+                    out += [ind + '#pragma unroll', ind + f'for (int __k = 0; __k < {V}; ++__k) {{',
+                            ind + f'  const int {r_ax} = __r0 + __k; (void){r_ax};'] + [ind + '  ' + l for l in per_element] + [ind + '}']
+                else:
+                    out += [ind + f'const int {r_ax} = __r0; (void){r_ax};'] + [ind + l for l in per_element]
+            out += [ind + l for l in per_chunk_after]
+            out += ['      }', '    }']
+            return out
+
         body = [_signature(symbol, args, tensors, dims, written) + ' {'] + _extents(m)
         body.append('  const long long __rows = ' + (' * '.join(f'(long long)__ext_{ax}' for ax, _ in D) or '1LL') + ';')
-        for st in sts[:-1]:
-            body.append(f'  __shared__ {HIP_TYPE[st.root.dtype]} __smem_{st.output}[4];')
-        body.append('  for (long long __o = blockIdx.x; __o < __rows; __o += gridDim.x) {')
-        body += _decompose('__o', D, '    ')
-        if per_thread:
+        if V > 1:
             for t in row_tensors:
-                body.append(f'    {HIP_TYPE[tensors[t].dtype]} __c_{t}[{per_thread}];')
-            body += walk_row + ['      {'] + [f'        __c_{t}[__e] = {t}[{plain.offset(t, d_idx + [r_ax])}];' for t in row_tensors] + ['      }'] + close
+                body.append(f'  typedef {HIP_TYPE[tensors[t].dtype]} __vec_{t} __attribute__((ext_vector_type({V})));')
+            body.append(f'  typedef {oct_m} __vec_out __attribute__((ext_vector_type({V})));')
+        if team == BLOCK:
+            for st in sts[:-1]:
+                body.append(f'  __shared__ {HIP_TYPE[st.root.dtype]} __smem_{st.output}[4];')
+            body.append('  for (long long __o = blockIdx.x; __o < __rows; __o += gridDim.x) {')
+        else:
+            per_block = BLOCK // team
+            body.append(f'  for (long long __o = (long long)blockIdx.x * {per_block} + (threadIdx.x >> 6); __o < __rows; '
+                        f'__o += (long long)gridDim.x * {per_block}) {{')
+        body += _decompose('__o', D, '    ')
+        if E:
+            for t in row_tensors:
+                ct = f'__vec_{t}' if V > 1 else HIP_TYPE[tensors[t].dtype]
+                body.append(f'    {ct} __c_{t}[{E}];')
+            loads = []
+            for t in row_tensors:
+                off = plain.offset(t, d_idx + ['__r0'])
+                loads.append(f'__c_{t}[__e] = ' + (f'*(const __vec_{t}*)&{t}[{off}];' if V > 1 else f'{t}[{off}];'))
+            body += over_row(loads, [], [])
         for st in sts[:-1]:
             act, oct_ = HIP_TYPE[st.root.dtype], HIP_TYPE[st.out_dtype]
             op = _REDUCE_OP[st.reduce] + '()'
             body.append(f'    {act} __acc_{st.output} = {reduce_identity(st.reduce, st.root.dtype)};')
-            body += walk_row + [f'        __acc_{st.output} = {op}(__acc_{st.output}, ({act})({em.expr(st.root)}));'] + close
-            body += [f'    const {oct_} __t_{st.output} = ({oct_})art_block_reduce(__acc_{st.output}, {op}, __smem_{st.output});',
-                     f'    if (threadIdx.x == 0) {st.output}[{em.offset(st.output, d_idx)}] = __t_{st.output};']
-        body += walk_row + [f'        {m.output}[{em.offset(m.output, d_idx + [r_ax])}] = ({HIP_TYPE[m.out_dtype]})({em.expr(m.root)});'] + close
+            body += over_row([], [f'__acc_{st.output} = {op}(__acc_{st.output}, ({act})({em.expr(st.root)}));'], [])
+            meet = (f'art_block_reduce(__acc_{st.output}, {op}, __smem_{st.output})' if team == BLOCK
+                    else f'art_wave_reduce(__acc_{st.output}, {op})')
+            body += [f'    const {oct_} __t_{st.output} = ({oct_}){meet};',
+                     f'    if ({lane} == 0) {st.output}[{em.offset(st.output, d_idx)}] = __t_{st.output};']
+        if V > 1:
+            body += over_row(['__vec_out __out;'], [f'__out[__k] = ({oct_m})({em.expr(m.root)});'],
+                             [f'*(__vec_out*)&{m.output}[{plain.offset(m.output, d_idx + ["__r0"])}] = __out;'])
+        else:
+            body += over_row([], [f'{m.output}[{em.offset(m.output, d_idx + [r_ax])}] = ({oct_m})({em.expr(m.root)});'], [])
         body += ['  }', '}']
         return '\n'.join(body)
 
     group = RowGroup(symbol=sym, args=args, count=count, row_axes=D, red_axis=(r_ax, r_ext))
-    code = [emit(sym, 0)]
+    code = [emit(sym, BLOCK, 1, 0)]
     if row_tensors:
-        for per_thread in (4, 16):
-            group.cached[per_thread] = f'{sym}_c{per_thread}'
-            code.append(emit(group.cached[per_thread], per_thread))
+        group.vec_tensors = sorted(set(row_tensors) | {m.output})
+        for V in sorted({1, vmax}):
+            for team, E in ((64, 4), (BLOCK, 4), (BLOCK, 16)):
+                name = f'{sym}_{"w" if team == 64 else "b"}{E}' + (f'v{V}' if V > 1 else '')
+                group.cached.append((team, V, E, name))
+                code.append(emit(name, team, V, E))
     return '\n\n'.join(code), group
 
 

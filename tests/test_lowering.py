@@ -20,13 +20,23 @@ def test_softmax_is_one_row_group_with_kernels_for_short_and_long_rows():
     assert group is not None and group.count == 3 and plans[1].row_group is None and plans[2].row_group is None
     assert group.args == ['input0', 'temp0', 'temp1', 'output0']
     assert group.red_axis[0] == 'C' and [a for a, _ in group.row_axes] == ['N']
-    # rows of up to 1024 / 4096 elements stay in registers, longer ones are walked; short rows are left alone
-    assert group.kernel({'N': 32, 'C': 1024}) == group.cached[4]
-    assert group.kernel({'N': 32, 'C': 1025}) == group.cached[16]
-    assert group.kernel({'N': 32, 'C': 4097}) == group.symbol
-    assert group.grid({'N': 32, 'C': 1024}) == 32 and group.grid({'N': 32, 'C': 127}) == 0
-    assert group.grid({'N': 10 ** 6, 'C': 1024}) == hip_codegen.MAX_GRID
-    for sym in [group.symbol] + list(group.cached.values()):
+    kernels = {(team, v, e): sym for team, v, e, sym in group.cached}
+    assert set(kernels) == {(64, 1, 4), (256, 1, 4), (256, 1, 16), (64, 4, 4), (256, 4, 4), (256, 4, 16)}
+    assert group.vec_tensors == ['input0', 'output0']
+    zero, odd = {n: 0 for n in group.args}, {**{n: 0 for n in group.args}, 'input0': 4}
+    # a block per row and 16-byte vectors where the row length and the addresses allow
+    assert group.choose({'N': 32, 'C': 1024}, zero) == (kernels[(256, 4, 4)], 32)
+    assert group.choose({'N': 32, 'C': 1024}, odd) == (kernels[(256, 1, 4)], 32)
+    assert group.choose({'N': 32, 'C': 1022}, zero) == (kernels[(256, 1, 4)], 32)
+    assert group.choose({'N': 32, 'C': 4100}, zero) == (kernels[(256, 4, 16)], 32)
+    assert group.choose({'N': 32, 'C': 4099}, zero) == (group.symbol, 32)           # too long for registers: walked
+    assert group.choose({'N': 32, 'C': 16388}, zero) == (group.symbol, 32)
+    # many short rows: a wavefront per row, four rows per block
+    assert group.choose({'N': 65536, 'C': 256}, zero) == (kernels[(64, 4, 4)], hip_codegen.MAX_GRID)
+    assert group.choose({'N': 10001, 'C': 250}, zero) == (kernels[(64, 1, 4)], 2501)
+    # rows shorter than two wavefronts are left to the per-statement kernels
+    assert group.choose({'N': 32, 'C': 127}, zero)[1] == 0
+    for sym in [group.symbol] + list(kernels.values()):
         assert f'void {sym}(' in src
 
 
