@@ -714,6 +714,9 @@ ROW_GROUP_CASES = [
     ('temp0[N] +=! input0[N, C]; temp1[N] +=! input0[N, C] * input0[N, C]; '
      'output0[N, C] = (input0[N, C] * C.val() - temp0[N]) * (temp1[N] * C.val() - temp0[N] * temp0[N] + 1e-5).call(`rsqrt`)',
      ['input0=float32[N:9, C:12000]'], [(9, 12000)], True),
+    # reductions with no map behind them: row sums, an integer row maximum of products with a weight row
+    ('output0[N] +=! input0[N, C]', ['input0=float32[N:600, C:1000]'], [(600, 1000)], True),
+    ('top[B, N] >=! v[B, N, C] * w[C]', ['v=int32[B:2, N:300, C:300]', 'w=int32[C:300]'], [(2, 300, 300), (300,)], True),
     # short rows: the per-statement kernels run, same result
     ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
      'output0[N, C] = (input0[N, C] - temp0[N]).call(`exp`) / temp1[N]', ['input0=float32[N:300, C:64]'], [(300, 64)], False),
@@ -747,7 +750,7 @@ def test_row_reductions_and_their_map_run_as_one_kernel(autort, ir, inputs, shap
         else:
             tensors.append(torch.randn(shape, generator=g).to(torch.float16 if rest.startswith('float16') else torch.float32))
     got = op(*[t.to(dev) for t in tensors]).cpu().numpy()
-    out_name = ir.rsplit(';', 1)[1].split('[', 1)[0].strip()
+    out_name = ir.rsplit(';', 1)[-1].split('[', 1)[0].strip()
     want = CpuModule(parse_program(ir, inputs), fast_math=False)(**{n: t.numpy() for n, t in zip(names, tensors)})[out_name]
     if got.dtype.kind == 'i':
         assert np.array_equal(got, want)

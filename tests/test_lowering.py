@@ -40,23 +40,40 @@ def test_softmax_is_one_row_group_with_kernels_for_short_and_long_rows():
         assert f'void {sym}(' in src
 
 
-@pytest.mark.parametrize('ir,inputs', [
-    # the map reads a result at another row's position
-    ('t[N] +=! x[N, C]; y[N, C] = x[N, C] - t[(N + 1) % 8]', ['x=float32[N:8, C:256]']),
-    # the reduction runs over the first axis: rows are not contiguous runs of its operand's last axis, and the map's
-    # axes are not (data axes + reduce axis) in that order
-    ('t[C] +=! x[N, C]; y[N, C] = x[N, C] - t[C]', ['x=float32[N:8, C:256]']),
-    # the map is over other axes than the reductions
-    ('t[N] +=! x[N, C]; y[N, K] = z[N, K] - t[N]', ['x=float32[N:8, C:256]', 'z=float32[N:8, K:256]']),
+@pytest.mark.parametrize('ir,inputs,covered', [
+    # the map reads a result at another row's position: the reduction alone is a group
+    ('t[N] +=! x[N, C]; y[N, C] = x[N, C] - t[(N + 1) % 8]', ['x=float32[N:8, C:256]'], 1),
+    # the map is over other axes than the reduction
+    ('t[N] +=! x[N, C]; y[N, K] = z[N, K] - t[N]', ['x=float32[N:8, C:256]', 'z=float32[N:8, K:256]'], 1),
     # a map that stores only where a condition holds
-    ('t[N] +=! x[N, C]; y[N, C] = (x[N, C] - t[N]).when([x[N, C] > 0])', ['x=float32[N:8, C:256]', 'y=float32[N:8, C:256]']),
-    # a reduction alone, and a map alone
-    ('t[N] +=! x[N, C]', ['x=float32[N:8, C:256]']),
-    ('y[N, C] = x[N, C] * 2', ['x=float32[N:8, C:256]']),
+    ('t[N] +=! x[N, C]; y[N, C] = (x[N, C] - t[N]).when([x[N, C] > 0])', ['x=float32[N:8, C:256]', 'y=float32[N:8, C:256]'], 1),
+    # a reduction alone; two of them; an offset in front of the reduced axis
+    ('t[N] +=! x[N, C]', ['x=float32[N:8, C:256]'], 1),
+    ('t[N] +=! x[N, C]; u[N] >=! x[N, C] * t[N]', ['x=float32[N:8, C:256]'], 2),
+    ('t[S] +=! x[S * 1024 + C] where C in 1024, S in 8', ['x=float32[N:8192]'], 1),
+    # the reduction runs over the first axis: lanes of a team would read addresses a row apart
+    ('t[C] +=! x[N, C]; y[N, C] = x[N, C] - t[C]', ['x=float32[N:8, C:256]'], 0),
+    ('t[N] +=! x[C, N]', ['x=float32[C:256, N:8]'], 0),
+    # a map alone
+    ('y[N, C] = x[N, C] * 2', ['x=float32[N:8, C:256]'], 0),
 ])
-def test_programs_that_are_no_row_group(ir, inputs):
+def test_which_statements_a_row_group_covers(ir, inputs, covered):
     _, plans = lowered(ir, inputs)
-    assert all(p.row_group is None for p in plans)
+    group = plans[0].row_group
+    if covered == 0:
+        assert all(p.row_group is None for p in plans)
+    else:
+        assert group is not None and group.count == covered and group.pure
+        zero = {n: 0 for n in group.args}
+        # reductions alone: with enough rows to fill the chip, or when all of it is one short launch out of
+        # registers; few long rows are left alone (they are sliced first)
+        assert group.choose({'N': 8, 'C': 256, 'K': 256, 'S': 8}, zero)[1] > 0
+        if 'S * 1024' not in ir:
+            assert group.choose({'N': 8, 'C': 65536, 'K': 256}, zero)[1] == 0
+            assert group.choose({'N': 100, 'C': 4096, 'K': 256}, zero)[1] == 0
+            assert group.choose({'N': 512, 'C': 4096, 'K': 256}, zero)[1] == 512
+    if 'S * 1024' in ir:
+        assert [sym for team, v, e, sym in group.cached if (team, v, e) == (64, 4, 4)]   # the offset 1024 S keeps rows 16-byte aligned
 
 
 def test_row_kernels_compile_for_gfx950(tmp_path, monkeypatch):
