@@ -215,7 +215,7 @@ class ExportedOp:
                 skip -= 1
                 continue
             group = plan.row_group
-            if group is not None and not trials:
+            if group is not None:
                 for n in group.args:
                     if n not in bound:
                         bound[n] = torch.empty(g.shape_of(n, env), dtype=TORCH_DTYPE[g.tensors[n].dtype], device=dev)
