@@ -161,6 +161,8 @@ class RowGroup:
         aligned = all(pointers[t] % 16 == 0 for t in self.vec_tensors)
         fits = [(team, v, e, sym) for team, v, e, sym in self.cached
                 if n <= team * v * e and (v == 1 or (aligned and n % v == 0))]
+        if not self.pure and rows < 64 and n > 65536:
+            return self.symbol, 0          # a handful of very long rows: too few blocks; the statements run one by one
         if self.pure and rows < 512 and not (fits and rows * n <= 65536):
             # few long rows: slicing them first (split_wide_reductions) fills the chip; what is left of a sliced
             # reduction - a few rows that fit in registers - is one short launch with every load in flight

@@ -34,7 +34,8 @@ def test_softmax_is_one_row_group_with_kernels_for_short_and_long_rows():
     # many short rows: a wavefront per row, four rows per block
     assert group.choose({'N': 65536, 'C': 256}, zero) == (kernels[(64, 4, 4)], hip_codegen.MAX_GRID)
     assert group.choose({'N': 10001, 'C': 250}, zero) == (kernels[(64, 1, 4)], 2501)
-    # rows shorter than two wavefronts are left to the per-statement kernels
+    # a handful of very long rows, and rows shorter than two wavefronts, are left to the per-statement kernels
+    assert group.choose({'N': 8, 'C': 1 << 20}, zero)[1] == 0 and group.choose({'N': 64, 'C': 1 << 20}, zero)[1] == 64
     assert group.choose({'N': 32, 'C': 127}, zero)[1] == 0
     for sym in [group.symbol] + list(kernels.values()):
         assert f'void {sym}(' in src
