@@ -232,3 +232,25 @@ def _batch_gemm_f32_handler(op, bound, env, stream) -> bool:
 
 
 register(BATCH_GEMM_F32_IR, BATCH_GEMM_F32_INPUTS, _batch_gemm_f32_handler)
+
+
+# ---------------------------------------------------------------------------
+# fp32 GEMM with an operand stored the other way round: A as [K, M], B as [N, K] (a linear layer's weight)
+# ---------------------------------------------------------------------------
+def _gemm_f32_layout_handler(trans_a: bool, trans_b: bool):
+    def handler(op, bound, env, stream) -> bool:
+        r = op.fast_roles
+        a, b, c = bound[r['a']], bound[r['b']], bound[r['c']]
+        (K, M) = a.shape if trans_a else a.shape[::-1]
+        N = b.shape[0] if trans_b else b.shape[1]
+        if K % 32 or (not trans_b and N % 4) or (trans_a and M % 4) or M * N < 128 * 128 * 32 or a.data_ptr() % 16 or b.data_ptr() % 16:
+            return False
+        capi.check(capi.lib().art_gemm_f32_ex(c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()), 1, M, N, K,
+                                             int(trans_a), int(trans_b), c_void_p(stream)))
+        return True
+    return handler
+
+
+register('c[M, N] +=! a[K, M] * b[K, N]', ['a=float32[K:512, M:512]', 'b=float32[K:512, N:512]'], _gemm_f32_layout_handler(True, False))
+register('c[M, N] +=! a[M, K] * b[N, K]', ['a=float32[M:512, K:512]', 'b=float32[N:512, K:512]'], _gemm_f32_layout_handler(False, True))
+register('c[M, N] +=! a[K, M] * b[N, K]', ['a=float32[K:512, M:512]', 'b=float32[N:512, K:512]'], _gemm_f32_layout_handler(True, True))

@@ -23,7 +23,10 @@
 //     instructions - issued in bursts they fill the LDS queues and the matrix pipe waits (measured at 4096^3:
 //     126 -> 141 TFLOP/s);
 //   * block -> tile mapping is XCD aware (a contiguous run of tiles per XCD, walked in 4 x 8 super-tiles);
-//   * C leaves straight from the accumulators: 32 lanes write 128 contiguous bytes of a row.
+//   * C leaves straight from the accumulators: 32 lanes write 128 contiguous bytes of a row;
+//   * the kernel is a template over the layouts of A ([M][K] or [K][M]) and B ([K][N] or [N][K]): an operand is
+//     staged in LDS as it lies in memory and read with a 16-byte vector where k is its contiguous axis, with four
+//     4-byte reads where it is not.
 #include "art_common.h"
 
 namespace {
@@ -33,14 +36,22 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 128, BN = 128, BK = 32, LD = BK + 4, LDB = BN + 8;
 constexpr int kThreads = 256;
-constexpr int TILE = BM * LD, TILE_B = BK * LDB;    // floats per operand tile in LDS
-constexpr size_t kLdsBytes = (size_t)2 * (TILE + TILE_B) * sizeof(float);     // A and B, two buffers each: 71680
+// An operand tile in LDS: 128 rows (m or n) of 32 k when k is the contiguous axis in memory ([x][k], pitch LD), 32 rows
+// of 128 m or n when it is not ([k][x], pitch LDB) - either way as it lies in memory.
+constexpr int TILE_XK = BM * LD, TILE_KX = BK * LDB;
+constexpr int kMaxTile = TILE_XK > TILE_KX ? TILE_XK : TILE_KX;
+template <bool TA, bool TB> constexpr size_t lds_bytes() {
+  return (size_t)2 * ((TA ? TILE_KX : TILE_XK) + (TB ? TILE_XK : TILE_KX)) * sizeof(float);
+}
 
+// TA: A is stored [K][M] (the product is A^T B); TB: B is stored [N][K] (A B^T).
+template <bool TA, bool TB>
 __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
                                                              float* __restrict__ C, int M, int N, int K, int tiles_n) {
   extern __shared__ __align__(16) float smem32[];
-  float* As = smem32;                               // [2][BM][LD]
-  float* Bs = smem32 + 2 * TILE;                    // [2][BK][LDB]
+  constexpr int TILE = TA ? TILE_KX : TILE_XK, TILE_B = TB ? TILE_XK : TILE_KX;
+  float* As = smem32;                               // [2][BM][LD], or [2][BK][LDB] when TA
+  float* Bs = smem32 + 2 * TILE;                    // [2][BK][LDB], or [2][BN][LD] when TB
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   A += (size_t)blockIdx.y * M * K;                  // one product of the batch per grid row
@@ -68,26 +79,41 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
   // repeat the last valid ones; their products are never stored.
   const float* pa[4];
   const float* pb[4];
+  size_t step_a, step_b;                            // floats from one k tile to the next
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int arow = tm * BM + (tid >> 3) + 32 * i;                  // 8 chunks per row of 32 k
-    pa[i] = A + (size_t)(arow < M ? arow : M - 1) * K + (tid & 7) * 4;
-    const int bcol = tn * BN + (tid & 31) * 4;                       // 32 chunks per row of 128 n
-    pb[i] = B + (size_t)((tid >> 5) + 8 * i) * N + (bcol < N ? bcol : N - 4);
+    if (!TA) {                                      // [M][K]: 8 chunks per row of 32 k
+      const int arow = tm * BM + (tid >> 3) + 32 * i;
+      pa[i] = A + (size_t)(arow < M ? arow : M - 1) * K + (tid & 7) * 4;
+    } else {                                        // [K][M]: 32 chunks per row of 128 m
+      const int acol = tm * BM + (tid & 31) * 4;
+      pa[i] = A + (size_t)((tid >> 5) + 8 * i) * M + (acol < M ? acol : M - 4);
+    }
+    if (!TB) {                                      // [K][N]: 32 chunks per row of 128 n
+      const int bcol = tn * BN + (tid & 31) * 4;
+      pb[i] = B + (size_t)((tid >> 5) + 8 * i) * N + (bcol < N ? bcol : N - 4);
+    } else {                                        // [N][K]: 8 chunks per row of 32 k
+      const int brow = tn * BN + (tid >> 3) + 32 * i;
+      pb[i] = B + (size_t)(brow < N ? brow : N - 1) * K + (tid & 7) * 4;
+    }
   }
+  step_a = TA ? (size_t)BK * M : (size_t)BK;
+  step_b = TB ? (size_t)BK : (size_t)BK * N;
   f32x4 ga[4], gb[4];
   auto load_tiles = [&](int kt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      ga[i] = *reinterpret_cast<const f32x4*>(pa[i] + (size_t)kt * BK);
-      gb[i] = *reinterpret_cast<const f32x4*>(pb[i] + (size_t)kt * BK * N);
+      ga[i] = *reinterpret_cast<const f32x4*>(pa[i] + (size_t)kt * step_a);
+      gb[i] = *reinterpret_cast<const f32x4*>(pb[i] + (size_t)kt * step_b);
     }
   };
   auto store_tiles = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<f32x4*>(As + buf * TILE + ((tid >> 3) + 32 * i) * LD + (tid & 7) * 4) = ga[i];
-      *reinterpret_cast<f32x4*>(Bs + buf * TILE_B + ((tid >> 5) + 8 * i) * LDB + (tid & 31) * 4) = gb[i];
+      float* da = TA ? As + buf * TILE + ((tid >> 5) + 8 * i) * LDB + (tid & 31) * 4 : As + buf * TILE + ((tid >> 3) + 32 * i) * LD + (tid & 7) * 4;
+      float* db = TB ? Bs + buf * TILE_B + ((tid >> 3) + 32 * i) * LD + (tid & 7) * 4 : Bs + buf * TILE_B + ((tid >> 5) + 8 * i) * LDB + (tid & 31) * 4;
+      *reinterpret_cast<f32x4*>(da) = ga[i];
+      *reinterpret_cast<f32x4*>(db) = gb[i];
     }
   };
 
@@ -129,11 +155,19 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
     const float* bs = Bs + buf * TILE_B;
     auto load_group = [&](int g, int s) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[s][i] = *reinterpret_cast<const f32x4*>(as + (row_a + 32 * i) * LD + g * 8 + k_half);
+      for (int i = 0; i < 2; ++i) {
+        if (!TA) a[s][i] = *reinterpret_cast<const f32x4*>(as + (row_a + 32 * i) * LD + g * 8 + k_half);
+        else
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+          for (int m = 0; m < 4; ++m) a[s][i][m] = as[(g * 8 + k_half + m) * LDB + row_a + 32 * i];
+      }
 #pragma unroll
-        for (int m = 0; m < 4; ++m) b[s][j][m] = bs[(g * 8 + k_half + m) * LDB + col_b + 32 * j];
+      for (int j = 0; j < 2; ++j) {
+        if (TB) b[s][j] = *reinterpret_cast<const f32x4*>(bs + (col_b + 32 * j) * LD + g * 8 + k_half);
+        else
+#pragma unroll
+          for (int m = 0; m < 4; ++m) b[s][j][m] = bs[(g * 8 + k_half + m) * LDB + col_b + 32 * j];
+      }
     };
     multiply(1);                                    // group 3 of the previous tile
     load_group(0, 0);
@@ -148,8 +182,9 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
     // Issue order of the tile (one scheduling region): memory instructions are spread between the matrix
     // instructions one at a time, so that neither the LDS queues nor the matrix pipe run dry or full.
     // masks: 0x008 matrix, 0x020 global read, 0x100 LDS read, 0x200 LDS write
+    constexpr int NDS = (TA ? 4 : 2) + (TB ? 2 : 4);                         // LDS reads per group: a 16-byte read per tile when k is contiguous, else four 4-byte reads in two instructions
 #pragma unroll
-    for (int n = 0; n < 6; ++n) {                                            // previous group 3 multiplies, group 0 is read
+    for (int n = 0; n < NDS; ++n) {                                          // previous group 3 multiplies, group 0 is read
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
@@ -158,18 +193,18 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    if constexpr (8 - NDS > 0) __builtin_amdgcn_sched_group_barrier(0x008, 8 - NDS, 0);
 #pragma unroll
     for (int h = 0; h < 2; ++h) {                                            // groups 0 and 1 multiply, 1 and 2 are read
 #pragma unroll
-      for (int n = 0; n < 6; ++n) {
+      for (int n = 0; n < NDS; ++n) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, 10, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 16 - NDS, 0);
     }
 #pragma unroll
-    for (int n = 0; n < 6; ++n) {                                            // group 2 multiplies, group 3 is read
+    for (int n = 0; n < NDS; ++n) {                                          // group 2 multiplies, group 3 is read
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
@@ -178,7 +213,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    if constexpr (8 - NDS > 0) __builtin_amdgcn_sched_group_barrier(0x008, 8 - NDS, 0);
     __syncthreads();
   }
   multiply(1);                                      // group 3 of the last tile
@@ -199,29 +234,50 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const float* __restr
 
 }  // namespace
 
-extern "C" int art_gemm_f32_batched(const void* a_dev, const void* b_dev, void* c_dev, int batch, int M, int N, int K, void* stream) {
+namespace {
+
+template <bool TA, bool TB>
+int launch_gemm_f32(const float* a, const float* b, float* c, int batch, int M, int N, int K, hipStream_t stream) {
+  static bool configured = false;
+  if (!configured) {
+    ART_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f32_kernel<TA, TB>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes<TA, TB>()));
+    configured = true;
+  }
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  ART_REQUIRE((long long)tiles_m * tiles_n <= 0x7fffffffLL, "art_gemm_f32: too many tiles");
+  gemm_f32_kernel<TA, TB><<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(kThreads), lds_bytes<TA, TB>(), stream>>>(a, b, c, M, N, K, tiles_n);
+  ART_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int art_gemm_f32_ex(const void* a_dev, const void* b_dev, void* c_dev, int batch, int M, int N, int K, int trans_a,
+                               int trans_b, void* stream) {
   ART_REQUIRE(a_dev && b_dev && c_dev, "art_gemm_f32: null pointer");
   ART_REQUIRE(batch > 0 && batch <= 65535, "art_gemm_f32: batch must be 1..65535 (got %d)", batch);
-  ART_REQUIRE(M > 0 && N >= 4 && K > 0 && N % 4 == 0 && K % 32 == 0,
-              "art_gemm_f32: N must be a multiple of 4 and K of 32 (M=%d N=%d K=%d)", M, N, K);
+  ART_REQUIRE(M > 0 && N > 0 && K > 0 && K % 32 == 0, "art_gemm_f32: K must be a multiple of 32 (M=%d N=%d K=%d)", M, N, K);
+  // an operand whose rows run along m or n is fetched in 16-byte pieces of those rows
+  ART_REQUIRE(trans_b || (N % 4 == 0 && N >= 4), "art_gemm_f32: N must be a multiple of 4 when B is stored [K][N] (N=%d)", N);
+  ART_REQUIRE(!trans_a || (M % 4 == 0 && M >= 4), "art_gemm_f32: M must be a multiple of 4 when A is stored [K][M] (M=%d)", M);
   ART_REQUIRE(((uintptr_t)a_dev % 16) == 0 && ((uintptr_t)b_dev % 16) == 0 && ((uintptr_t)c_dev % 4) == 0,
               "art_gemm_f32: A and B must be 16-byte aligned");
   const size_t nb = (size_t)batch;
   ART_REQUIRE(!art::overlaps(a_dev, nb * M * K * 4, c_dev, nb * M * N * 4) && !art::overlaps(b_dev, nb * K * N * 4, c_dev, nb * M * N * 4),
               "art_gemm_f32: C must not overlap A or B");
-  static bool configured = false;
-  if (!configured) {
-    ART_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f32_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes));
-    configured = true;
-  }
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  ART_REQUIRE((long long)tiles_m * tiles_n <= 0x7fffffffLL, "art_gemm_f32: too many tiles");
-  gemm_f32_kernel<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(kThreads), kLdsBytes, (hipStream_t)stream>>>(
-      (const float*)a_dev, (const float*)b_dev, (float*)c_dev, M, N, K, tiles_n);
-  ART_LAUNCH_CHECK();
-  return 0;
+  const float* a = (const float*)a_dev;
+  const float* b = (const float*)b_dev;
+  float* c = (float*)c_dev;
+  hipStream_t st = (hipStream_t)stream;
+  if (trans_a) return trans_b ? launch_gemm_f32<true, true>(a, b, c, batch, M, N, K, st) : launch_gemm_f32<true, false>(a, b, c, batch, M, N, K, st);
+  return trans_b ? launch_gemm_f32<false, true>(a, b, c, batch, M, N, K, st) : launch_gemm_f32<false, false>(a, b, c, batch, M, N, K, st);
+}
+
+extern "C" int art_gemm_f32_batched(const void* a_dev, const void* b_dev, void* c_dev, int batch, int M, int N, int K, void* stream) {
+  return art_gemm_f32_ex(a_dev, b_dev, c_dev, batch, M, N, K, 0, 0, stream);
 }
 
 extern "C" int art_gemm_f32(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream) {
-  return art_gemm_f32_batched(a_dev, b_dev, c_dev, 1, M, N, K, stream);
+  return art_gemm_f32_ex(a_dev, b_dev, c_dev, 1, M, N, K, 0, 0, stream);
 }

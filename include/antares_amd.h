@@ -247,6 +247,12 @@ int art_gemm_f32(const void* a_dev, const void* b_dev, void* c_dev, int M, int N
  * Replaces the kernel the reference generates for `output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]`
  * (AntaresIR.md:121). */
 int art_gemm_f32_batched(const void* a_dev, const void* b_dev, void* c_dev, int batch, int M, int N, int K, void* stream);
+/* The same with either operand stored the other way round: trans_a != 0 means A is [K][M] (C = A^T B, M % 4 == 0),
+ * trans_b != 0 means B is [N][K] (C = A B^T, the layout of a linear layer's weight; N need not be a multiple of 4 then).
+ * Replaces the kernels the reference generates for `out[M, N] +=! a[K, M] * b[K, N]`, `... a[M, K] * b[N, K]` and
+ * `... a[K, M] * b[N, K]` (the same tiled schedule, backends/c-rocm/schedule/standard/algo_tiling.py:35-98). */
+int art_gemm_f32_ex(const void* a_dev, const void* b_dev, void* c_dev, int batch, int M, int N, int K, int trans_a, int trans_b,
+                    void* stream);
 
 /* Stable even-first partition of int32 values: all even values in input order,
  * then all odd values in input order.  Two launches (count, then rank + scatter),

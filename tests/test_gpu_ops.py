@@ -765,3 +765,31 @@ def test_row_reductions_and_their_map_run_as_one_kernel(autort, ir, inputs, shap
         assert np.array_equal(got, apart)
     else:
         assert np.allclose(got.astype(np.float64), apart.astype(np.float64), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize('ir,ta,tb,M,N,K', [
+    ('out[M, N] +=! x[K, M] * w[K, N]', True, False, 1028, 512, 96),
+    ('out[M, N] +=! x[M, K] * w[N, K]', False, True, 1000, 1030, 64),       # a linear layer: N need not be a multiple of 4
+    ('out[M, N] +=! x[K, M] * w[N, K]', True, True, 2048, 129, 160),
+    ('out[M, N] +=! x[M, K] * w[N, K]', False, True, 4096, 4096, 1024),
+])
+def test_fp32_gemm_with_operands_stored_the_other_way_round(autort, ir, ta, tb, M, N, K):
+    """`A^T B`, `A B^T` and `A^T B^T` in float32 go to art_gemm_f32_ex; results are the float64 products' to fp32
+    accuracy, and a one-hot operand pins which axis of each operand is k."""
+    note(f'gemm_f32 layouts {ir} {M}x{N}x{K}')
+    dev = autort.device()
+    sa, sb = (f'x=float32[K:{K}, M:{M}]' if ta else f'x=float32[M:{M}, K:{K}]'), (f'w=float32[N:{N}, K:{K}]' if tb else f'w=float32[K:{K}, N:{N}]')
+    op = autort.export(ir=ir, inputs=[sa, sb], name=f'gemm_f32_l{int(ta)}{int(tb)}_{M}_{N}_{K}')
+    assert op.fast_path is not None
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn((K, M) if ta else (M, K), generator=g)
+    b = torch.randn((N, K) if tb else (K, N), generator=g)
+    got = op(a.to(dev), b.to(dev)).cpu()
+    am, bm = (a.t() if ta else a).double(), (b.t() if tb else b).double()
+    want = am @ bm
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5 * max(1.0, K ** 0.5)), (got.double() - want).abs().max()
+    if M <= 2048:
+        sel = torch.zeros(M, K)
+        sel[torch.arange(M), torch.arange(M) % K] = 1.0              # row m of the result = row m % K of B
+        sel_in = sel.t().contiguous() if ta else sel
+        assert torch.equal(op(sel_in.to(dev), b.to(dev)).cpu(), (b.t() if tb else b)[torch.arange(M) % K].contiguous())
