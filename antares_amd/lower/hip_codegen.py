@@ -17,7 +17,10 @@ templates:
   output (DPP / readlane reduction), one 256-thread block per output, one
   thread per output, and for contractions one thread per 4 x 4 patch of
   outputs (register tiling: operands that are constant along one of the two
-  tiled axes are loaded once per patch) — and the launcher picks by extents
+  tiled axes are loaded once per patch), and for float32 sums of products of
+  two loads whose indices split into a row / column part and a k part (matrix
+  products in any layout, batched, convolutions) a kernel on the fp32 matrix
+  instructions with its address arithmetic in LDS tables — and the launcher picks by extents
   and by which axis is contiguous in memory (the reference reduces through LDS because its TVM patch
   disables wavefront shuffles off CUDA, engine/device-stub/tvm_v0.8.0.patch:186-191);
 * scatter statements: one thread per point of the iteration space, atomics for
@@ -203,6 +206,7 @@ class KernelPlan:
     tile_axes: Optional[Tuple[str, str]] = None   # permutation copies: last axis of the load, last axis of the store
     tile_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for the vector form of it
     row_group: Optional[RowGroup] = None          # set on the first statement of a run that one row kernel can compute
+    matrix: Optional[Dict[str, List[object]]] = None   # matrix-instruction variant: extents of its row, column, batch and k axes
 
     def _tiles(self, env: Dict[str, int]) -> int:
         """64 x 64 tiles of the transposing variant, 0 when it does not apply or an axis is too short to pay."""
@@ -244,6 +248,24 @@ class KernelPlan:
             return 0
         return total // self.row_vec
 
+    def _matrix_blocks(self, env: Dict[str, int]) -> int:
+        """Blocks of the matrix-instruction variant (128 x 128 outputs each, per batch), 0 when it does not apply:
+        k must come in whole tiles of 16, and there must be enough tiles and enough k to pay for staging them."""
+        if self.matrix is None or 'matrix' not in self.variants:
+            return 0
+        def prod(key):
+            n = 1
+            for e in self.matrix[key]:
+                n *= e if isinstance(e, int) else env[e]
+            return n
+        M, N, B, K = prod('m'), prod('n'), prod('batch'), prod('k')
+        if K % 16 or K < 64 or M < 64 or N < 64:
+            return 0
+        blocks = ((M + 127) // 128) * ((N + 127) // 128) * B
+        if blocks < 64 or blocks > MAX_GRID * 64:
+            return 0
+        return blocks
+
     def _patches(self, env: Dict[str, int], total: int) -> int:
         """Threads of the register-tiled reduce variant for these extents, 0 when it does not apply."""
         if 'patch' not in self.variants or self.patch is None:
@@ -280,6 +302,9 @@ class KernelPlan:
         if self.kind == 'scatter':
             return self.variants['scalar'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
         # reduce
+        blocks = self._matrix_blocks(env)
+        if blocks:
+            return self.variants['matrix'], blocks, BLOCK
         patches = self._patches(env, total)
         if patches >= 131072 and red >= 8:           # two wavefronts per SIMD and more: below that one output per thread hides latency better
             return self.variants['patch'], min((patches + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
@@ -756,8 +781,154 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
             src.append('\n'.join(b))
             variants['patch'] = sym
             plan.patch, plan.patch_dims = (TX, TY), [ext[xa], ext[ya]]
+        mc = _matrix_contraction(st, tensors)
+        if mc is not None:
+            src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_m', mc))
+            variants['matrix'] = name + '_m'
+            ext = dict(st.data_axes + st.reduce_axes)
+            plan.matrix = {key: [ext[a] for a in mc[key]] for key in ('m', 'n', 'batch', 'k')}
 
     return '\n\n'.join(src), plan
+
+
+def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
+    """A sum of products of two loads on v_mfma_f32_32x32x2_f32 (the reference's counterpart: its tiled schedule for
+    contractions, backends/c-rocm/schedule/standard/algo_tiling.py:35-98, on the vector units).  A block of 256
+    threads = 2 x 2 wavefronts owns 128 rows x 128 columns of one batch, where a row is a point of the axes only
+    the first load uses and a column a point of those only the second uses; k runs over the reduce axes in tiles of
+    16.  An element's address is (row or column offset) + (k offset): the row, column and output offsets of the tile
+    are worked out once into LDS tables, the k offsets once per tile, so the inner loads are a table look-up and an
+    add - whatever the index expressions are (a convolution's `HO + KH`, a gathered row, a transposed operand).
+    Both operands are staged in LDS as [row or column][k] and fed to the matrix instruction exactly as the fp32
+    GEMM kernel of the library feeds it; rows, columns and batches past the extents are clamped on the way in and
+    cut on the way out.  k must be a multiple of 16."""
+    la, lb = mc['la'], mc['lb']
+    ta, tb, oct_ = HIP_TYPE[tensors[la.name].dtype], HIP_TYPE[tensors[lb.name].dtype], HIP_TYPE[st.out_dtype]
+    plain = ExprEmitter(tensors)
+    ext = dict(st.data_axes + st.reduce_axes)
+
+    def prod(names):
+        return ' * '.join(f'(long long)__ext_{a}' for a in names) or '1LL'
+
+    def decompose(var, names, indent):
+        out = [f'{indent}long long __q = {var};']
+        for a in reversed(names):
+            out.append(f'{indent}const int {a} = (int)(__q % __ext_{a}); __q /= __ext_{a}; (void){a};')
+        return out
+    out_axes = [a for a, _ in st.data_axes]
+    rows_of_out = plain.offset(st.output, [a if (a in mc['m'] or a in mc['batch']) else '0' for a in out_axes])
+    cols_of_out = plain.offset(st.output, [a if a in mc['n'] else '0' for a in out_axes])
+    val_a = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__ra[{j}]').expr(mc['fa']) for j in range(8)]
+    val_b = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__rb[{j}]').expr(mc['fb']) for j in range(8)]
+    b = [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st)
+    b += ['  typedef float __f16v __attribute__((ext_vector_type(16)));',
+          '  typedef float __f4 __attribute__((ext_vector_type(4)));',
+          '  __shared__ __attribute__((aligned(16))) float __As[2][128 * 20];     // [row][k], 16 k and 4 floats of padding per row',
+          '  __shared__ __attribute__((aligned(16))) float __Bs[2][128 * 20];     // [column][k]',
+          '  __shared__ long long __am[128], __bn[128], __cm[128], __cn[128], __ak[2][16], __bk[2][16];',
+          f'  const long long __M = {prod(mc["m"])}, __N = {prod(mc["n"])}, __B = {prod(mc["batch"])};',
+          f'  const int __T = (int)(({prod(mc["k"])}) / 16);',
+          '  const long long __tn_n = (__N + 127) / 128, __tiles = ((__M + 127) / 128) * __tn_n;',
+          '  const int __tid = threadIdx.x, __lane = __tid & 63, __wave = __tid >> 6, __wm = __wave >> 1, __wn = __wave & 1;',
+          '  for (long long __blk = blockIdx.x; __blk < __tiles * __B; __blk += gridDim.x) {',
+          '    const long long __t0 = __blk % __tiles, __tm = __t0 / __tn_n, __tn = __t0 % __tn_n;']
+    b += decompose('__blk / __tiles', mc['batch'], '    ')
+    b += ['    if (__tid < 128) {                            // row offsets of the first operand and of the output',
+          '      long long __row = __tm * 128 + __tid;',
+          '      if (__row >= __M) __row = __M - 1;']
+    b += decompose('__row', mc['m'], '      ')
+    b += [f'      __am[__tid] = {mc["parts"]["a"][0]};', f'      __cm[__tid] = {rows_of_out};',
+          '    } else {                                      // column offsets of the second operand and of the output',
+          '      long long __colq = __tn * 128 + (__tid - 128);',
+          '      if (__colq >= __N) __colq = __N - 1;']
+    b += decompose('__colq', mc['n'], '      ')
+    b += [f'      __bn[__tid - 128] = {mc["parts"]["b"][0]};', f'      __cn[__tid - 128] = {cols_of_out};',
+          '    }',
+          '    auto __ktab = [&](int __kt, int __buf) {       // k offsets of tile __kt: 16 for each operand',
+          '      if (__tid < 32) {',
+          '        const long long __kk = (long long)__kt * 16 + (__tid & 15);']
+    b += decompose('__kk', mc['k'], '        ')
+    b += [f'        if (__tid < 16) __ak[__buf][__tid] = {mc["parts"]["a"][1]};',
+          f'        else __bk[__buf][__tid - 16] = {mc["parts"]["b"][1]};',
+          '      }',
+          '    };',
+          '    __ktab(0, 0);',
+          '    if (__T > 1) __ktab(1, 1);',
+          '    __syncthreads();',
+          '    const int __ml = __tid & 127, __kh = (__tid >> 7) * 8;     // lanes along rows: 8 k of one row (column) per thread',
+          '    const int __kl = __tid & 15, __rw = __tid >> 4;             // lanes along k: one k of 8 rows (columns) per thread',
+          '    (void)__ml; (void)__kh; (void)__kl; (void)__rw;']
+    for x, ld, ct, tab, ktab_, lds, vals in (('a', la, ta, '__am', '__ak', '__As', val_a), ('b', lb, tb, '__bn', '__bk', '__Bs', val_b)):
+        if mc['parts'][x][2]:
+            b += [f'    const {ct}* __p{x}[8];', '    #pragma unroll',
+                  f'    for (int __j = 0; __j < 8; ++__j) __p{x}[__j] = {ld.name} + {tab}[__rw + 16 * __j];']
+        else:
+            b.append(f'    const {ct}* __p{x} = {ld.name} + {tab}[__ml];')
+        b.append(f'    {ct} __r{x}[8];')
+    b += ['    auto __load = [&](int __buf) {']
+    for x, ktab_ in (('a', '__ak'), ('b', '__bk')):
+        if mc['parts'][x][2]:
+            b += [f'      {{ const long long __ko = {ktab_}[__buf][__kl];', '        #pragma unroll',
+                  f'        for (int __j = 0; __j < 8; ++__j) __r{x}[__j] = __p{x}[__j][__ko]; }}']
+        else:
+            b += ['      #pragma unroll', f'      for (int __j = 0; __j < 8; ++__j) __r{x}[__j] = __p{x}[{ktab_}[__buf][__kh + __j]];']
+    b += ['    };', '    auto __stage = [&](int __buf) {']
+    for x, lds, vals in (('a', '__As', val_a), ('b', '__Bs', val_b)):
+        if mc['parts'][x][2]:
+            b += [f'      {lds}[__buf][(__rw + {16 * j}) * 20 + __kl] = (float)({vals[j]});' for j in range(8)]
+        else:
+            b += [f'      *(__f4*)&{lds}[__buf][__ml * 20 + __kh] = __f4{{(float)({vals[0]}), (float)({vals[1]}), (float)({vals[2]}), (float)({vals[3]})}};',
+                  f'      *(__f4*)&{lds}[__buf][__ml * 20 + __kh + 4] = __f4{{(float)({vals[4]}), (float)({vals[5]}), (float)({vals[6]}), (float)({vals[7]})}};']
+    b += ['    };',
+          '    __f16v __acc[2][2];',
+          '    #pragma unroll',
+          '    for (int __i = 0; __i < 2; ++__i)',
+          '      #pragma unroll',
+          '      for (int __j = 0; __j < 2; ++__j)',
+          '        #pragma unroll',
+          '        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = 0.f;',
+          '    const int __row0 = __wm * 64 + (__lane & 31), __col0 = __wn * 64 + (__lane & 31), __kq = (__lane >> 5) * 4;',
+          '    __load(0);',
+          '    __stage(0);',
+          '    __syncthreads();',
+          '    for (int __t = 0; __t < __T; ++__t) {',
+          '      const int __buf = __t & 1;',
+          '      if (__t + 1 < __T) __load(__buf ^ 1);           // tile t + 1 travels while tile t is multiplied',
+          '      if (__t + 2 < __T) __ktab(__t + 2, __buf);       // its k offsets were read a tile ago',
+          '      #pragma unroll',
+          '      for (int __g = 0; __g < 2; ++__g) {',
+          '        __f4 __a[2], __b[2];',
+          '        #pragma unroll',
+          '        for (int __i = 0; __i < 2; ++__i) {',
+          '          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * 20 + __g * 8 + __kq];',
+          '          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * 20 + __g * 8 + __kq];',
+          '        }',
+          '        #pragma unroll',
+          '        for (int __m = 0; __m < 4; ++__m)',
+          '          #pragma unroll',
+          '          for (int __i = 0; __i < 2; ++__i)',
+          '            #pragma unroll',
+          '            for (int __j = 0; __j < 2; ++__j)',
+          '              __acc[__i][__j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__a[__i][__m], __b[__j][__m], __acc[__i][__j], 0, 0, 0);',
+          '      }',
+          '      if (__t + 1 < __T) __stage(__buf ^ 1);          // the other buffer: everybody left it at the last barrier',
+          '      __syncthreads();',
+          '    }',
+          '    // accumulator element e of tile (i, j): row i*32 + (e/4)*8 + (lane/32)*4 + e%4, column j*32 + lane%32',
+          '    #pragma unroll',
+          '    for (int __i = 0; __i < 2; ++__i)',
+          '      #pragma unroll',
+          '      for (int __j = 0; __j < 2; ++__j) {',
+          '        const int __c = __wn * 64 + __j * 32 + (__lane & 31);',
+          '        #pragma unroll',
+          '        for (int __e = 0; __e < 16; ++__e) {',
+          '          const int __r = __wm * 64 + __i * 32 + (__e >> 2) * 8 + (__lane >> 5) * 4 + (__e & 3);',
+          f'          if (__tm * 128 + __r < __M && __tn * 128 + __c < __N) {st.output}[__cm[__r] + __cn[__c]] = ({oct_})__acc[__i][__j][__e];',
+          '        }',
+          '      }',
+          '    __syncthreads();                               // the tables and buffers are rewritten by the next tile',
+          '  }', '}']
+    return '\n'.join(b)
 
 
 def _patch_axes(st):
@@ -802,6 +973,79 @@ def _reduce_axis_contiguous(st, tensors) -> Optional[bool]:
         return None
     return score > 0
 
+
+
+def _axes_of(e: Expr) -> set:
+    return {m.name for m in walk(e) if m.kind == 'axis'}
+
+
+def _axes_of_all(load: Expr) -> set:
+    return set().union(*[_axes_of(a) for a in load.args]) if load.args else set()
+
+
+def _split_index(e: Expr, em: ExprEmitter, outer: set, inner: set):
+    """An index expression as (part that depends on `outer` axes only, part that depends on `inner` axes only), each
+    as C text or None, when it is one of the two or a sum of such parts; else None."""
+    used = _axes_of(e)
+    if used <= outer:
+        return em.expr(e), None
+    if used <= inner:
+        return None, em.expr(e)
+    if e.kind == 'op' and e.name == '+' and len(e.args) == 2:
+        l, r = _split_index(e.args[0], em, outer, inner), _split_index(e.args[1], em, outer, inner)
+        if l is None or r is None:
+            return None
+
+        def add(x, y):
+            return y if x is None else (x if y is None else f'({x}) + ({y})')
+        return add(l[0], r[0]), add(l[1], r[1])
+    return None
+
+
+def _matrix_contraction(st, tensors):
+    """Reads a sum of products of two factors, one load each, as a matrix product on the fp32 matrix instructions:
+    data axes that only the first load uses are rows (M), those only the second uses are columns (N), those both use
+    are a batch, the reduce axes are k.  Every index of a load must split into a part that depends on k axes and a
+    part that does not, so that an element's address is a row (column) offset plus a k offset.  -> dict or None."""
+    if st.scatter or st.reduce != '+' or st.root.dtype != 'float32' or not st.reduce_axes or not st.data_axes:
+        return None
+    root = st.root
+    if root.kind == 'when' or root.kind != 'op' or root.name != '*' or len(root.args) != 2:
+        return None
+    axes = [a for a, _ in st.data_axes]
+    if [i.name if i.kind == 'axis' else None for i in st.out_index] != axes:
+        return None
+    fa, fb = root.args
+    la, lb = [n for n in walk(fa) if n.kind == 'load'], [n for n in walk(fb) if n.kind == 'load']
+    if len(la) != 1 or len(lb) != 1 or st.output in (la[0].name, lb[0].name):
+        return None
+    la, lb = la[0], lb[0]
+    # axes may be used inside the indices of the two loads only
+    inside = sum(1 for n in (la, lb) for a in n.args for m in walk(a) if m.kind == 'axis')
+    if sum(1 for m in walk(root) if m.kind == 'axis') != inside:
+        return None
+    ua, ub = set().union(*[_axes_of(a) for a in la.args]), set().union(*[_axes_of(a) for a in lb.args])
+    k_axes = [a for a, _ in st.reduce_axes]
+    if not set(k_axes) <= ua or not set(k_axes) <= ub:
+        return None
+    m_axes = [a for a in axes if a in ua and a not in ub]
+    n_axes = [a for a in axes if a in ub and a not in ua]
+    batch = [a for a in axes if a in ua and a in ub]
+    if not m_axes or not n_axes or len(m_axes) + len(n_axes) + len(batch) != len(axes):
+        return None
+    if ITEMSIZE[tensors[la.name].dtype] not in (2, 4) or ITEMSIZE[tensors[lb.name].dtype] not in (2, 4):
+        return None
+    plain = ExprEmitter(tensors)
+    parts = {}
+    for tag, ld, own in (('a', la, m_axes), ('b', lb, n_axes)):
+        outer, inner = set(own) | set(batch), set(k_axes)
+        sp = [_split_index(ix, plain, outer, inner) for ix in ld.args]
+        if any(x is None for x in sp):
+            return None
+        # lanes walk k when the operand's last index is made of k axes alone (k is then the contiguous axis), else rows
+        parts[tag] = (plain.offset(ld.name, [x[0] or '0' for x in sp]), plain.offset(ld.name, [x[1] or '0' for x in sp]),
+                      sp[-1][0] is None)
+    return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts}
 
 
 def _row_group_at(graph, i: int) -> int:
@@ -851,6 +1095,11 @@ def _row_group_at(graph, i: int) -> int:
                 and list(tensors[m.output].shape) == [e for _, e in D + [R]]
                 and loads_fit(m, len(order), ()))
     forbidden = (m.output,) if with_map else ()
+    # a row is a run of memory of its own: some load of every reduction is indexed by all the data axes (in a
+    # contraction no load is - its operands are shared between outputs, which the other reduce variants exploit)
+    for k in range(len(order)):
+        if not any(n.kind == 'load' and set(d_names) <= _axes_of_all(n) for n in walk(sts[i + k].root)):
+            return 0
     # a reduction that does not fit ends the run before it
     for k in range(len(order)):
         if not loads_fit(sts[i + k], k, forbidden):

@@ -628,23 +628,77 @@ def test_register_tiled_contractions_match_the_oracle(autort, ir, inputs, shapes
 
 
 def test_large_contractions_take_the_register_tiled_variant(autort):
-    """A 2048 x 2048 x 256 fp32 matrix product is large enough for it (a 1024 x 1024 one is not); the result is the
-    float64 product's."""
-    note('register-tiled reduce picked for a 2048x2048x256 fp32 matmul')
+    """A 2048 x 2048 x 250 fp32 matrix product is large enough for it (a 1024 x 1024 one is not; with k a multiple of
+    16 the matrix-instruction variant takes over); the result is the float64 product's."""
+    note('register-tiled reduce picked for a 2048x2048x250 fp32 matmul')
     dev = autort.device()
-    op = autort.export(ir='output0[N, M] +=! input0[N, K] * input1[K, M]', inputs=['input0=float32[N:2048, K:256]', 'input1=float32[K:256, M:2048]'],
+    op = autort.export(ir='output0[N, M] +=! input0[N, K] * input1[K, M]', inputs=['input0=float32[N:2048, K:250]', 'input1=float32[K:250, M:2048]'],
                        name='patch_matmul_2048')
-    op.fast_path = None               # this shape would go to the matrix-core kernel: the generic lowering is what is tested here
+    op.fast_path = None               # the generic lowering is what is tested here
     plan = op.plans[0]
     zero = {n: 0 for n in plan.args}
-    assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['patch']
-    assert plan.choose({'N': 2046, 'K': 256, 'M': 2048}, zero)[0] != plan.variants['patch']
-    assert plan.choose({'N': 1024, 'K': 256, 'M': 1024}, zero)[0] != plan.variants['patch']
+    assert plan.choose({'N': 2048, 'K': 250, 'M': 2048}, zero)[0] == plan.variants['patch']
+    assert plan.choose({'N': 2046, 'K': 250, 'M': 2048}, zero)[0] != plan.variants['patch']
+    assert plan.choose({'N': 1024, 'K': 250, 'M': 1024}, zero)[0] != plan.variants['patch']
+    assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['matrix']
     g = torch.Generator().manual_seed(2)
-    a, b = torch.randn(2048, 256, generator=g), torch.randn(256, 2048, generator=g)
+    a, b = torch.randn(2048, 250, generator=g), torch.randn(250, 2048, generator=g)
     got = op(a.to(dev), b.to(dev)).cpu()
     want = (a.double() @ b.double()).float()
     assert torch.allclose(got, want, rtol=1e-4, atol=1e-3)
+
+
+MATRIX_CASES = [
+    # a convolution; the same with stride 2; a batched product with ragged tiles and k = 5 x 16; fp16 operands cast to
+    # float32 with B stored [N, K]; elementwise work on one factor (AntaresIR.md:247 over all of K); a product whose
+    # output axes are stored columns first
+    ('output0[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[F, C, KH, KW] where HO in 32, WO in 32',
+     ['input0=float32[N:8, C:16, H:34, W:34]', 'input1=float32[F:64, C:16, KH:3, KW:3]'], [(8, 16, 34, 34), (64, 16, 3, 3)]),
+    ('output0[N, F, HO, WO] +=! input0[N, C, HO * 2 + KH, WO * 2 + KW] * input1[F, C, KH, KW] where HO in 32, WO in 32',
+     ['input0=float32[N:8, C:16, H:66, W:66]', 'input1=float32[F:70, C:16, KH:3, KW:3]'], [(8, 16, 66, 66), (70, 16, 3, 3)]),
+    ('output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]', ['input0=float32[B:3, N:700, K:80]', 'input1=float32[B:3, K:80, M:520]'],
+     [(3, 700, 80), (3, 80, 520)]),
+    ('output0[N, M] +=! input0[N, K].to(`float32`) * input1[M, K].to(`float32`)', ['input0=float16[N:1024, K:64]', 'input1=float16[M:1000, K:64]'],
+     [(1024, 64), (1000, 64)]),
+    ('temp0[K, N] = input0[N, K] + 100; output0[N, M] +=! temp0[K, N] * input1[K, M]',
+     ['input0=float32[N:1024, K:512]', 'input1=float32[K:512, M:1024]'], [(1024, 512), (512, 1024)]),
+    ('output0[M, N] +=! input0[N, K] * input1[K, M]', ['input0=float32[N:1030, K:64]', 'input1=float32[K:64, M:1024]'], [(1030, 64), (64, 1024)]),
+]
+
+
+@pytest.mark.parametrize('ir,inputs,shapes', MATRIX_CASES)
+def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, ir, inputs, shapes):
+    """Sums of products of two loads whose indices split into a row (or column) part and a k part run on
+    v_mfma_f32_32x32x2_f32 when k is a multiple of 16 and there are enough tiles; results are the oracle's to the
+    rounding of a float32 sum in another order, and the register-tiled variant gives the same to that rounding."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'matrix-instruction contraction {ir[:60]} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='mfma_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    op.fast_path = None
+    plan = op.plans[-1]
+    env = {}
+    for spec, shape in zip(inputs, shapes):
+        for d, v in zip(spec.split('[', 1)[1].rstrip(']').split(','), shape):
+            env[d.split(':')[0].strip()] = v
+    assert 'matrix' in plan.variants and plan.choose(env, {n: 0 for n in plan.args})[0] == plan.variants['matrix']
+    assert plan.row_group is None                 # nothing else takes the statement
+    g = torch.Generator().manual_seed(len(ir))
+    tensors = [torch.randn(shape, generator=g).to(torch.float16 if 'float16' in spec else torch.float32) for spec, shape in zip(inputs, shapes)]
+    got = op(*[t.to(dev) for t in tensors]).cpu().numpy()
+    names = [spec.split('=')[0] for spec in inputs]
+    want = CpuModule(parse_program(ir, inputs), fast_math=False)(**{n: t.numpy() for n, t in zip(names, tensors)})['output0']
+    K = 1
+    for ax, e in plan.reduce_axes:
+        K *= e if isinstance(e, int) else env[e]
+    scale = 100.0 if '+ 100' in ir else 1.0
+    assert got.shape == want.shape
+    assert np.allclose(got, want, rtol=1e-4, atol=2e-5 * scale * K ** 0.5 * 4), np.abs(got - want).max()
+    # the same statement through the register-tiled variant
+    del plan.variants['matrix']
+    apart = op(*[t.to(dev) for t in tensors]).cpu().numpy()
+    assert np.allclose(got, apart, rtol=1e-4, atol=2e-5 * scale * K ** 0.5 * 4)
 
 
 @pytest.mark.parametrize('M,N,K', [(512, 1024, 32), (1000, 1028, 96), (4096, 4096, 512), (129, 8192, 64), (2048, 2048, 2048)])

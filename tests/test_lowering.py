@@ -51,10 +51,14 @@ def test_softmax_is_one_row_group_with_kernels_for_short_and_long_rows():
     # a reduction alone; two of them; an offset in front of the reduced axis
     ('t[N] +=! x[N, C]', ['x=float32[N:8, C:256]'], 1),
     ('t[N] +=! x[N, C]; u[N] >=! x[N, C] * t[N]', ['x=float32[N:8, C:256]'], 2),
+    ('t[N] +=! x[N, C] * w[C]', ['x=float32[N:8, C:256]', 'w=float32[C:256]'], 1),
     ('t[S] +=! x[S * 1024 + C] where C in 1024, S in 8', ['x=float32[N:8192]'], 1),
     # the reduction runs over the first axis: lanes of a team would read addresses a row apart
     ('t[C] +=! x[N, C]; y[N, C] = x[N, C] - t[C]', ['x=float32[N:8, C:256]'], 0),
     ('t[N] +=! x[C, N]', ['x=float32[C:256, N:8]'], 0),
+    # contractions: no load is indexed by all the data axes
+    ('c[N, M] +=! a[N, K] * b[K, M]', ['a=float32[N:64, K:256]', 'b=float32[K:256, M:64]'], 0),
+    ('c[N, M] +=! a[N, K] * b[M, K]', ['a=float32[N:64, K:256]', 'b=float32[M:64, K:256]'], 0),
     # a map alone
     ('y[N, C] = x[N, C] * 2', ['x=float32[N:8, C:256]'], 0),
 ])
