@@ -344,6 +344,8 @@ class KernelPlan:
             tags += [('thread', total), ('wave', (total + waves_per_block - 1) // waves_per_block * BLOCK), ('block', total * BLOCK)]
             if self._patches(env, total):
                 tags.append(('patch', self._patches(env, total)))
+            if self._matrix_blocks(env):
+                tags.append(('matrix', self._matrix_blocks(env) * BLOCK))
         out = []
         for tag, work in tags:
             if tag not in self.variants:
