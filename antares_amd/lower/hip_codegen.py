@@ -250,7 +250,7 @@ class KernelPlan:
 
     def _matrix_blocks(self, env: Dict[str, int]) -> int:
         """Blocks of the matrix-instruction variant (128 x 128 outputs each, per batch), 0 when it does not apply:
-        k must come in whole tiles of 16, and there must be enough tiles and enough k to pay for staging them."""
+        there must be enough tiles and enough k to pay for staging them."""
         if self.matrix is None or 'matrix' not in self.variants:
             return 0
         def prod(key):
@@ -259,7 +259,7 @@ class KernelPlan:
                 n *= e if isinstance(e, int) else env[e]
             return n
         M, N, B, K = prod('m'), prod('n'), prod('batch'), prod('k')
-        if K % 16 or K < 64 or M < 64 or N < 64:
+        if K < 32 or M < 64 or N < 64:
             return 0
         blocks = ((M + 127) // 128) * ((N + 127) // 128) * B
         if blocks < 64 or blocks > MAX_GRID * 64:
@@ -803,7 +803,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
     add - whatever the index expressions are (a convolution's `HO + KH`, a gathered row, a transposed operand).
     Both operands are staged in LDS as [row or column][k] and fed to the matrix instruction exactly as the fp32
     GEMM kernel of the library feeds it; rows, columns and batches past the extents are clamped on the way in and
-    cut on the way out.  k must be a multiple of 16."""
+    cut on the way out; the k a last partial tile lacks are staged as zeros (their addresses wrap into the
+    tensors)."""
     la, lb = mc['la'], mc['lb']
     ta, tb, oct_ = HIP_TYPE[tensors[la.name].dtype], HIP_TYPE[tensors[lb.name].dtype], HIP_TYPE[st.out_dtype]
     plain = ExprEmitter(tensors)
@@ -829,7 +830,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
           '  __shared__ __attribute__((aligned(16))) float __Bs[2][128 * 20];     // [column][k]',
           '  __shared__ long long __am[128], __bn[128], __cm[128], __cn[128], __ak[2][16], __bk[2][16];',
           f'  const long long __M = {prod(mc["m"])}, __N = {prod(mc["n"])}, __B = {prod(mc["batch"])};',
-          f'  const int __T = (int)(({prod(mc["k"])}) / 16);',
+          f'  const long long __K = {prod(mc["k"])};',
+          '  const int __T = (int)((__K + 15) / 16);      // the last tile may be partial: its missing k are staged as zeros',
           '  const long long __tn_n = (__N + 127) / 128, __tiles = ((__M + 127) / 128) * __tn_n;',
           '  const int __tid = threadIdx.x, __lane = __tid & 63, __wave = __tid >> 6, __wm = __wave >> 1, __wn = __wave & 1;',
           '  for (long long __blk = blockIdx.x; __blk < __tiles * __B; __blk += gridDim.x) {',
@@ -874,13 +876,19 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
                   f'        for (int __j = 0; __j < 8; ++__j) __r{x}[__j] = __p{x}[__j][__ko]; }}']
         else:
             b += ['      #pragma unroll', f'      for (int __j = 0; __j < 8; ++__j) __r{x}[__j] = __p{x}[{ktab_}[__buf][__kh + __j]];']
-    b += ['    };', '    auto __stage = [&](int __buf) {']
+    b += ['    };', '    auto __stage = [&](int __buf, int __kt) {']
     for x, lds, vals in (('a', '__As', val_a), ('b', '__Bs', val_b)):
         if mc['parts'][x][2]:
-            b += [f'      {lds}[__buf][(__rw + {16 * j}) * 20 + __kl] = (float)({vals[j]});' for j in range(8)]
+            b += [f'      {{ const bool __in = (long long)__kt * 16 + __kl < __K;']
+            b += [f'        {lds}[__buf][(__rw + {16 * j}) * 20 + __kl] = __in ? (float)({vals[j]}) : 0.f;' for j in range(8)]
+            b += ['      }']
         else:
-            b += [f'      *(__f4*)&{lds}[__buf][__ml * 20 + __kh] = __f4{{(float)({vals[0]}), (float)({vals[1]}), (float)({vals[2]}), (float)({vals[3]})}};',
-                  f'      *(__f4*)&{lds}[__buf][__ml * 20 + __kh + 4] = __f4{{(float)({vals[4]}), (float)({vals[5]}), (float)({vals[6]}), (float)({vals[7]})}};']
+            def guarded(j):
+                return f'(__k0 + {j} < __K ? (float)({vals[j]}) : 0.f)'
+            b += ['      { const long long __k0 = (long long)__kt * 16 + __kh;',
+                  f'        *(__f4*)&{lds}[__buf][__ml * 20 + __kh] = __f4{{{guarded(0)}, {guarded(1)}, {guarded(2)}, {guarded(3)}}};',
+                  f'        *(__f4*)&{lds}[__buf][__ml * 20 + __kh + 4] = __f4{{{guarded(4)}, {guarded(5)}, {guarded(6)}, {guarded(7)}}};',
+                  '      }']
     b += ['    };',
           '    __f16v __acc[2][2];',
           '    #pragma unroll',
@@ -891,7 +899,7 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
           '        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = 0.f;',
           '    const int __row0 = __wm * 64 + (__lane & 31), __col0 = __wn * 64 + (__lane & 31), __kq = (__lane >> 5) * 4;',
           '    __load(0);',
-          '    __stage(0);',
+          '    __stage(0, 0);',
           '    __syncthreads();',
           '    for (int __t = 0; __t < __T; ++__t) {',
           '      const int __buf = __t & 1;',
@@ -913,7 +921,7 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
           '            for (int __j = 0; __j < 2; ++__j)',
           '              __acc[__i][__j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__a[__i][__m], __b[__j][__m], __acc[__i][__j], 0, 0, 0);',
           '      }',
-          '      if (__t + 1 < __T) __stage(__buf ^ 1);          // the other buffer: everybody left it at the last barrier',
+          '      if (__t + 1 < __T) __stage(__buf ^ 1, __t + 1);   // the other buffer: everybody left it at the last barrier',
           '      __syncthreads();',
           '    }',
           '    // accumulator element e of tile (i, j): row i*32 + (e/4)*8 + (lane/32)*4 + e%4, column j*32 + lane%32',

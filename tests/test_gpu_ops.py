@@ -628,21 +628,22 @@ def test_register_tiled_contractions_match_the_oracle(autort, ir, inputs, shapes
 
 
 def test_large_contractions_take_the_register_tiled_variant(autort):
-    """A 2048 x 2048 x 250 fp32 matrix product is large enough for it (a 1024 x 1024 one is not; with k a multiple of
-    16 the matrix-instruction variant takes over); the result is the float64 product's."""
-    note('register-tiled reduce picked for a 2048x2048x250 fp32 matmul')
+    """Without the matrix-instruction variant a 2048 x 2048 x 256 fp32 matrix product is large enough for the
+    register-tiled one (a 1024 x 1024 one is not); the result is the float64 product's."""
+    note('register-tiled reduce picked for a 2048x2048x256 fp32 matmul')
     dev = autort.device()
-    op = autort.export(ir='output0[N, M] +=! input0[N, K] * input1[K, M]', inputs=['input0=float32[N:2048, K:250]', 'input1=float32[K:250, M:2048]'],
+    op = autort.export(ir='output0[N, M] +=! input0[N, K] * input1[K, M]', inputs=['input0=float32[N:2048, K:256]', 'input1=float32[K:256, M:2048]'],
                        name='patch_matmul_2048')
     op.fast_path = None               # the generic lowering is what is tested here
     plan = op.plans[0]
     zero = {n: 0 for n in plan.args}
-    assert plan.choose({'N': 2048, 'K': 250, 'M': 2048}, zero)[0] == plan.variants['patch']
-    assert plan.choose({'N': 2046, 'K': 250, 'M': 2048}, zero)[0] != plan.variants['patch']
-    assert plan.choose({'N': 1024, 'K': 250, 'M': 1024}, zero)[0] != plan.variants['patch']
     assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['matrix']
+    del plan.variants['matrix']
+    assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['patch']
+    assert plan.choose({'N': 2046, 'K': 256, 'M': 2048}, zero)[0] != plan.variants['patch']
+    assert plan.choose({'N': 1024, 'K': 256, 'M': 1024}, zero)[0] != plan.variants['patch']
     g = torch.Generator().manual_seed(2)
-    a, b = torch.randn(2048, 250, generator=g), torch.randn(250, 2048, generator=g)
+    a, b = torch.randn(2048, 256, generator=g), torch.randn(256, 2048, generator=g)
     got = op(a.to(dev), b.to(dev)).cpu()
     want = (a.double() @ b.double()).float()
     assert torch.allclose(got, want, rtol=1e-4, atol=1e-3)
@@ -663,6 +664,10 @@ MATRIX_CASES = [
     ('temp0[K, N] = input0[N, K] + 100; output0[N, M] +=! temp0[K, N] * input1[K, M]',
      ['input0=float32[N:1024, K:512]', 'input1=float32[K:512, M:1024]'], [(1024, 512), (512, 1024)]),
     ('output0[M, N] +=! input0[N, K] * input1[K, M]', ['input0=float32[N:1030, K:64]', 'input1=float32[K:64, M:1024]'], [(1030, 64), (64, 1024)]),
+    # k that is no multiple of the tile: a first-layer convolution (3 channels, 7 x 7, stride 2: k = 147), a product with k = 250
+    ('output0[N, F, HO, WO] +=! input0[N, C, HO * 2 + KH, WO * 2 + KW] * input1[F, C, KH, KW] where HO in 29, WO in 29',
+     ['input0=float32[N:10, C:3, H:64, W:64]', 'input1=float32[F:64, C:3, KH:7, KW:7]'], [(10, 3, 64, 64), (64, 3, 7, 7)]),
+    ('output0[N, M] +=! input0[N, K] * input1[M, K]', ['input0=float32[N:1024, K:250]', 'input1=float32[M:1024, K:250]'], [(1024, 250), (1024, 250)]),
 ]
 
 
