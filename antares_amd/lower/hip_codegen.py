@@ -248,23 +248,31 @@ class KernelPlan:
             return 0
         return total // self.row_vec
 
-    def _matrix_blocks(self, env: Dict[str, int]) -> int:
-        """Blocks of the matrix-instruction variant (128 x 128 outputs each, per batch), 0 when it does not apply:
-        there must be enough tiles and enough k to pay for staging them."""
+    def _matrix_choice(self, env: Dict[str, int]) -> Tuple[Optional[str], int]:
+        """(variant tag, blocks) of the matrix-instruction variants, (None, 0) when they do not apply: there must be
+        enough k to pay for staging it, and enough tiles - of 128 x 128 outputs when those fill the chip, else of
+        64 x 64 (a block multiplies a quarter as much per k, so small products spread over four times the compute
+        units)."""
         if self.matrix is None or 'matrix' not in self.variants:
-            return 0
+            return None, 0
         def prod(key):
             n = 1
             for e in self.matrix[key]:
                 n *= e if isinstance(e, int) else env[e]
             return n
         M, N, B, K = prod('m'), prod('n'), prod('batch'), prod('k')
-        if K < 32 or M < 64 or N < 64:
-            return 0
-        blocks = ((M + 127) // 128) * ((N + 127) // 128) * B
-        if blocks < 64 or blocks > MAX_GRID * 64:
-            return 0
-        return blocks
+        if K < 32 or M < 32 or N < 32:
+            return None, 0
+        big = ((M + 127) // 128) * ((N + 127) // 128) * B
+        small = ((M + 63) // 64) * ((N + 63) // 64) * B
+        if big >= 192 and big <= MAX_GRID * 64:
+            return 'matrix', big
+        if 'matrix64' in self.variants and small >= 16 and small <= MAX_GRID * 64:
+            return 'matrix64', small
+        return None, 0
+
+    def _matrix_blocks(self, env: Dict[str, int]) -> int:
+        return self._matrix_choice(env)[1]
 
     def _patches(self, env: Dict[str, int], total: int) -> int:
         """Threads of the register-tiled reduce variant for these extents, 0 when it does not apply."""
@@ -302,9 +310,9 @@ class KernelPlan:
         if self.kind == 'scatter':
             return self.variants['scalar'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
         # reduce
-        blocks = self._matrix_blocks(env)
-        if blocks:
-            return self.variants['matrix'], blocks, BLOCK
+        tag, blocks = self._matrix_choice(env)
+        if tag:
+            return self.variants[tag], blocks, BLOCK
         patches = self._patches(env, total)
         if patches >= 131072 and red >= 8:           # two wavefronts per SIMD and more: below that one output per thread hides latency better
             return self.variants['patch'], min((patches + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
@@ -344,8 +352,8 @@ class KernelPlan:
             tags += [('thread', total), ('wave', (total + waves_per_block - 1) // waves_per_block * BLOCK), ('block', total * BLOCK)]
             if self._patches(env, total):
                 tags.append(('patch', self._patches(env, total)))
-            if self._matrix_blocks(env):
-                tags.append(('matrix', self._matrix_blocks(env) * BLOCK))
+            if self._matrix_choice(env)[0]:
+                tags.append((self._matrix_choice(env)[0], self._matrix_blocks(env) * BLOCK))
         out = []
         for tag, work in tags:
             if tag not in self.variants:
@@ -786,14 +794,15 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
         mc = _matrix_contraction(st, tensors)
         if mc is not None:
             src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_m', mc))
-            variants['matrix'] = name + '_m'
+            src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_m64', mc, TS=64))
+            variants['matrix'], variants['matrix64'] = name + '_m', name + '_m64'
             ext = dict(st.data_axes + st.reduce_axes)
             plan.matrix = {key: [ext[a] for a in mc[key]] for key in ('m', 'n', 'batch', 'k')}
 
     return '\n\n'.join(src), plan
 
 
-def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
+def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128) -> str:
     """A sum of products of two loads on v_mfma_f32_32x32x2_f32 (the reference's counterpart: its tiled schedule for
     contractions, backends/c-rocm/schedule/standard/algo_tiling.py:35-98, on the vector units).  A block of 256
     threads = 2 x 2 wavefronts owns 128 rows x 128 columns of one batch, where a row is a point of the axes only
@@ -804,8 +813,10 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
     Both operands are staged in LDS as [row or column][k] and fed to the matrix instruction exactly as the fp32
     GEMM kernel of the library feeds it; rows, columns and batches past the extents are clamped on the way in and
     cut on the way out; the k a last partial tile lacks are staged as zeros (their addresses wrap into the
-    tensors)."""
+    tensors).  TS = 64 gives blocks of 64 x 64 outputs (a wavefront then owns one 32 x 32 tile): four times the
+    blocks for products too small to fill the chip with the big ones."""
     la, lb = mc['la'], mc['lb']
+    NT, PER, HALF = TS // 64, TS // 16, TS // 2       # accumulator tiles per wavefront and direction, elements a thread stages per operand and tile, rows of a wavefront
     ta, tb, oct_ = HIP_TYPE[tensors[la.name].dtype], HIP_TYPE[tensors[lb.name].dtype], HIP_TYPE[st.out_dtype]
     plain = ExprEmitter(tensors)
     ext = dict(st.data_axes + st.reduce_axes)
@@ -821,32 +832,32 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
     out_axes = [a for a, _ in st.data_axes]
     rows_of_out = plain.offset(st.output, [a if (a in mc['m'] or a in mc['batch']) else '0' for a in out_axes])
     cols_of_out = plain.offset(st.output, [a if a in mc['n'] else '0' for a in out_axes])
-    val_a = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__ra[{j}]').expr(mc['fa']) for j in range(8)]
-    val_b = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__rb[{j}]').expr(mc['fb']) for j in range(8)]
+    val_a = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__ra[{j}]').expr(mc['fa']) for j in range(PER)]
+    val_b = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__rb[{j}]').expr(mc['fb']) for j in range(PER)]
     b = [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st)
     b += ['  typedef float __f16v __attribute__((ext_vector_type(16)));',
           '  typedef float __f4 __attribute__((ext_vector_type(4)));',
-          '  __shared__ __attribute__((aligned(16))) float __As[2][128 * 20];     // [row][k], 16 k and 4 floats of padding per row',
-          '  __shared__ __attribute__((aligned(16))) float __Bs[2][128 * 20];     // [column][k]',
-          '  __shared__ long long __am[128], __bn[128], __cm[128], __cn[128], __ak[2][16], __bk[2][16];',
+          f'  __shared__ __attribute__((aligned(16))) float __As[2][{TS} * 20];     // [row][k], 16 k and 4 floats of padding per row',
+          f'  __shared__ __attribute__((aligned(16))) float __Bs[2][{TS} * 20];     // [column][k]',
+          f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][16], __bk[2][16];',
           f'  const long long __M = {prod(mc["m"])}, __N = {prod(mc["n"])}, __B = {prod(mc["batch"])};',
           f'  const long long __K = {prod(mc["k"])};',
           '  const int __T = (int)((__K + 15) / 16);      // the last tile may be partial: its missing k are staged as zeros',
-          '  const long long __tn_n = (__N + 127) / 128, __tiles = ((__M + 127) / 128) * __tn_n;',
+          f'  const long long __tn_n = (__N + {TS - 1}) / {TS}, __tiles = ((__M + {TS - 1}) / {TS}) * __tn_n;',
           '  const int __tid = threadIdx.x, __lane = __tid & 63, __wave = __tid >> 6, __wm = __wave >> 1, __wn = __wave & 1;',
           '  for (long long __blk = blockIdx.x; __blk < __tiles * __B; __blk += gridDim.x) {',
           '    const long long __t0 = __blk % __tiles, __tm = __t0 / __tn_n, __tn = __t0 % __tn_n;']
     b += decompose('__blk / __tiles', mc['batch'], '    ')
-    b += ['    if (__tid < 128) {                            // row offsets of the first operand and of the output',
-          '      long long __row = __tm * 128 + __tid;',
+    b += [f'    if (__tid < {TS}) {{                            // row offsets of the first operand and of the output',
+          f'      long long __row = __tm * {TS} + __tid;',
           '      if (__row >= __M) __row = __M - 1;']
     b += decompose('__row', mc['m'], '      ')
     b += [f'      __am[__tid] = {mc["parts"]["a"][0]};', f'      __cm[__tid] = {rows_of_out};',
-          '    } else {                                      // column offsets of the second operand and of the output',
-          '      long long __colq = __tn * 128 + (__tid - 128);',
+          f'    }} else if (__tid < {2 * TS}) {{                  // column offsets of the second operand and of the output',
+          f'      long long __colq = __tn * {TS} + (__tid - {TS});',
           '      if (__colq >= __N) __colq = __N - 1;']
     b += decompose('__colq', mc['n'], '      ')
-    b += [f'      __bn[__tid - 128] = {mc["parts"]["b"][0]};', f'      __cn[__tid - 128] = {cols_of_out};',
+    b += [f'      __bn[__tid - {TS}] = {mc["parts"]["b"][0]};', f'      __cn[__tid - {TS}] = {cols_of_out};',
           '    }',
           '    auto __ktab = [&](int __kt, int __buf) {       // k offsets of tile __kt: 16 for each operand',
           '      if (__tid < 32) {',
@@ -859,45 +870,45 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
           '    __ktab(0, 0);',
           '    if (__T > 1) __ktab(1, 1);',
           '    __syncthreads();',
-          '    const int __ml = __tid & 127, __kh = (__tid >> 7) * 8;     // lanes along rows: 8 k of one row (column) per thread',
-          '    const int __kl = __tid & 15, __rw = __tid >> 4;             // lanes along k: one k of 8 rows (columns) per thread',
+          f'    const int __ml = __tid & {TS - 1}, __kh = (__tid / {TS}) * {PER};     // lanes along rows: {PER} k of one row (column) per thread',
+          f'    const int __kl = __tid & 15, __rw = __tid >> 4;             // lanes along k: one k of {PER} rows (columns) per thread',
           '    (void)__ml; (void)__kh; (void)__kl; (void)__rw;']
     for x, ld, ct, tab, ktab_, lds, vals in (('a', la, ta, '__am', '__ak', '__As', val_a), ('b', lb, tb, '__bn', '__bk', '__Bs', val_b)):
         if mc['parts'][x][2]:
-            b += [f'    const {ct}* __p{x}[8];', '    #pragma unroll',
-                  f'    for (int __j = 0; __j < 8; ++__j) __p{x}[__j] = {ld.name} + {tab}[__rw + 16 * __j];']
+            b += [f'    const {ct}* __p{x}[{PER}];', '    #pragma unroll',
+                  f'    for (int __j = 0; __j < {PER}; ++__j) __p{x}[__j] = {ld.name} + {tab}[__rw + 16 * __j];']
         else:
             b.append(f'    const {ct}* __p{x} = {ld.name} + {tab}[__ml];')
-        b.append(f'    {ct} __r{x}[8];')
+        b.append(f'    {ct} __r{x}[{PER}];')
     b += ['    auto __load = [&](int __buf) {']
     for x, ktab_ in (('a', '__ak'), ('b', '__bk')):
         if mc['parts'][x][2]:
             b += [f'      {{ const long long __ko = {ktab_}[__buf][__kl];', '        #pragma unroll',
-                  f'        for (int __j = 0; __j < 8; ++__j) __r{x}[__j] = __p{x}[__j][__ko]; }}']
+                  f'        for (int __j = 0; __j < {PER}; ++__j) __r{x}[__j] = __p{x}[__j][__ko]; }}']
         else:
-            b += ['      #pragma unroll', f'      for (int __j = 0; __j < 8; ++__j) __r{x}[__j] = __p{x}[{ktab_}[__buf][__kh + __j]];']
+            b += ['      #pragma unroll', f'      for (int __j = 0; __j < {PER}; ++__j) __r{x}[__j] = __p{x}[{ktab_}[__buf][__kh + __j]];']
     b += ['    };', '    auto __stage = [&](int __buf, int __kt) {']
     for x, lds, vals in (('a', '__As', val_a), ('b', '__Bs', val_b)):
         if mc['parts'][x][2]:
             b += [f'      {{ const bool __in = (long long)__kt * 16 + __kl < __K;']
-            b += [f'        {lds}[__buf][(__rw + {16 * j}) * 20 + __kl] = __in ? (float)({vals[j]}) : 0.f;' for j in range(8)]
+            b += [f'        {lds}[__buf][(__rw + {16 * j}) * 20 + __kl] = __in ? (float)({vals[j]}) : 0.f;' for j in range(PER)]
             b += ['      }']
         else:
             def guarded(j):
                 return f'(__k0 + {j} < __K ? (float)({vals[j]}) : 0.f)'
-            b += ['      { const long long __k0 = (long long)__kt * 16 + __kh;',
-                  f'        *(__f4*)&{lds}[__buf][__ml * 20 + __kh] = __f4{{{guarded(0)}, {guarded(1)}, {guarded(2)}, {guarded(3)}}};',
-                  f'        *(__f4*)&{lds}[__buf][__ml * 20 + __kh + 4] = __f4{{{guarded(4)}, {guarded(5)}, {guarded(6)}, {guarded(7)}}};',
-                  '      }']
+            b += ['      { const long long __k0 = (long long)__kt * 16 + __kh;']
+            for q in range(PER // 4):
+                b += [f'        *(__f4*)&{lds}[__buf][__ml * 20 + __kh + {4 * q}] = __f4{{{guarded(4 * q)}, {guarded(4 * q + 1)}, {guarded(4 * q + 2)}, {guarded(4 * q + 3)}}};']
+            b += ['      }']
     b += ['    };',
-          '    __f16v __acc[2][2];',
+          f'    __f16v __acc[{NT}][{NT}];',
           '    #pragma unroll',
-          '    for (int __i = 0; __i < 2; ++__i)',
+          f'    for (int __i = 0; __i < {NT}; ++__i)',
           '      #pragma unroll',
-          '      for (int __j = 0; __j < 2; ++__j)',
+          f'      for (int __j = 0; __j < {NT}; ++__j)',
           '        #pragma unroll',
           '        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = 0.f;',
-          '    const int __row0 = __wm * 64 + (__lane & 31), __col0 = __wn * 64 + (__lane & 31), __kq = (__lane >> 5) * 4;',
+          f'    const int __row0 = __wm * {HALF} + (__lane & 31), __col0 = __wn * {HALF} + (__lane & 31), __kq = (__lane >> 5) * 4;',
           '    __load(0);',
           '    __stage(0, 0);',
           '    __syncthreads();',
@@ -907,18 +918,18 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
           '      if (__t + 2 < __T) __ktab(__t + 2, __buf);       // its k offsets were read a tile ago',
           '      #pragma unroll',
           '      for (int __g = 0; __g < 2; ++__g) {',
-          '        __f4 __a[2], __b[2];',
+          f'        __f4 __a[{NT}], __b[{NT}];',
           '        #pragma unroll',
-          '        for (int __i = 0; __i < 2; ++__i) {',
+          f'        for (int __i = 0; __i < {NT}; ++__i) {{',
           '          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * 20 + __g * 8 + __kq];',
           '          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * 20 + __g * 8 + __kq];',
           '        }',
           '        #pragma unroll',
           '        for (int __m = 0; __m < 4; ++__m)',
           '          #pragma unroll',
-          '          for (int __i = 0; __i < 2; ++__i)',
+          f'          for (int __i = 0; __i < {NT}; ++__i)',
           '            #pragma unroll',
-          '            for (int __j = 0; __j < 2; ++__j)',
+          f'            for (int __j = 0; __j < {NT}; ++__j)',
           '              __acc[__i][__j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__a[__i][__m], __b[__j][__m], __acc[__i][__j], 0, 0, 0);',
           '      }',
           '      if (__t + 1 < __T) __stage(__buf ^ 1, __t + 1);   // the other buffer: everybody left it at the last barrier',
@@ -926,14 +937,14 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc) -> str:
           '    }',
           '    // accumulator element e of tile (i, j): row i*32 + (e/4)*8 + (lane/32)*4 + e%4, column j*32 + lane%32',
           '    #pragma unroll',
-          '    for (int __i = 0; __i < 2; ++__i)',
+          f'    for (int __i = 0; __i < {NT}; ++__i)',
           '      #pragma unroll',
-          '      for (int __j = 0; __j < 2; ++__j) {',
-          '        const int __c = __wn * 64 + __j * 32 + (__lane & 31);',
+          f'      for (int __j = 0; __j < {NT}; ++__j) {{',
+          f'        const int __c = __wn * {HALF} + __j * 32 + (__lane & 31);',
           '        #pragma unroll',
           '        for (int __e = 0; __e < 16; ++__e) {',
-          '          const int __r = __wm * 64 + __i * 32 + (__e >> 2) * 8 + (__lane >> 5) * 4 + (__e & 3);',
-          f'          if (__tm * 128 + __r < __M && __tn * 128 + __c < __N) {st.output}[__cm[__r] + __cn[__c]] = ({oct_})__acc[__i][__j][__e];',
+          f'          const int __r = __wm * {HALF} + __i * 32 + (__e >> 2) * 8 + (__lane >> 5) * 4 + (__e & 3);',
+          f'          if (__tm * {TS} + __r < __M && __tn * {TS} + __c < __N) {st.output}[__cm[__r] + __cn[__c]] = ({oct_})__acc[__i][__j][__e];',
           '        }',
           '      }',
           '    __syncthreads();                               // the tables and buffers are rewritten by the next tile',

@@ -638,7 +638,7 @@ def test_large_contractions_take_the_register_tiled_variant(autort):
     plan = op.plans[0]
     zero = {n: 0 for n in plan.args}
     assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['matrix']
-    del plan.variants['matrix']
+    del plan.variants['matrix'], plan.variants['matrix64']
     assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['patch']
     assert plan.choose({'N': 2046, 'K': 256, 'M': 2048}, zero)[0] != plan.variants['patch']
     assert plan.choose({'N': 1024, 'K': 256, 'M': 1024}, zero)[0] != plan.variants['patch']
@@ -687,66 +687,30 @@ def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, ir, in
     for spec, shape in zip(inputs, shapes):
         for d, v in zip(spec.split('[', 1)[1].rstrip(']').split(','), shape):
             env[d.split(':')[0].strip()] = v
-    assert 'matrix' in plan.variants and plan.choose(env, {n: 0 for n in plan.args})[0] == plan.variants['matrix']
+    assert plan.choose(env, {n: 0 for n in plan.args})[0] in (plan.variants['matrix'], plan.variants['matrix64'])
     assert plan.row_group is None                 # nothing else takes the statement
     g = torch.Generator().manual_seed(len(ir))
     tensors = [torch.randn(shape, generator=g).to(torch.float16 if 'float16' in spec else torch.float32) for spec, shape in zip(inputs, shapes)]
-    got = op(*[t.to(dev) for t in tensors]).cpu().numpy()
     names = [spec.split('=')[0] for spec in inputs]
     want = CpuModule(parse_program(ir, inputs), fast_math=False)(**{n: t.numpy() for n, t in zip(names, tensors)})['output0']
     K = 1
     for ax, e in plan.reduce_axes:
         K *= e if isinstance(e, int) else env[e]
     scale = 100.0 if '+ 100' in ir else 1.0
-    assert got.shape == want.shape
-    assert np.allclose(got, want, rtol=1e-4, atol=2e-5 * scale * K ** 0.5 * 4), np.abs(got - want).max()
+    tol = 2e-5 * scale * K ** 0.5 * 4
+    M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
+    rule = plan.choose
+    for tag, side in (('matrix', 128), ('matrix64', 64)):       # blocks of 128 x 128 and of 64 x 64 outputs
+        blocks = ((M + side - 1) // side) * ((N + side - 1) // side) * B
+        plan.choose = lambda env_, ptrs, tag=tag, blocks=blocks: (plan.variants[tag], blocks, 256)
+        got = op(*[t.to(dev) for t in tensors]).cpu().numpy()
+        assert got.shape == want.shape
+        assert np.allclose(got, want, rtol=1e-4, atol=tol), (tag, np.abs(got - want).max())
     # the same statement through the register-tiled variant
-    del plan.variants['matrix']
+    plan.choose = rule
+    del plan.variants['matrix'], plan.variants['matrix64']
     apart = op(*[t.to(dev) for t in tensors]).cpu().numpy()
-    assert np.allclose(got, apart, rtol=1e-4, atol=2e-5 * scale * K ** 0.5 * 4)
-
-
-@pytest.mark.parametrize('M,N,K', [(512, 1024, 32), (1000, 1028, 96), (4096, 4096, 512), (129, 8192, 64), (2048, 2048, 2048)])
-def test_fp32_gemm_on_the_matrix_cores_matches_the_float64_product(autort, M, N, K):
-    """`C[M,N] +=! A[M,K] * B[K,N]` in float32 goes to art_gemm_f32 (edge tiles in M and N included); the result is
-    the float64 product's to fp32 accuracy, and identity / one-hot operands pin operand order and transposition."""
-    note(f'gemm_f32 {M}x{N}x{K}')
-    dev = autort.device()
-    op = autort.export(ir='c[M, N] +=! a[M, K] * b[K, N]', inputs=[f'a=float32[M:{M}, K:{K}]', f'b=float32[K:{K}, N:{N}]'], name=f'gemm_f32_{M}_{N}_{K}')
-    assert op.fast_path is not None
-    g = torch.Generator().manual_seed(M + N + K)
-    a, b = torch.randn(M, K, generator=g), torch.randn(K, N, generator=g)
-    got = op(a.to(dev), b.to(dev)).cpu()
-    want = a.double() @ b.double()
-    # fp32 sums of K products of N(0,1) values: error about sqrt(K) * 2^-24 * |terms|
-    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5 * max(1.0, K ** 0.5)), (got.double() - want).abs().max()
-    if M == 512:
-        sel = torch.zeros(M, K)
-        sel[torch.arange(M), torch.arange(M) % K] = 1.0              # row m of the result = row m % K of b
-        assert torch.equal(op(sel.to(dev), b.to(dev)).cpu(), b[torch.arange(M) % K])
-    # shapes the kernel does not take run through the generic lowering, same operator
-    small = autort.export(ir='c[M, N] +=! a[M, K] * b[K, N]', inputs=['a=float32[M:40, K:24]', 'b=float32[K:24, N:36]'], name='gemm_f32_small')
-    a2, b2 = torch.randn(40, 24, generator=g), torch.randn(24, 36, generator=g)
-    assert torch.allclose(small(a2.to(dev), b2.to(dev)).cpu().double(), a2.double() @ b2.double(), rtol=1e-5, atol=1e-5)
-
-
-@pytest.mark.parametrize('B,M,N,K', [(3, 1024, 512, 512), (5, 130, 1028, 64), (16, 256, 256, 128)])
-def test_batched_fp32_gemm_on_the_matrix_cores_matches_the_float64_products(autort, B, M, N, K):
-    """`C[B,M,N] +=! A[B,M,K] * B[B,K,N]` (AntaresIR.md:121, written there with other names) goes to
-    art_gemm_f32_batched: every product of the batch is the float64 product's to fp32 accuracy, and one batch with
-    all-zero operands stays zero (no product reads its neighbour's operands)."""
-    note(f'batched gemm_f32 {B}x{M}x{N}x{K}')
-    dev = autort.device()
-    op = autort.export(ir='output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]',
-                       inputs=[f'input0=float32[B:{B}, N:{M}, K:{K}]', f'input1=float32[B:{B}, K:{K}, M:{N}]'], name=f'bmm_f32_{B}_{M}_{N}_{K}')
-    assert op.fast_path is not None
-    g = torch.Generator().manual_seed(B + M + N + K)
-    a, b = torch.randn(B, M, K, generator=g), torch.randn(B, K, N, generator=g)
-    a[1].zero_()
-    got = op(a.to(dev), b.to(dev)).cpu()
-    want = a.double() @ b.double()
-    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5 * max(1.0, K ** 0.5)), (got.double() - want).abs().max()
-    assert not got[1].any() and got[0].any() and got[2].any()
+    assert np.allclose(got, apart, rtol=1e-4, atol=tol)
 
 
 ROW_GROUP_CASES = [
