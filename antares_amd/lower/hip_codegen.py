@@ -817,6 +817,7 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     blocks for products too small to fill the chip with the big ones."""
     la, lb = mc['la'], mc['lb']
     NT, PER, HALF = TS // 64, TS // 16, TS // 2       # accumulator tiles per wavefront and direction, elements a thread stages per operand and tile, rows of a wavefront
+    DEPTH = 2 if TS == 64 else 1                      # tiles on their way in registers: small blocks have nothing else to hide a load behind
     ta, tb, oct_ = HIP_TYPE[tensors[la.name].dtype], HIP_TYPE[tensors[lb.name].dtype], HIP_TYPE[st.out_dtype]
     plain = ExprEmitter(tensors)
     ext = dict(st.data_axes + st.reduce_axes)
@@ -824,16 +825,21 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     def prod(names):
         return ' * '.join(f'(long long)__ext_{a}' for a in names) or '1LL'
 
-    def decompose(var, names, indent):
-        out = [f'{indent}long long __q = {var};']
+    def decompose(var, names, indent, wide=True):
+        # 64-bit division costs some hundred instructions; k (walked once per tile by one wavefront, on every
+        # other wavefront's way to the barrier) always fits 32 bits
+        out = [f'{indent}long long __q = {var};' if wide else f'{indent}unsigned int __q = (unsigned int)({var});']
         for a in reversed(names):
-            out.append(f'{indent}const int {a} = (int)(__q % __ext_{a}); __q /= __ext_{a}; (void){a};')
+            if wide:
+                out.append(f'{indent}const int {a} = (int)(__q % __ext_{a}); __q /= __ext_{a}; (void){a};')
+            else:
+                out.append(f'{indent}const int {a} = (int)(__q % (unsigned int)__ext_{a}); __q /= (unsigned int)__ext_{a}; (void){a};')
         return out
     out_axes = [a for a, _ in st.data_axes]
     rows_of_out = plain.offset(st.output, [a if (a in mc['m'] or a in mc['batch']) else '0' for a in out_axes])
     cols_of_out = plain.offset(st.output, [a if a in mc['n'] else '0' for a in out_axes])
-    val_a = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__ra[{j}]').expr(mc['fa']) for j in range(PER)]
-    val_b = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__rb[{j}]').expr(mc['fb']) for j in range(PER)]
+    val_a = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__ra[__S][{j}]').expr(mc['fa']) for j in range(PER)]
+    val_b = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__rb[__S][{j}]').expr(mc['fb']) for j in range(PER)]
     b = [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st)
     b += ['  typedef float __f16v __attribute__((ext_vector_type(16)));',
           '  typedef float __f4 __attribute__((ext_vector_type(4)));',
@@ -862,7 +868,7 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           '    auto __ktab = [&](int __kt, int __buf) {       // k offsets of tile __kt: 16 for each operand',
           '      if (__tid < 32) {',
           '        const long long __kk = (long long)__kt * 16 + (__tid & 15);']
-    b += decompose('__kk', mc['k'], '        ')
+    b += decompose('__kk', mc['k'], '        ', wide=False)
     b += [f'        if (__tid < 16) __ak[__buf][__tid] = {mc["parts"]["a"][1]};',
           f'        else __bk[__buf][__tid - 16] = {mc["parts"]["b"][1]};',
           '      }',
@@ -879,15 +885,15 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
                   f'    for (int __j = 0; __j < {PER}; ++__j) __p{x}[__j] = {ld.name} + {tab}[__rw + 16 * __j];']
         else:
             b.append(f'    const {ct}* __p{x} = {ld.name} + {tab}[__ml];')
-        b.append(f'    {ct} __r{x}[{PER}];')
-    b += ['    auto __load = [&](int __buf) {']
+        b.append(f'    {ct} __r{x}[{DEPTH}][{PER}];')
+    b += ['    auto __load = [&](auto __set, int __buf) {', '      constexpr int __S = decltype(__set)::value;']
     for x, ktab_ in (('a', '__ak'), ('b', '__bk')):
         if mc['parts'][x][2]:
             b += [f'      {{ const long long __ko = {ktab_}[__buf][__kl];', '        #pragma unroll',
-                  f'        for (int __j = 0; __j < {PER}; ++__j) __r{x}[__j] = __p{x}[__j][__ko]; }}']
+                  f'        for (int __j = 0; __j < {PER}; ++__j) __r{x}[__S][__j] = __p{x}[__j][__ko]; }}']
         else:
-            b += ['      #pragma unroll', f'      for (int __j = 0; __j < {PER}; ++__j) __r{x}[__j] = __p{x}[{ktab_}[__buf][__kh + __j]];']
-    b += ['    };', '    auto __stage = [&](int __buf, int __kt) {']
+            b += ['      #pragma unroll', f'      for (int __j = 0; __j < {PER}; ++__j) __r{x}[__S][__j] = __p{x}[{ktab_}[__buf][__kh + __j]];']
+    b += ['    };', '    auto __stage = [&](auto __set, int __buf, int __kt) {', '      constexpr int __S = decltype(__set)::value; (void)__S;']
     for x, lds, vals in (('a', '__As', val_a), ('b', '__Bs', val_b)):
         if mc['parts'][x][2]:
             b += [f'      {{ const bool __in = (long long)__kt * 16 + __kl < __K;']
@@ -909,13 +915,7 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           '        #pragma unroll',
           '        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = 0.f;',
           f'    const int __row0 = __wm * {HALF} + (__lane & 31), __col0 = __wn * {HALF} + (__lane & 31), __kq = (__lane >> 5) * 4;',
-          '    __load(0);',
-          '    __stage(0, 0);',
-          '    __syncthreads();',
-          '    for (int __t = 0; __t < __T; ++__t) {',
-          '      const int __buf = __t & 1;',
-          '      if (__t + 1 < __T) __load(__buf ^ 1);           // tile t + 1 travels while tile t is multiplied',
-          '      if (__t + 2 < __T) __ktab(__t + 2, __buf);       // its k offsets were read a tile ago',
+          '    auto __multiply = [&](int __buf) {',
           '      #pragma unroll',
           '      for (int __g = 0; __g < 2; ++__g) {',
           f'        __f4 __a[{NT}], __b[{NT}];',
@@ -932,9 +932,44 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           f'            for (int __j = 0; __j < {NT}; ++__j)',
           '              __acc[__i][__j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__a[__i][__m], __b[__j][__m], __acc[__i][__j], 0, 0, 0);',
           '      }',
-          '      if (__t + 1 < __T) __stage(__buf ^ 1, __t + 1);   // the other buffer: everybody left it at the last barrier',
-          '      __syncthreads();',
-          '    }',
+          '    };']
+    if DEPTH == 1:
+        b += ['    __load(art_ic<0>{}, 0);',
+              '    __stage(art_ic<0>{}, 0, 0);',
+              '    __syncthreads();',
+              '    for (int __t = 0; __t < __T; ++__t) {',
+              '      const int __buf = __t & 1;',
+              '      if (__t + 1 < __T) __load(art_ic<0>{}, __buf ^ 1);    // tile t + 1 travels while tile t is multiplied',
+              '      if (__t + 2 < __T) __ktab(__t + 2, __buf);            // its k offsets were read a tile ago',
+              '      __multiply(__buf);',
+              '      if (__t + 1 < __T) __stage(art_ic<0>{}, __buf ^ 1, __t + 1);   // the other buffer: everybody left it at the last barrier',
+              '      __syncthreads();',
+              '    }']
+    else:
+        b += ['    // Tile t is multiplied out of LDS buffer t % 2 and came through register set t % 2.  While it is multiplied,',
+              '    // tile t + 1 waits in the other register set and tile t + 2 is asked for into the set tile t has left; the k',
+              '    // offsets of tile t + 3 go into the table that the loads of tile t + 1 read one barrier ago.',
+              '    __load(art_ic<0>{}, 0);',
+              '    if (__T > 1) __load(art_ic<1>{}, 1);',
+              '    __syncthreads();                               // everybody has read the k offsets of tile 0',
+              '    if (__T > 2) __ktab(2, 0);',
+              '    __stage(art_ic<0>{}, 0, 0);',
+              '    __syncthreads();',
+              '    for (int __t = 0; __t < __T; __t += 2) {',
+              '      if (__t + 2 < __T) __load(art_ic<0>{}, 0);',
+              '      if (__t + 3 < __T) __ktab(__t + 3, 1);',
+              '      __multiply(0);',
+              '      if (__t + 1 < __T) __stage(art_ic<1>{}, 1, __t + 1);    // the other buffer: everybody left it at the last barrier',
+              '      __syncthreads();',
+              '      if (__t + 1 < __T) {',
+              '        if (__t + 3 < __T) __load(art_ic<1>{}, 1);',
+              '        if (__t + 4 < __T) __ktab(__t + 4, 0);',
+              '        __multiply(1);',
+              '        if (__t + 2 < __T) __stage(art_ic<0>{}, 0, __t + 2);',
+              '        __syncthreads();',
+              '      }',
+              '    }']
+    b += [
           '    // accumulator element e of tile (i, j): row i*32 + (e/4)*8 + (lane/32)*4 + e%4, column j*32 + lane%32',
           '    #pragma unroll',
           f'    for (int __i = 0; __i < {NT}; ++__i)',

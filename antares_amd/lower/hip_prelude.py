@@ -95,6 +95,9 @@ template <class T, class Op> ART_DEV T art_wave_reduce(T v, Op op) {
   }
 }
 
+// A compile-time integer as a function argument (selects a register set without run-time indexing).
+template <int V> struct art_ic { static constexpr int value = V; };
+
 // Reduction over a block of 256 threads (4 wavefronts); `smem` holds 4 values.
 template <class T, class Op> ART_DEV T art_block_reduce(T v, Op op, T* smem) {
   v = art_wave_reduce(v, op);
