@@ -816,7 +816,9 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     tensors).  TS = 64 gives blocks of 64 x 64 outputs (a wavefront then owns one 32 x 32 tile): four times the
     blocks for products too small to fill the chip with the big ones."""
     la, lb = mc['la'], mc['lb']
-    NT, PER, HALF = TS // 64, TS // 16, TS // 2       # accumulator tiles per wavefront and direction, elements a thread stages per operand and tile, rows of a wavefront
+    BK = 32 if TS == 64 else 16                       # k per tile: the small blocks take twice the k per barrier
+    LD, RS = BK + 4, BLOCK // BK                      # floats per row of a staged tile (16-byte aligned, rows on distinct banks); rows between a lane's elements when lanes walk k
+    NT, PER, HALF = TS // 64, TS * BK // BLOCK, TS // 2   # accumulator tiles per wavefront and direction, elements a thread stages per operand and tile, rows of a wavefront
     DEPTH = 2 if TS == 64 else 1                      # tiles on their way in registers: small blocks have nothing else to hide a load behind
     ta, tb, oct_ = HIP_TYPE[tensors[la.name].dtype], HIP_TYPE[tensors[lb.name].dtype], HIP_TYPE[st.out_dtype]
     plain = ExprEmitter(tensors)
@@ -843,12 +845,12 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     b = [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st)
     b += ['  typedef float __f16v __attribute__((ext_vector_type(16)));',
           '  typedef float __f4 __attribute__((ext_vector_type(4)));',
-          f'  __shared__ __attribute__((aligned(16))) float __As[2][{TS} * 20];     // [row][k], 16 k and 4 floats of padding per row',
-          f'  __shared__ __attribute__((aligned(16))) float __Bs[2][{TS} * 20];     // [column][k]',
-          f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][16], __bk[2][16];',
+          f'  __shared__ __attribute__((aligned(16))) float __As[2][{TS} * {LD}];     // [row][k], {BK} k and 4 floats of padding per row',
+          f'  __shared__ __attribute__((aligned(16))) float __Bs[2][{TS} * {LD}];     // [column][k]',
+          f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][{BK}], __bk[2][{BK}];',
           f'  const long long __M = {prod(mc["m"])}, __N = {prod(mc["n"])}, __B = {prod(mc["batch"])};',
           f'  const long long __K = {prod(mc["k"])};',
-          '  const int __T = (int)((__K + 15) / 16);      // the last tile may be partial: its missing k are staged as zeros',
+          f'  const int __T = (int)((__K + {BK - 1}) / {BK});      // the last tile may be partial: its missing k are staged as zeros',
           f'  const long long __tn_n = (__N + {TS - 1}) / {TS}, __tiles = ((__M + {TS - 1}) / {TS}) * __tn_n;',
           '  const int __tid = threadIdx.x, __lane = __tid & 63, __wave = __tid >> 6, __wm = __wave >> 1, __wn = __wave & 1;',
           '  for (long long __blk = blockIdx.x; __blk < __tiles * __B; __blk += gridDim.x) {',
@@ -865,24 +867,24 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     b += decompose('__colq', mc['n'], '      ')
     b += [f'      __bn[__tid - {TS}] = {mc["parts"]["b"][0]};', f'      __cn[__tid - {TS}] = {cols_of_out};',
           '    }',
-          '    auto __ktab = [&](int __kt, int __buf) {       // k offsets of tile __kt: 16 for each operand',
-          '      if (__tid < 32) {',
-          '        const long long __kk = (long long)__kt * 16 + (__tid & 15);']
+          f'    auto __ktab = [&](int __kt, int __buf) {{       // k offsets of tile __kt: {BK} for each operand',
+          f'      if (__tid < {2 * BK}) {{',
+          f'        const long long __kk = (long long)__kt * {BK} + (__tid & {BK - 1});']
     b += decompose('__kk', mc['k'], '        ', wide=False)
-    b += [f'        if (__tid < 16) __ak[__buf][__tid] = {mc["parts"]["a"][1]};',
-          f'        else __bk[__buf][__tid - 16] = {mc["parts"]["b"][1]};',
+    b += [f'        if (__tid < {BK}) __ak[__buf][__tid] = {mc["parts"]["a"][1]};',
+          f'        else __bk[__buf][__tid - {BK}] = {mc["parts"]["b"][1]};',
           '      }',
           '    };',
           '    __ktab(0, 0);',
           '    if (__T > 1) __ktab(1, 1);',
           '    __syncthreads();',
           f'    const int __ml = __tid & {TS - 1}, __kh = (__tid / {TS}) * {PER};     // lanes along rows: {PER} k of one row (column) per thread',
-          f'    const int __kl = __tid & 15, __rw = __tid >> 4;             // lanes along k: one k of {PER} rows (columns) per thread',
+          f'    const int __kl = __tid & {BK - 1}, __rw = __tid / {BK};             // lanes along k: one k of {PER} rows (columns) per thread',
           '    (void)__ml; (void)__kh; (void)__kl; (void)__rw;']
     for x, ld, ct, tab, ktab_, lds, vals in (('a', la, ta, '__am', '__ak', '__As', val_a), ('b', lb, tb, '__bn', '__bk', '__Bs', val_b)):
         if mc['parts'][x][2]:
             b += [f'    const {ct}* __p{x}[{PER}];', '    #pragma unroll',
-                  f'    for (int __j = 0; __j < {PER}; ++__j) __p{x}[__j] = {ld.name} + {tab}[__rw + 16 * __j];']
+                  f'    for (int __j = 0; __j < {PER}; ++__j) __p{x}[__j] = {ld.name} + {tab}[__rw + {RS} * __j];']
         else:
             b.append(f'    const {ct}* __p{x} = {ld.name} + {tab}[__ml];')
         b.append(f'    {ct} __r{x}[{DEPTH}][{PER}];')
@@ -896,15 +898,15 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     b += ['    };', '    auto __stage = [&](auto __set, int __buf, int __kt) {', '      constexpr int __S = decltype(__set)::value; (void)__S;']
     for x, lds, vals in (('a', '__As', val_a), ('b', '__Bs', val_b)):
         if mc['parts'][x][2]:
-            b += [f'      {{ const bool __in = (long long)__kt * 16 + __kl < __K;']
-            b += [f'        {lds}[__buf][(__rw + {16 * j}) * 20 + __kl] = __in ? (float)({vals[j]}) : 0.f;' for j in range(PER)]
+            b += [f'      {{ const bool __in = (long long)__kt * {BK} + __kl < __K;']
+            b += [f'        {lds}[__buf][(__rw + {RS * j}) * {LD} + __kl] = __in ? (float)({vals[j]}) : 0.f;' for j in range(PER)]
             b += ['      }']
         else:
             def guarded(j):
                 return f'(__k0 + {j} < __K ? (float)({vals[j]}) : 0.f)'
-            b += ['      { const long long __k0 = (long long)__kt * 16 + __kh;']
+            b += [f'      {{ const long long __k0 = (long long)__kt * {BK} + __kh;']
             for q in range(PER // 4):
-                b += [f'        *(__f4*)&{lds}[__buf][__ml * 20 + __kh + {4 * q}] = __f4{{{guarded(4 * q)}, {guarded(4 * q + 1)}, {guarded(4 * q + 2)}, {guarded(4 * q + 3)}}};']
+                b += [f'        *(__f4*)&{lds}[__buf][__ml * {LD} + __kh + {4 * q}] = __f4{{{guarded(4 * q)}, {guarded(4 * q + 1)}, {guarded(4 * q + 2)}, {guarded(4 * q + 3)}}};']
             b += ['      }']
     b += ['    };',
           f'    __f16v __acc[{NT}][{NT}];',
@@ -917,12 +919,12 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           f'    const int __row0 = __wm * {HALF} + (__lane & 31), __col0 = __wn * {HALF} + (__lane & 31), __kq = (__lane >> 5) * 4;',
           '    auto __multiply = [&](int __buf) {',
           '      #pragma unroll',
-          '      for (int __g = 0; __g < 2; ++__g) {',
+          f'      for (int __g = 0; __g < {BK // 8}; ++__g) {{',
           f'        __f4 __a[{NT}], __b[{NT}];',
           '        #pragma unroll',
           f'        for (int __i = 0; __i < {NT}; ++__i) {{',
-          '          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * 20 + __g * 8 + __kq];',
-          '          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * 20 + __g * 8 + __kq];',
+          f'          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * {LD} + __g * 8 + __kq];',
+          f'          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * {LD} + __g * 8 + __kq];',
           '        }',
           '        #pragma unroll',
           '        for (int __m = 0; __m < 4; ++__m)',
