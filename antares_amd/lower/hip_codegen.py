@@ -816,8 +816,16 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     tensors).  TS = 64 gives blocks of 64 x 64 outputs (a wavefront then owns one 32 x 32 tile): four times the
     blocks for products too small to fill the chip with the big ones."""
     la, lb = mc['la'], mc['lb']
-    BK = 32 if TS == 64 else 16                       # k per tile: the small blocks take twice the k per barrier
-    LD, RS = BK + 4, BLOCK // BK                      # floats per row of a staged tile (16-byte aligned, rows on distinct banks); rows between a lane's elements when lanes walk k
+
+    def half_cast(f, ld):
+        return f.kind == 'cast' and f.dtype == 'float32' and f.args[0] is ld and tensors[ld.name].dtype == 'float16'
+    # fp16 operands that are only cast up: the tiles stay fp16 in LDS and go to v_mfma_f32_32x32x16_f16 - the
+    # products of two fp16 values are exact in float32 either way, and the matrix time is a sixteenth
+    HM = half_cast(mc['fa'], la) and half_cast(mc['fb'], lb)
+    BK = 32 if (TS == 64 or HM) else 16               # k per tile: the small blocks take twice the k per barrier
+    LD, RS = BK + (8 if HM else 4), BLOCK // BK       # elements per row of a staged tile (16-byte aligned, rows on distinct banks); rows between a lane's elements when lanes walk k
+    ET = 'half_t' if HM else 'float'                  # element type of the staged tiles
+    VW = 8 if HM else 4                               # elements per 16-byte vector of them
     NT, PER, HALF = TS // 64, TS * BK // BLOCK, TS // 2   # accumulator tiles per wavefront and direction, elements a thread stages per operand and tile, rows of a wavefront
     DEPTH = 2 if TS == 64 else 1                      # tiles on their way in registers: small blocks have nothing else to hide a load behind
     ta, tb, oct_ = HIP_TYPE[tensors[la.name].dtype], HIP_TYPE[tensors[lb.name].dtype], HIP_TYPE[st.out_dtype]
@@ -842,11 +850,13 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     cols_of_out = plain.offset(st.output, [a if a in mc['n'] else '0' for a in out_axes])
     val_a = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__ra[__S][{j}]').expr(mc['fa']) for j in range(PER)]
     val_b = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__rb[__S][{j}]').expr(mc['fb']) for j in range(PER)]
+    if HM:
+        val_a, val_b = [f'__ra[__S][{j}]' for j in range(PER)], [f'__rb[__S][{j}]' for j in range(PER)]
     b = [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st)
     b += ['  typedef float __f16v __attribute__((ext_vector_type(16)));',
-          '  typedef float __f4 __attribute__((ext_vector_type(4)));',
-          f'  __shared__ __attribute__((aligned(16))) float __As[2][{TS} * {LD}];     // [row][k], {BK} k and 4 floats of padding per row',
-          f'  __shared__ __attribute__((aligned(16))) float __Bs[2][{TS} * {LD}];     // [column][k]',
+          f'  typedef {ET} __f4 __attribute__((ext_vector_type({VW})));      // 16 bytes of a staged tile',
+          f'  __shared__ __attribute__((aligned(16))) {ET} __As[2][{TS} * {LD}];     // [row][k], {BK} k and 16 bytes of padding per row',
+          f'  __shared__ __attribute__((aligned(16))) {ET} __Bs[2][{TS} * {LD}];     // [column][k]',
           f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][{BK}], __bk[2][{BK}];',
           f'  const long long __M = {prod(mc["m"])}, __N = {prod(mc["n"])}, __B = {prod(mc["batch"])};',
           f'  const long long __K = {prod(mc["k"])};',
@@ -899,14 +909,14 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     for x, lds, vals in (('a', '__As', val_a), ('b', '__Bs', val_b)):
         if mc['parts'][x][2]:
             b += [f'      {{ const bool __in = (long long)__kt * {BK} + __kl < __K;']
-            b += [f'        {lds}[__buf][(__rw + {RS * j}) * {LD} + __kl] = __in ? (float)({vals[j]}) : 0.f;' for j in range(PER)]
+            b += [f'        {lds}[__buf][(__rw + {RS * j}) * {LD} + __kl] = __in ? ({ET})({vals[j]}) : ({ET})0.f;' for j in range(PER)]
             b += ['      }']
         else:
             def guarded(j):
-                return f'(__k0 + {j} < __K ? (float)({vals[j]}) : 0.f)'
+                return f'(__k0 + {j} < __K ? ({ET})({vals[j]}) : ({ET})0.f)'
             b += [f'      {{ const long long __k0 = (long long)__kt * {BK} + __kh;']
-            for q in range(PER // 4):
-                b += [f'        *(__f4*)&{lds}[__buf][__ml * {LD} + __kh + {4 * q}] = __f4{{{guarded(4 * q)}, {guarded(4 * q + 1)}, {guarded(4 * q + 2)}, {guarded(4 * q + 3)}}};']
+            for q in range(PER // VW):
+                b += [f'        *(__f4*)&{lds}[__buf][__ml * {LD} + __kh + {VW * q}] = __f4{{' + ', '.join(guarded(VW * q + e) for e in range(VW)) + '};']
             b += ['      }']
     b += ['    };',
           f'    __f16v __acc[{NT}][{NT}];',
@@ -916,24 +926,31 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           f'      for (int __j = 0; __j < {NT}; ++__j)',
           '        #pragma unroll',
           '        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = 0.f;',
-          f'    const int __row0 = __wm * {HALF} + (__lane & 31), __col0 = __wn * {HALF} + (__lane & 31), __kq = (__lane >> 5) * 4;',
+          f'    const int __row0 = __wm * {HALF} + (__lane & 31), __col0 = __wn * {HALF} + (__lane & 31), __kq = (__lane >> 5) * {VW};',
           '    auto __multiply = [&](int __buf) {',
           '      #pragma unroll',
-          f'      for (int __g = 0; __g < {BK // 8}; ++__g) {{',
+          f'      for (int __g = 0; __g < {BK // (16 if HM else 8)}; ++__g) {{',
           f'        __f4 __a[{NT}], __b[{NT}];',
           '        #pragma unroll',
           f'        for (int __i = 0; __i < {NT}; ++__i) {{',
-          f'          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * {LD} + __g * 8 + __kq];',
-          f'          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * {LD} + __g * 8 + __kq];',
-          '        }',
-          '        #pragma unroll',
-          '        for (int __m = 0; __m < 4; ++__m)',
-          '          #pragma unroll',
-          f'          for (int __i = 0; __i < {NT}; ++__i)',
-          '            #pragma unroll',
-          f'            for (int __j = 0; __j < {NT}; ++__j)',
-          '              __acc[__i][__j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__a[__i][__m], __b[__j][__m], __acc[__i][__j], 0, 0, 0);',
-          '      }',
+          f'          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * {LD} + __g * {16 if HM else 8} + __kq];',
+          f'          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * {LD} + __g * {16 if HM else 8} + __kq];',
+          '        }']
+    if HM:      # a lane supplies 8 consecutive k of its row (column): k = (lane / 32) * 8 .. + 7 of the 16
+        b += ['        #pragma unroll',
+              f'        for (int __i = 0; __i < {NT}; ++__i)',
+              '          #pragma unroll',
+              f'          for (int __j = 0; __j < {NT}; ++__j)',
+              '            __acc[__i][__j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__a[__i], __b[__j], __acc[__i][__j], 0, 0, 0);']
+    else:       # instruction m multiplies k = m (lanes 0-31) and k = 4 + m (lanes 32-63) of the 8
+        b += ['        #pragma unroll',
+              '        for (int __m = 0; __m < 4; ++__m)',
+              '          #pragma unroll',
+              f'          for (int __i = 0; __i < {NT}; ++__i)',
+              '            #pragma unroll',
+              f'            for (int __j = 0; __j < {NT}; ++__j)',
+              '              __acc[__i][__j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__a[__i][__m], __b[__j][__m], __acc[__i][__j], 0, 0, 0);']
+    b += ['      }',
           '    };']
     if DEPTH == 1:
         b += ['    __load(art_ic<0>{}, 0);',

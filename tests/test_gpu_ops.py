@@ -668,6 +668,12 @@ MATRIX_CASES = [
     ('output0[N, F, HO, WO] +=! input0[N, C, HO * 2 + KH, WO * 2 + KW] * input1[F, C, KH, KW] where HO in 29, WO in 29',
      ['input0=float32[N:10, C:3, H:64, W:64]', 'input1=float32[F:64, C:3, KH:7, KW:7]'], [(10, 3, 64, 64), (64, 3, 7, 7)]),
     ('output0[N, M] +=! input0[N, K] * input1[M, K]', ['input0=float32[N:1024, K:250]', 'input1=float32[M:1024, K:250]'], [(1024, 250), (1024, 250)]),
+    # fp16 operands that are only cast up stay fp16 in the tiles (v_mfma_f32_32x32x16_f16): B stored [K, M], k = 2.5 tiles;
+    # a batched product of fp16 operands
+    ('output0[N, M] +=! input0[N, K].to(`float32`) * input1[K, M].to(`float32`)', ['input0=float16[N:1100, K:80]', 'input1=float16[K:80, M:1024]'],
+     [(1100, 80), (80, 1024)]),
+    ('output0[B, N, M] +=! input0[B, N, K].to(`float32`) * input1[B, M, K].to(`float32`)',
+     ['input0=float16[B:4, N:520, K:96]', 'input1=float16[B:4, M:500, K:96]'], [(4, 520, 96), (4, 500, 96)]),
 ]
 
 
