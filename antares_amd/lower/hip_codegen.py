@@ -206,7 +206,7 @@ class KernelPlan:
     tile_axes: Optional[Tuple[str, str]] = None   # permutation copies: last axis of the load, last axis of the store
     tile_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for the vector form of it
     row_group: Optional[RowGroup] = None          # set on the first statement of a run that one row kernel can compute
-    matrix: Optional[Dict[str, List[object]]] = None   # matrix-instruction variant: extents of its row, column, batch and k axes
+    matrix: Optional[Dict[str, List[object]]] = None   # matrix-instruction variant: extents of its row, column, batch and k axes (and what its vector form needs)
 
     def _tiles(self, env: Dict[str, int]) -> int:
         """64 x 64 tiles of the transposing variant, 0 when it does not apply or an axis is too short to pay."""
@@ -248,7 +248,7 @@ class KernelPlan:
             return 0
         return total // self.row_vec
 
-    def _matrix_choice(self, env: Dict[str, int]) -> Tuple[Optional[str], int]:
+    def _matrix_choice(self, env: Dict[str, int], pointers: Optional[Dict[str, int]] = None) -> Tuple[Optional[str], int]:
         """(variant tag, blocks) of the matrix-instruction variants, (None, 0) when they do not apply: there must be
         enough k to pay for staging it, and enough tiles - of 128 x 128 outputs when those fill the chip, else of
         64 x 64 (a block multiplies a quarter as much per k, so small products spread over four times the compute
@@ -265,10 +265,15 @@ class KernelPlan:
             return None, 0
         big = ((M + 127) // 128) * ((N + 127) // 128) * B
         small = ((M + 63) // 64) * ((N + 63) // 64) * B
+        # the kernels that fetch k-contiguous operands in 16-byte vectors need whole vectors and aligned tensors
+        v = ''
+        if 'matrixv' in self.variants and pointers is not None and K % self.matrix['vec_width'][0] == 0 and \
+                all(pointers[t] % 16 == 0 for t in self.matrix['vec_tensors']):
+            v = 'v'
         if big >= 192 and big <= MAX_GRID * 64:
-            return 'matrix', big
+            return 'matrix' + v, big
         if 'matrix64' in self.variants and small >= 16 and small <= MAX_GRID * 64:
-            return 'matrix64', small
+            return 'matrix64' + v, small
         return None, 0
 
     def _matrix_blocks(self, env: Dict[str, int]) -> int:
@@ -310,7 +315,7 @@ class KernelPlan:
         if self.kind == 'scatter':
             return self.variants['scalar'], min((total + BLOCK - 1) // BLOCK, MAX_GRID), BLOCK
         # reduce
-        tag, blocks = self._matrix_choice(env)
+        tag, blocks = self._matrix_choice(env, pointers)
         if tag:
             return self.variants[tag], blocks, BLOCK
         patches = self._patches(env, total)
@@ -352,8 +357,8 @@ class KernelPlan:
             tags += [('thread', total), ('wave', (total + waves_per_block - 1) // waves_per_block * BLOCK), ('block', total * BLOCK)]
             if self._patches(env, total):
                 tags.append(('patch', self._patches(env, total)))
-            if self._matrix_choice(env)[0]:
-                tags.append((self._matrix_choice(env)[0], self._matrix_blocks(env) * BLOCK))
+            if self._matrix_choice(env, pointers)[0]:
+                tags.append((self._matrix_choice(env, pointers)[0], self._matrix_blocks(env) * BLOCK))
         out = []
         for tag, work in tags:
             if tag not in self.variants:
@@ -798,11 +803,18 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
             variants['matrix'], variants['matrix64'] = name + '_m', name + '_m64'
             ext = dict(st.data_axes + st.reduce_axes)
             plan.matrix = {key: [ext[a] for a in mc[key]] for key in ('m', 'n', 'batch', 'k')}
+            if mc['vec']['a'] or mc['vec']['b']:
+                src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_mv', mc, vectors=True))
+                src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_m64v', mc, TS=64, vectors=True))
+                variants['matrixv'], variants['matrix64v'] = name + '_mv', name + '_m64v'
+                wide = [ITEMSIZE[tensors[mc['l' + t].name].dtype] for t in ('a', 'b') if mc['vec'][t]]
+                plan.matrix['vec_tensors'] = [mc['l' + t].name for t in ('a', 'b') if mc['vec'][t]]
+                plan.matrix['vec_width'] = [16 // min(wide)]
 
     return '\n\n'.join(src), plan
 
 
-def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128) -> str:
+def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128, vectors: bool = False) -> str:
     """A sum of products of two loads on v_mfma_f32_32x32x2_f32 (the reference's counterpart: its tiled schedule for
     contractions, backends/c-rocm/schedule/standard/algo_tiling.py:35-98, on the vector units).  A block of 256
     threads = 2 x 2 wavefronts owns 128 rows x 128 columns of one batch, where a row is a point of the axes only
@@ -826,6 +838,14 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     LD, RS = BK + (8 if HM else 4), BLOCK // BK       # elements per row of a staged tile (16-byte aligned, rows on distinct banks); rows between a lane's elements when lanes walk k
     ET = 'half_t' if HM else 'float'                  # element type of the staged tiles
     VW = 8 if HM else 4                               # elements per 16-byte vector of them
+    # how an operand travels: 'rows' (lanes along rows, PER k each), 'k' (lanes along k, PER rows each), or 'kvec' (a
+    # lane fetches 16 bytes of k of PER / VL rows: rows of k in memory, whole vectors, aligned - the launcher checks)
+    def vector_ok(x, ld):       # the staged value must be the loaded one, in the tile's element type
+        return vectors and mc['vec'][x] and (HM or (tensors[ld.name].dtype == 'float32' and mc['f' + x] is ld))
+    mode = {x: ('kvec' if vector_ok(x, ld) else ('k' if mc['parts'][x][2] else 'rows')) for x, ld in (('a', la), ('b', lb))}
+    VL = 16 // ITEMSIZE[tensors[la.name].dtype] if mode['a'] == 'kvec' else (16 // ITEMSIZE[tensors[lb.name].dtype] if mode['b'] == 'kvec' else VW)
+    VPR = BK // VL                                    # vectors per row of a tile
+    RV = BLOCK // VPR                                 # rows a pass of the 256 threads covers
     NT, PER, HALF = TS // 64, TS * BK // BLOCK, TS // 2   # accumulator tiles per wavefront and direction, elements a thread stages per operand and tile, rows of a wavefront
     DEPTH = 2 if TS == 64 else 1                      # tiles on their way in registers: small blocks have nothing else to hide a load behind
     ta, tb, oct_ = HIP_TYPE[tensors[la.name].dtype], HIP_TYPE[tensors[lb.name].dtype], HIP_TYPE[st.out_dtype]
@@ -892,22 +912,40 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           f'    const int __kl = __tid & {BK - 1}, __rw = __tid / {BK};             // lanes along k: one k of {PER} rows (columns) per thread',
           '    (void)__ml; (void)__kh; (void)__kl; (void)__rw;']
     for x, ld, ct, tab, ktab_, lds, vals in (('a', la, ta, '__am', '__ak', '__As', val_a), ('b', lb, tb, '__bn', '__bk', '__Bs', val_b)):
-        if mc['parts'][x][2]:
+        if mode[x] == 'kvec':
+            b += [f'    typedef {ct} __v{x} __attribute__((ext_vector_type({VL})));',
+                  f'    const {ct}* __p{x}[{TS // RV}];', '    #pragma unroll',
+                  f'    for (int __j = 0; __j < {TS // RV}; ++__j) __p{x}[__j] = {ld.name} + {tab}[__tid / {VPR} + {RV} * __j];',
+                  f'    __v{x} __r{x}[{DEPTH}][{TS // RV}];']
+            continue
+        if mode[x] == 'k':
             b += [f'    const {ct}* __p{x}[{PER}];', '    #pragma unroll',
                   f'    for (int __j = 0; __j < {PER}; ++__j) __p{x}[__j] = {ld.name} + {tab}[__rw + {RS} * __j];']
         else:
             b.append(f'    const {ct}* __p{x} = {ld.name} + {tab}[__ml];')
         b.append(f'    {ct} __r{x}[{DEPTH}][{PER}];')
-    b += ['    auto __load = [&](auto __set, int __buf) {', '      constexpr int __S = decltype(__set)::value;']
+    b += ['    auto __load = [&](auto __set, int __buf, int __ktile) {', '      constexpr int __S = decltype(__set)::value; (void)__ktile;']
     for x, ktab_ in (('a', '__ak'), ('b', '__bk')):
-        if mc['parts'][x][2]:
+        if mode[x] == 'kvec':       # the k offset of a row of k is k itself; a vector past the end re-reads the row's first
+            b += [f'      {{ const long long __k0 = (long long)__ktile * {BK} + (__tid % {VPR}) * {VL};',
+                  f'        const long long __ko = __k0 + {VL} <= __K ? __k0 : 0;', '        #pragma unroll',
+                  f'        for (int __j = 0; __j < {TS // RV}; ++__j) __r{x}[__S][__j] = *(const __v{x}*)(__p{x}[__j] + __ko); }}']
+            continue
+        if mode[x] == 'k':
             b += [f'      {{ const long long __ko = {ktab_}[__buf][__kl];', '        #pragma unroll',
                   f'        for (int __j = 0; __j < {PER}; ++__j) __r{x}[__S][__j] = __p{x}[__j][__ko]; }}']
         else:
             b += ['      #pragma unroll', f'      for (int __j = 0; __j < {PER}; ++__j) __r{x}[__S][__j] = __p{x}[{ktab_}[__buf][__kh + __j]];']
     b += ['    };', '    auto __stage = [&](auto __set, int __buf, int __kt) {', '      constexpr int __S = decltype(__set)::value; (void)__S;']
     for x, lds, vals in (('a', '__As', val_a), ('b', '__Bs', val_b)):
-        if mc['parts'][x][2]:
+        if mode[x] == 'kvec':
+            b += [f'      {{ const bool __in = (long long)__kt * {BK} + (__tid % {VPR}) * {VL} + {VL} <= __K;']
+            for j in range(TS // RV):
+                dst = f'&{lds}[__buf][(__tid / {VPR} + {RV * j}) * {LD} + (__tid % {VPR}) * {VL}]'
+                b += [f'        *(__v{x}*){dst} = __in ? __r{x}[__S][{j}] : (__v{x})(0);']
+            b += ['      }']
+            continue
+        if mode[x] == 'k':
             b += [f'      {{ const bool __in = (long long)__kt * {BK} + __kl < __K;']
             b += [f'        {lds}[__buf][(__rw + {RS * j}) * {LD} + __kl] = __in ? ({ET})({vals[j]}) : ({ET})0.f;' for j in range(PER)]
             b += ['      }']
@@ -953,12 +991,12 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     b += ['      }',
           '    };']
     if DEPTH == 1:
-        b += ['    __load(art_ic<0>{}, 0);',
+        b += ['    __load(art_ic<0>{}, 0, 0);',
               '    __stage(art_ic<0>{}, 0, 0);',
               '    __syncthreads();',
               '    for (int __t = 0; __t < __T; ++__t) {',
               '      const int __buf = __t & 1;',
-              '      if (__t + 1 < __T) __load(art_ic<0>{}, __buf ^ 1);    // tile t + 1 travels while tile t is multiplied',
+              '      if (__t + 1 < __T) __load(art_ic<0>{}, __buf ^ 1, __t + 1);    // tile t + 1 travels while tile t is multiplied',
               '      if (__t + 2 < __T) __ktab(__t + 2, __buf);            // its k offsets were read a tile ago',
               '      __multiply(__buf);',
               '      if (__t + 1 < __T) __stage(art_ic<0>{}, __buf ^ 1, __t + 1);   // the other buffer: everybody left it at the last barrier',
@@ -968,20 +1006,20 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         b += ['    // Tile t is multiplied out of LDS buffer t % 2 and came through register set t % 2.  While it is multiplied,',
               '    // tile t + 1 waits in the other register set and tile t + 2 is asked for into the set tile t has left; the k',
               '    // offsets of tile t + 3 go into the table that the loads of tile t + 1 read one barrier ago.',
-              '    __load(art_ic<0>{}, 0);',
-              '    if (__T > 1) __load(art_ic<1>{}, 1);',
+              '    __load(art_ic<0>{}, 0, 0);',
+              '    if (__T > 1) __load(art_ic<1>{}, 1, 1);',
               '    __syncthreads();                               // everybody has read the k offsets of tile 0',
               '    if (__T > 2) __ktab(2, 0);',
               '    __stage(art_ic<0>{}, 0, 0);',
               '    __syncthreads();',
               '    for (int __t = 0; __t < __T; __t += 2) {',
-              '      if (__t + 2 < __T) __load(art_ic<0>{}, 0);',
+              '      if (__t + 2 < __T) __load(art_ic<0>{}, 0, __t + 2);',
               '      if (__t + 3 < __T) __ktab(__t + 3, 1);',
               '      __multiply(0);',
               '      if (__t + 1 < __T) __stage(art_ic<1>{}, 1, __t + 1);    // the other buffer: everybody left it at the last barrier',
               '      __syncthreads();',
               '      if (__t + 1 < __T) {',
-              '        if (__t + 3 < __T) __load(art_ic<1>{}, 1);',
+              '        if (__t + 3 < __T) __load(art_ic<1>{}, 1, __t + 3);',
               '        if (__t + 4 < __T) __ktab(__t + 4, 0);',
               '        __multiply(1);',
               '        if (__t + 2 < __T) __stage(art_ic<0>{}, 0, __t + 2);',
@@ -1120,7 +1158,15 @@ def _matrix_contraction(st, tensors):
         # lanes walk k when the operand's last index is made of k axes alone (k is then the contiguous axis), else rows
         parts[tag] = (plain.offset(ld.name, [x[0] or '0' for x in sp]), plain.offset(ld.name, [x[1] or '0' for x in sp]),
                       sp[-1][0] is None)
-    return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts}
+    # an operand whose last index is THE reduce axis, bare, and whose last extent is that axis' extent, lies in memory
+    # as rows of k: 16-byte vectors of k can be fetched when k is a multiple of the vector and the tensor is aligned
+    vec = {}
+    for tag, ld in (('a', la), ('b', lb)):
+        last = ld.args[-1]
+        vec[tag] = (len(k_axes) == 1 and last.kind == 'axis' and last.name == k_axes[0] and
+                    not any(k_axes[0] in _axes_of(a) for a in ld.args[:-1]) and
+                    tensors[ld.name].shape[-1] == dict(st.reduce_axes)[k_axes[0]])
+    return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts, 'vec': vec}
 
 
 def _row_group_at(graph, i: int) -> int:

@@ -637,8 +637,9 @@ def test_large_contractions_take_the_register_tiled_variant(autort):
     op.fast_path = None               # the generic lowering is what is tested here
     plan = op.plans[0]
     zero = {n: 0 for n in plan.args}
-    assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['matrix']
-    del plan.variants['matrix'], plan.variants['matrix64']
+    assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['matrixv']
+    for tag in [t for t in plan.variants if t.startswith('matrix')]:
+        del plan.variants[tag]
     assert plan.choose({'N': 2048, 'K': 256, 'M': 2048}, zero)[0] == plan.variants['patch']
     assert plan.choose({'N': 2046, 'K': 256, 'M': 2048}, zero)[0] != plan.variants['patch']
     assert plan.choose({'N': 1024, 'K': 256, 'M': 1024}, zero)[0] != plan.variants['patch']
@@ -693,7 +694,7 @@ def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, ir, in
     for spec, shape in zip(inputs, shapes):
         for d, v in zip(spec.split('[', 1)[1].rstrip(']').split(','), shape):
             env[d.split(':')[0].strip()] = v
-    assert plan.choose(env, {n: 0 for n in plan.args})[0] in (plan.variants['matrix'], plan.variants['matrix64'])
+    assert plan.choose(env, {n: 0 for n in plan.args})[0] in [v for t, v in plan.variants.items() if t.startswith('matrix')]
     assert plan.row_group is None                 # nothing else takes the statement
     g = torch.Generator().manual_seed(len(ir))
     tensors = [torch.randn(shape, generator=g).to(torch.float16 if 'float16' in spec else torch.float32) for spec, shape in zip(inputs, shapes)]
@@ -706,7 +707,14 @@ def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, ir, in
     tol = 2e-5 * scale * K ** 0.5 * 4
     M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
     rule = plan.choose
-    for tag, side in (('matrix', 128), ('matrix64', 64)):       # blocks of 128 x 128 and of 64 x 64 outputs
+    sizes = [('matrix', 128), ('matrix64', 64)]                # blocks of 128 x 128 and of 64 x 64 outputs
+    if 'matrixv' in plan.variants and K % plan.matrix['vec_width'][0] == 0:
+        sizes += [('matrixv', 128), ('matrix64v', 64)]          # ... and their forms that fetch rows of k in 16-byte vectors
+        ptrs = {n: 0 for n in plan.args}
+        assert plan.choose(env, ptrs)[0] in (plan.variants['matrixv'], plan.variants['matrix64v'])
+        ptrs[plan.matrix['vec_tensors'][0]] = 8                 # a tensor that is not 16-byte aligned: scalar fetches
+        assert plan.choose(env, ptrs)[0] in (plan.variants['matrix'], plan.variants['matrix64'])
+    for tag, side in sizes:
         blocks = ((M + side - 1) // side) * ((N + side - 1) // side) * B
         plan.choose = lambda env_, ptrs, tag=tag, blocks=blocks: (plan.variants[tag], blocks, 256)
         got = op(*[t.to(dev) for t in tensors]).cpu().numpy()
@@ -714,7 +722,8 @@ def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, ir, in
         assert np.allclose(got, want, rtol=1e-4, atol=tol), (tag, np.abs(got - want).max())
     # the same statement through the register-tiled variant
     plan.choose = rule
-    del plan.variants['matrix'], plan.variants['matrix64']
+    for tag in [t for t in plan.variants if t.startswith('matrix')]:
+        del plan.variants[tag]
     apart = op(*[t.to(dev) for t in tensors]).cpu().numpy()
     assert np.allclose(got, apart, rtol=1e-4, atol=tol)
 
