@@ -270,7 +270,9 @@ class KernelPlan:
         if 'matrixv' in self.variants and pointers is not None and K % self.matrix['vec_width'][0] == 0 and \
                 all(pointers[t] % 16 == 0 for t in self.matrix['vec_tensors']):
             v = 'v'
-        if big >= 192 and big <= MAX_GRID * 64:
+        # ... and when the big tiles are not mostly padding: 64 columns in tiles of 128 multiply twice what they need,
+        # which costs more than the small tiles' lower rate (about three quarters of the big ones')
+        if big >= 192 and big <= MAX_GRID * 64 and ('matrix64' not in self.variants or small >= 3 * big):
             return 'matrix' + v, big
         if 'matrix64' in self.variants and small >= 16 and small <= MAX_GRID * 64:
             return 'matrix64' + v, small
@@ -826,7 +828,9 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     GEMM kernel of the library feeds it; rows, columns and batches past the extents are clamped on the way in and
     cut on the way out; the k a last partial tile lacks are staged as zeros (their addresses wrap into the
     tensors).  TS = 64 gives blocks of 64 x 64 outputs (a wavefront then owns one 32 x 32 tile): four times the
-    blocks for products too small to fill the chip with the big ones."""
+    blocks for products too small to fill the chip with the big ones.  A guarded operand (AntaresIR.md:166, a padded
+    convolution) has the row part and the k part of every compared value tabled the same way and is fetched from
+    its own address only where its conditions hold."""
     la, lb = mc['la'], mc['lb']
 
     def half_cast(f, ld):
@@ -851,6 +855,21 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     ta, tb, oct_ = HIP_TYPE[tensors[la.name].dtype], HIP_TYPE[tensors[lb.name].dtype], HIP_TYPE[st.out_dtype]
     plain = ExprEmitter(tensors)
     ext = dict(st.data_axes + st.reduce_axes)
+    # A guarded operand (`x[...].when([conditions], 0)`, the padding of a convolution): every compared value is (row
+    # part) + (k part) like an address, both parts are tabled beside the offsets, an element is fetched only where all
+    # its conditions hold - rows and k are points of the statement's own axes, clamped or wrapped, so a fetch that
+    # happens is one the statement makes - and staged as zero where they do not.
+    G = mc.get('guards') or {'a': [], 'b': []}
+    # the two bounds of a padded index compare the same value: one pair of tables per distinct value
+    GV = {x: list(dict.fromkeys((g[0], g[1]) for g in G[x])) for x in 'ab'}
+
+    def holds(x, row, k):       # C text: the compared values of (row slot, k slot), then the conjunction over them
+        vals = [f'const int __v{c} = __gm{x}[{c}][{row}] + __gk{x}[__buf][{k}][{c}];' for c in range(len(GV[x]))]
+        terms = []
+        for qm, qk, op, other, left in G[x]:
+            v = f'__v{GV[x].index((qm, qk))}'
+            terms.append(f'({v} {op} {other})' if left else f'({other} {op} {v})')
+        return ' '.join(vals), ' && '.join(terms)
 
     def prod(names):
         return ' * '.join(f'(long long)__ext_{a}' for a in names) or '1LL'
@@ -877,7 +896,9 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           f'  typedef {ET} __f4 __attribute__((ext_vector_type({VW})));      // 16 bytes of a staged tile',
           f'  __shared__ __attribute__((aligned(16))) {ET} __As[2][{TS} * {LD}];     // [row][k], {BK} k and 16 bytes of padding per row',
           f'  __shared__ __attribute__((aligned(16))) {ET} __Bs[2][{TS} * {LD}];     // [column][k]',
-          f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][{BK}], __bk[2][{BK}];',
+          f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][{BK}], __bk[2][{BK}];'] + \
+         [f'  __shared__ int __gm{x}[{len(GV[x])}][{TS}], __gk{x}[2][{BK}][{len(GV[x])}];      // the guards of operand {x}: row part and k part of each compared value'
+          for x in 'ab' if G[x]] + [
           f'  const long long __M = {prod(mc["m"])}, __N = {prod(mc["n"])}, __B = {prod(mc["batch"])};',
           f'  const long long __K = {prod(mc["k"])};',
           f'  const int __T = (int)((__K + {BK - 1}) / {BK});      // the last tile may be partial: its missing k are staged as zeros',
@@ -890,19 +911,23 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           f'      long long __row = __tm * {TS} + __tid;',
           '      if (__row >= __M) __row = __M - 1;']
     b += decompose('__row', mc['m'], '      ')
+    b += [f'      __gma[{c}][__tid] = {g[0]};' for c, g in enumerate(GV['a'])]
     b += [f'      __am[__tid] = {mc["parts"]["a"][0]};', f'      __cm[__tid] = {rows_of_out};',
           f'    }} else if (__tid < {2 * TS}) {{                  // column offsets of the second operand and of the output',
           f'      long long __colq = __tn * {TS} + (__tid - {TS});',
           '      if (__colq >= __N) __colq = __N - 1;']
     b += decompose('__colq', mc['n'], '      ')
+    b += [f'      __gmb[{c}][__tid - {TS}] = {g[0]};' for c, g in enumerate(GV['b'])]
     b += [f'      __bn[__tid - {TS}] = {mc["parts"]["b"][0]};', f'      __cn[__tid - {TS}] = {cols_of_out};',
           '    }',
           f'    auto __ktab = [&](int __kt, int __buf) {{       // k offsets of tile __kt: {BK} for each operand',
           f'      if (__tid < {2 * BK}) {{',
           f'        const long long __kk = (long long)__kt * {BK} + (__tid & {BK - 1});']
     b += decompose('__kk', mc['k'], '        ', wide=False)
-    b += [f'        if (__tid < {BK}) __ak[__buf][__tid] = {mc["parts"]["a"][1]};',
-          f'        else __bk[__buf][__tid - {BK}] = {mc["parts"]["b"][1]};',
+    b += [f'        if (__tid < {BK}) {{ __ak[__buf][__tid] = {mc["parts"]["a"][1]}; ' +
+          ' '.join(f'__gka[__buf][__tid][{c}] = {g[1]};' for c, g in enumerate(GV['a'])) + ' }',
+          f'        else {{ __bk[__buf][__tid - {BK}] = {mc["parts"]["b"][1]}; ' +
+          ' '.join(f'__gkb[__buf][__tid - {BK}][{c}] = {g[1]};' for c, g in enumerate(GV['b'])) + ' }',
           '      }',
           '    };',
           '    __ktab(0, 0);',
@@ -924,6 +949,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         else:
             b.append(f'    const {ct}* __p{x} = {ld.name} + {tab}[__ml];')
         b.append(f'    {ct} __r{x}[{DEPTH}][{PER}];')
+        if G[x]:
+            b.append(f'    unsigned int __g{x}[{DEPTH}];              // bit j: element j of the set is inside its guards')
     b += ['    auto __load = [&](auto __set, int __buf, int __ktile) {', '      constexpr int __S = decltype(__set)::value; (void)__ktile;']
     for x, ktab_ in (('a', '__ak'), ('b', '__bk')):
         if mode[x] == 'kvec':       # the k offset of a row of k is k itself; a vector past the end re-reads the row's first
@@ -931,7 +958,16 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
                   f'        const long long __ko = __k0 + {VL} <= __K ? __k0 : 0;', '        #pragma unroll',
                   f'        for (int __j = 0; __j < {TS // RV}; ++__j) __r{x}[__S][__j] = *(const __v{x}*)(__p{x}[__j] + __ko); }}']
             continue
-        if mode[x] == 'k':
+        if G[x]:
+            row, k = (f'__rw + {RS} * __j', '__kl') if mode[x] == 'k' else ('__ml', '__kh + __j')
+            at = f'__p{x}[__j] + {ktab_}[__buf][__kl]' if mode[x] == 'k' else f'__p{x} + {ktab_}[__buf][__kh + __j]'
+            b += [f'      {{ unsigned int __in = 0u;', '        #pragma unroll',
+                  f'        for (int __j = 0; __j < {PER}; ++__j) {{',
+                  f'          {holds(x, row, k)[0]}',
+                  f'          const bool __h = {holds(x, row, k)[1]};',
+                  f'          __r{x}[__S][__j] = *(__h ? {at} : {(la if x == "a" else lb).name});       // outside: the tensor\'s first element, not used',
+                  '          __in |= (unsigned int)__h << __j;', '        }', f'        __g{x}[__S] = __in; }}']
+        elif mode[x] == 'k':
             b += [f'      {{ const long long __ko = {ktab_}[__buf][__kl];', '        #pragma unroll',
                   f'        for (int __j = 0; __j < {PER}; ++__j) __r{x}[__S][__j] = __p{x}[__j][__ko]; }}']
         else:
@@ -945,13 +981,15 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
                 b += [f'        *(__v{x}*){dst} = __in ? __r{x}[__S][{j}] : (__v{x})(0);']
             b += ['      }']
             continue
+        def inside(j, x=x):
+            return f' && ((__g{x}[__S] >> {j}) & 1u)' if G[x] else ''
         if mode[x] == 'k':
             b += [f'      {{ const bool __in = (long long)__kt * {BK} + __kl < __K;']
-            b += [f'        {lds}[__buf][(__rw + {RS * j}) * {LD} + __kl] = __in ? ({ET})({vals[j]}) : ({ET})0.f;' for j in range(PER)]
+            b += [f'        {lds}[__buf][(__rw + {RS * j}) * {LD} + __kl] = __in{inside(j)} ? ({ET})({vals[j]}) : ({ET})0.f;' for j in range(PER)]
             b += ['      }']
         else:
             def guarded(j):
-                return f'(__k0 + {j} < __K ? ({ET})({vals[j]}) : ({ET})0.f)'
+                return f'(__k0 + {j} < __K{inside(j)} ? ({ET})({vals[j]}) : ({ET})0.f)'
             b += [f'      {{ const long long __k0 = (long long)__kt * {BK} + __kh;']
             for q in range(PER // VW):
                 b += [f'        *(__f4*)&{lds}[__buf][__ml * {LD} + __kh + {VW * q}] = __f4{{' + ', '.join(guarded(VW * q + e) for e in range(VW)) + '};']
@@ -1112,6 +1150,14 @@ def _split_index(e: Expr, em: ExprEmitter, outer: set, inner: set):
         def add(x, y):
             return y if x is None else (x if y is None else f'({x}) + ({y})')
         return add(l[0], r[0]), add(l[1], r[1])
+    if e.kind == 'op' and e.name == '-' and len(e.args) == 2:
+        l, r = _split_index(e.args[0], em, outer, inner), _split_index(e.args[1], em, outer, inner)
+        if l is None or r is None:
+            return None
+
+        def sub(x, y):
+            return x if y is None else (f'-({y})' if x is None else f'({x}) - ({y})')
+        return sub(l[0], r[0]), sub(l[1], r[1])
     return None
 
 
@@ -1129,12 +1175,28 @@ def _matrix_contraction(st, tensors):
     if [i.name if i.kind == 'axis' else None for i in st.out_index] != axes:
         return None
     fa, fb = root.args
+    # a factor may be guarded: `x[...].when([conditions], 0)` - the padding of a convolution
+    guards = {'a': [], 'b': []}
+    for tag in ('a', 'b'):
+        f = fa if tag == 'a' else fb
+        if f.kind == 'when':
+            zero = len(f.args) == 2 and f.args[1].kind == 'const' and f.args[1].value == 0
+            if not zero or f.merge != 'all':
+                return None
+            guards[tag] = list(f.conds)
+            if tag == 'a':
+                fa = f.args[0]
+            else:
+                fb = f.args[0]
     la, lb = [n for n in walk(fa) if n.kind == 'load'], [n for n in walk(fb) if n.kind == 'load']
     if len(la) != 1 or len(lb) != 1 or st.output in (la[0].name, lb[0].name):
         return None
     la, lb = la[0], lb[0]
-    # axes may be used inside the indices of the two loads only
-    inside = sum(1 for n in (la, lb) for a in n.args for m in walk(a) if m.kind == 'axis')
+    if any(n.kind in ('load', 'when') for tag in guards for c in guards[tag] for n in walk(c)):
+        return None
+    # axes may be used inside the indices of the two loads and inside the guards only
+    inside = sum(1 for n in (la, lb) for a in n.args for m in walk(a) if m.kind == 'axis') + \
+        sum(1 for tag in guards for c in guards[tag] for m in walk(c) if m.kind == 'axis')
     if sum(1 for m in walk(root) if m.kind == 'axis') != inside:
         return None
     ua, ub = set().union(*[_axes_of(a) for a in la.args]), set().union(*[_axes_of(a) for a in lb.args])
@@ -1158,6 +1220,19 @@ def _matrix_contraction(st, tensors):
         # lanes walk k when the operand's last index is made of k axes alone (k is then the contiguous axis), else rows
         parts[tag] = (plain.offset(ld.name, [x[0] or '0' for x in sp]), plain.offset(ld.name, [x[1] or '0' for x in sp]),
                       sp[-1][0] is None)
+        # a guard compares an expression that splits the same way with something free of axes
+        conds = []
+        for c in guards[tag]:
+            if c.kind != 'op' or c.name not in ('<', '<=', '>', '>=', '==', '!=') or len(c.args) != 2:
+                return None
+            left = bool(_axes_of(c.args[0]))
+            if left == bool(_axes_of(c.args[1])):
+                return None
+            sp_c = _split_index(c.args[0 if left else 1], plain, outer, inner)
+            if sp_c is None:
+                return None
+            conds.append((sp_c[0] or '0', sp_c[1] or '0', c.name, plain.expr(c.args[1 if left else 0]), left))
+        guards[tag] = conds
     # an operand whose last index is THE reduce axis, bare, and whose last extent is that axis' extent, lies in memory
     # as rows of k: 16-byte vectors of k can be fetched when k is a multiple of the vector and the tensor is aligned
     vec = {}
@@ -1165,8 +1240,9 @@ def _matrix_contraction(st, tensors):
         last = ld.args[-1]
         vec[tag] = (len(k_axes) == 1 and last.kind == 'axis' and last.name == k_axes[0] and
                     not any(k_axes[0] in _axes_of(a) for a in ld.args[:-1]) and
-                    tensors[ld.name].shape[-1] == dict(st.reduce_axes)[k_axes[0]])
-    return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts, 'vec': vec}
+                    tensors[ld.name].shape[-1] == dict(st.reduce_axes)[k_axes[0]] and not guards[tag])
+    return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts, 'vec': vec,
+            'guards': guards}
 
 
 def _row_group_at(graph, i: int) -> int:

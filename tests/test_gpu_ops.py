@@ -675,6 +675,16 @@ MATRIX_CASES = [
      [(1100, 80), (80, 1024)]),
     ('output0[B, N, M] +=! input0[B, N, K].to(`float32`) * input1[B, M, K].to(`float32`)',
      ['input0=float16[B:4, N:520, K:96]', 'input1=float16[B:4, M:500, K:96]'], [(4, 520, 96), (4, 500, 96)]),
+    # guarded factors: a convolution that pads by one with zeros (AntaresIR.md:166), in float32 and with fp16 tiles; a
+    # product whose first operand is shifted along k and cut where it runs out, lanes along k
+    ('output0[N, F, HO, WO] +=! input0[N, C, HO + KH - 1, WO + KW - 1].when([HO + KH - 1 >= 0, HO + KH - 1 < 32, WO + KW - 1 >= 0, '
+     'WO + KW - 1 < 32], 0.0) * input1[F, C, KH, KW] where HO in 32, WO in 32',
+     ['input0=float32[N:6, C:16, H:32, W:32]', 'input1=float32[F:64, C:16, KH:3, KW:3]'], [(6, 16, 32, 32), (64, 16, 3, 3)]),
+    ('output0[N, F, HO, WO] +=! input0[N, C, HO + KH - 1, WO + KW - 1].to(`float32`).when([HO + KH - 1 >= 0, HO + KH - 1 < 30, '
+     'WO + KW - 1 >= 0, WO + KW - 1 < 30], 0.0) * input1[F, C, KH, KW].to(`float32`) where HO in 30, WO in 30',
+     ['input0=float16[N:5, C:20, H:30, W:30]', 'input1=float16[F:72, C:20, KH:3, KW:3]'], [(5, 20, 30, 30), (72, 20, 3, 3)]),
+    ('output0[N, M] +=! input0[N, K + 5].when([K + 5 < 80], 0.0) * input1[K, M] where K in 80',
+     ['input0=float32[N:1024, J:80]', 'input1=float32[K:80, M:1024]'], [(1024, 80), (80, 1024)]),
 ]
 
 

@@ -89,3 +89,31 @@ def test_row_kernels_compile_for_gfx950(tmp_path, monkeypatch):
     src, plans = lowered(ir, ['x=float16[B:3, N:17, C:520]', 'w=float16[C:520]'])
     assert plans[0].row_group is not None and plans[0].row_group.count == 2
     assert len(compile_cached(src)) > 1000
+
+
+PADDED_CONV = ('output0[N, F, HO, WO] +=! input0[N, C, HO + KH - 1, WO + KW - 1].when([HO + KH - 1 >= 0, HO + KH - 1 < 56, '
+               'WO + KW - 1 >= 0, WO + KW - 1 < 56], 0.0) * input1[F, C, KH, KW] where HO in 56, WO in 56')
+
+
+def test_a_padded_convolution_goes_to_the_matrix_kernels_with_its_guards_tabled(tmp_path, monkeypatch):
+    """AntaresIR.md:166: the zero padding is a `when` around the image operand.  Its four conditions compare two values,
+    each a row part plus a k part; the kernels table those beside the addresses and never fetch outside them."""
+    monkeypatch.setenv('AUTORT_CACHE_DIR', str(tmp_path / 'cache'))
+    from antares_amd.autort.op import compile_cached
+    graph = fuse_elementwise(parse_program(PADDED_CONV, ['input0=float32[N:8, C:64, H:56, W:56]', 'input1=float32[F:64, C:64, KH:3, KW:3]']))
+    mc = hip_codegen._matrix_contraction(graph.statements[0], graph.tensors)
+    assert [g[2] for g in mc['guards']['a']] == ['<=', '<', '<=', '<'] and mc['guards']['b'] == []
+    assert len({(g[0], g[1]) for g in mc['guards']['a']}) == 2 and not mc['vec']['a']
+    src, plans = hip_codegen.lower_graph(graph)
+    assert {'matrix', 'matrix64'} <= set(plans[0].variants) and 'matrixv' not in plans[0].variants
+    assert '__gma[2][128]' in src and '__gma[2][64]' in src
+    # 25088 rows x 64 columns: tiles of 128 columns would be half padding, the small tiles take it
+    env = {'N': 8, 'C': 64, 'H': 56, 'W': 56, 'F': 64, 'KH': 3, 'KW': 3}
+    assert plans[0]._matrix_choice(env, {n: 0 for n in plans[0].args}) == ('matrix64', 392)
+    assert plans[0]._matrix_choice({**env, 'F': 128}, {n: 0 for n in plans[0].args}) == ('matrix', 196)
+    assert len(compile_cached(src)) > 1000
+    # a guard that mixes rows and k in a product, or reads a tensor, leaves the statement to the other variants
+    for cond in ('HO * KH < 56', 'input1[F, C, KH, KW] > 0'):
+        ir = f'output0[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW].when([{cond}], 0.0) * input1[F, C, KH, KW] where HO in 54, WO in 54'
+        g2 = fuse_elementwise(parse_program(ir, ['input0=float32[N:8, C:64, H:56, W:56]', 'input1=float32[F:64, C:64, KH:3, KW:3]']))
+        assert hip_codegen._matrix_contraction(g2.statements[0], g2.tensors) is None
