@@ -1233,14 +1233,17 @@ def _matrix_contraction(st, tensors):
                 return None
             conds.append((sp_c[0] or '0', sp_c[1] or '0', c.name, plain.expr(c.args[1 if left else 0]), left))
         guards[tag] = conds
-    # an operand whose last index is THE reduce axis, bare, and whose last extent is that axis' extent, lies in memory
-    # as rows of k: 16-byte vectors of k can be fetched when k is a multiple of the vector and the tensor is aligned
+    # an operand whose last indices are THE reduce axes, bare and in their order, over dimensions of exactly their
+    # extents (`input1[F, C, KH, KW]` of a convolution; the `[N, K]` of a product), lies in memory as rows of k:
+    # 16-byte vectors of k can be fetched when k is a multiple of the vector and the tensor is aligned
     vec = {}
+    red = dict(st.reduce_axes)
     for tag, ld in (('a', la), ('b', lb)):
-        last = ld.args[-1]
-        vec[tag] = (len(k_axes) == 1 and last.kind == 'axis' and last.name == k_axes[0] and
-                    not any(k_axes[0] in _axes_of(a) for a in ld.args[:-1]) and
-                    tensors[ld.name].shape[-1] == dict(st.reduce_axes)[k_axes[0]] and not guards[tag])
+        nk = len(k_axes)
+        tail = ld.args[-nk:] if len(ld.args) >= nk else []
+        vec[tag] = (len(tail) == nk and all(ix.kind == 'axis' and ix.name == k for ix, k in zip(tail, k_axes)) and
+                    not any(set(k_axes) & _axes_of(a) for a in ld.args[:-nk]) and
+                    all(d == red[k] for d, k in zip(tensors[ld.name].shape[-nk:], k_axes)) and not guards[tag])
     return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts, 'vec': vec,
             'guards': guards}
 

@@ -105,12 +105,15 @@ def test_a_padded_convolution_goes_to_the_matrix_kernels_with_its_guards_tabled(
     assert [g[2] for g in mc['guards']['a']] == ['<=', '<', '<=', '<'] and mc['guards']['b'] == []
     assert len({(g[0], g[1]) for g in mc['guards']['a']}) == 2 and not mc['vec']['a']
     src, plans = hip_codegen.lower_graph(graph)
-    assert {'matrix', 'matrix64'} <= set(plans[0].variants) and 'matrixv' not in plans[0].variants
+    # the guarded image is fetched element by element; the weights lie as rows of k = (C, KH, KW): 16-byte vectors
+    assert mc['vec']['b'] and {'matrix', 'matrix64', 'matrixv', 'matrix64v'} <= set(plans[0].variants)
+    assert plans[0].matrix['vec_tensors'] == ['input1']
     assert '__gma[2][128]' in src and '__gma[2][64]' in src
     # 25088 rows x 64 columns: tiles of 128 columns would be half padding, the small tiles take it
     env = {'N': 8, 'C': 64, 'H': 56, 'W': 56, 'F': 64, 'KH': 3, 'KW': 3}
-    assert plans[0]._matrix_choice(env, {n: 0 for n in plans[0].args}) == ('matrix64', 392)
-    assert plans[0]._matrix_choice({**env, 'F': 128}, {n: 0 for n in plans[0].args}) == ('matrix', 196)
+    assert plans[0]._matrix_choice(env, {n: 0 for n in plans[0].args}) == ('matrix64v', 392)
+    assert plans[0]._matrix_choice({**env, 'F': 128}, {n: 0 for n in plans[0].args}) == ('matrixv', 196)
+    assert plans[0]._matrix_choice(env, {**{n: 0 for n in plans[0].args}, 'input1': 4}) == ('matrix64', 392)
     assert len(compile_cached(src)) > 1000
     # a guard that mixes rows and k in a product, or reads a tensor, leaves the statement to the other variants
     for cond in ('HO * KH < 56', 'input1[F, C, KH, KW] > 0'):
