@@ -18,7 +18,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..ir import Graph, fuse_elementwise, parse_program, split_wide_reductions
+from ..ir import Graph, bake_small_reduce_extents, fuse_elementwise, parse_program, split_wide_reductions
 from ..lower import lower_graph
 from ..runtime import capi
 
@@ -185,13 +185,15 @@ class ExportedOp:
 
     def _variant(self, env: Dict[str, int]) -> dict:
         """Graph, plans and module for these values of the named dimensions: the default ones, unless a reduction
-        of the program is worth slicing at these sizes (split_wide_reductions), which needs its own kernels."""
+        of the program is worth slicing at these sizes (split_wide_reductions) or runs over a window of a few elements
+        given by named dimensions (bake_small_reduce_extents), which need their own kernels."""
         key = tuple(env[d] for d in self.fused.dim_names)
         v = self._variants.get(key)
         if v is None:
             # rows that one row kernel reduces and maps in a single launch are not sliced
             in_rows = any(p.row_group is not None and p.row_group.choose(env, {n: 0 for n in p.row_group.args})[1] for p in self.plans)
-            g = split_wide_reductions(self.lowered, env) if self.fused.dims and not in_rows else self.lowered
+            g = bake_small_reduce_extents(self.lowered, env) if self.fused.dims else self.lowered
+            g = split_wide_reductions(g, env) if self.fused.dims and not in_rows else g
             if g is self.lowered:
                 v = {'graph': self.lowered, 'plans': self.plans, 'module': None, 'source': None}
             else:
@@ -202,6 +204,11 @@ class ExportedOp:
         if v['module'] is None:
             v['module'] = self._load() if v['source'] is None else capi.Module(compile_cached(v['source']))
         return v
+
+    def plans_for(self, env: Dict[str, int]) -> list:
+        """The kernel plans (one per statement of the lowered graph) that a call with these values of the named
+        dimensions launches from."""
+        return self._variant(env)['plans']
 
     def _run_generic(self, bound: Dict[str, torch.Tensor], env: Dict[str, int], dev, stream: int):
         variant = self._variant(env)

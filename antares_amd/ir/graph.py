@@ -230,6 +230,27 @@ def _divisor_near(extent: int, target: int) -> int:
     return best
 
 
+def bake_small_reduce_extents(graph: Graph, env: Dict[str, int], limit: int = 8) -> Graph:
+    """Named dimensions that are the extent of a reduce axis and at most `limit` in this call (the window of a
+    pooling, the filter of a convolution given as `input1[F, C, KH:3, KW:3]`) become constants of the graph: the
+    lowering then writes loops the compiler unrolls, divides by constants and keeps one copy of the loads that the
+    terms of neighbouring outputs share.  The kernels keep all dimensions as arguments; the result is valid for these
+    values only and the caller keeps it per shape.  The same graph object comes back when nothing is small."""
+    small = {d: env[d] for st in graph.statements for _, d in st.reduce_axes
+             if isinstance(d, str) and env.get(d) is not None and 0 < env[d] <= limit}
+    if not small:
+        return graph
+
+    def fix(dims):
+        return [small.get(d, d) if isinstance(d, str) else d for d in dims]
+    tensors = {n: replace(t, shape=fix(t.shape)) for n, t in graph.tensors.items()}
+    statements = [replace(st, data_axes=[(a, small.get(d, d) if isinstance(d, str) else d) for a, d in st.data_axes],
+                          reduce_axes=[(a, small.get(d, d) if isinstance(d, str) else d) for a, d in st.reduce_axes],
+                          out_shape=fix(st.out_shape)) for st in graph.statements]
+    return Graph(statements=statements, tensors=tensors, declared=graph.declared, outputs=graph.outputs, dims=graph.dims,
+                 source=graph.source)
+
+
 def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None) -> Graph:
     """A reduction whose outputs are too few to fill the chip is rewritten as
 
@@ -280,7 +301,7 @@ def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None) ->
             continue
         target = max(2, min(want_outputs // max(outputs, 1), extent * inner // min_chunk, extent))
         S = _divisor_near(extent, target)
-        if S < 2 or S >= extent:
+        if S < 2 or S > extent or (S == extent and inner == 1):     # a slice per value of the axis: only when other reduce axes remain
             out.append(st)
             continue
         chunk = extent // S

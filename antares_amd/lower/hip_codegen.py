@@ -388,10 +388,24 @@ def _extents(st) -> List[str]:
     return [f'  const int __ext_{ax} = {dim_c(e)}; (void)__ext_{ax};' for ax, e in st.data_axes + st.reduce_axes]
 
 
-def _decompose(var: str, axes, indent: str) -> List[str]:
-    out = [f'{indent}long long __r = {var};']
+def _decompose(var: str, axes, indent: str, bound: Optional[str] = None, tmp: str = '__r') -> List[str]:
+    """The axis values of flat position `var`, last axis fastest.  With `bound` (C text of an exclusive upper limit of
+    `var`) the divisions are 32-bit whenever that limit fits: a 64-bit division by a run-time value costs this part
+    some hundred instructions, and a thread-per-output kernel makes one per axis and output."""
+    if bound is None or not axes:
+        out = [f'{indent}long long {tmp} = {var};']
+        for ax, _ in reversed(axes):
+            out.append(f'{indent}const int {ax} = (int)({tmp} % __ext_{ax}); {tmp} /= __ext_{ax};')
+        return out
+    out = [f'{indent}int ' + ', '.join(ax for ax, _ in axes) + ';',
+           f'{indent}if ({bound} <= 0x7fffffffLL) {{', f'{indent}  unsigned int {tmp} = (unsigned int)({var});']
     for ax, _ in reversed(axes):
-        out.append(f'{indent}const int {ax} = (int)(__r % __ext_{ax}); __r /= __ext_{ax};')
+        out.append(f'{indent}  {ax} = (int)({tmp} % (unsigned int)__ext_{ax}); {tmp} /= (unsigned int)__ext_{ax};')
+    out += [f'{indent}}} else {{', f'{indent}  long long {tmp} = {var};']
+    for ax, _ in reversed(axes):
+        out.append(f'{indent}  {ax} = (int)({tmp} % __ext_{ax}); {tmp} /= __ext_{ax};')
+    out.append(f'{indent}}}')
+    out.append(indent + ' '.join(f'(void){ax};' for ax, _ in axes))
     return out
 
 
@@ -525,7 +539,7 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
         sym = name
         body = header(sym)
         body.append('  for (long long __i = __tid; __i < __total; __i += __nthr) {')
-        body += _decompose('__i', st.data_axes, '    ')
+        body += _decompose('__i', st.data_axes, '    ', '__total')
         store = f'{dst} = ({oct_})({em.expr(root)});'
         body.append(f'    if ({cond}) {{ {store} }}' if cond else f'    {store}')
         body += ['  }', '}']
@@ -562,7 +576,7 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
                 body.append(f'    __builtin_nontemporal_store(__out, &{dst_});' if streamed(st.output) else f'    {dst_} = __out;')
                 body.append('  }')
                 body.append(f'  for (long long __i = __nvec * {V} + __tid; __i < __total; __i += __nthr) {{')
-                body += _decompose('__i', st.data_axes, '    ')
+                body += _decompose('__i', st.data_axes, '    ', '__total')
                 body.append(f'    {dst} = ({oct_})({em.expr(root)});')
                 body += ['  }', '}']
                 src.append('\n'.join(body))
@@ -703,7 +717,7 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
         sym = name
         body = header(sym)
         body.append('  for (long long __i = __tid; __i < __total; __i += __nthr) {')
-        body += _decompose('__i', st.data_axes, '    ')
+        body += _decompose('__i', st.data_axes, '    ', '__total')
         val = f'({oct_})({em.expr(root)})'
         store = {'set': f'{dst} = {val};', 'add': f'atomicAdd(&{dst}, {val});',
                  'min': f'atomicMin(&{dst}, {val});', 'max': f'atomicMax(&{dst}, {val});'}[st.set_op]
@@ -726,13 +740,23 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
             if sym.endswith('_b'):
                 b.append(f'  __shared__ {act} __smem[4];')
             b.append(f'  for (long long __o = {out_var}; __o < __total; __o += {out_step}) {{')
-            b += _decompose('__o', st.data_axes, '    ')
+            b += _decompose('__o', st.data_axes, '    ', '__total')
             b.append(f'    {act} __acc = {ident};')
-            b.append('    #pragma unroll 4')
-            b.append(f'    for (long long __k = {lane}; __k < __red; __k += {nlanes}) {{')
-            b += [l.replace('__r', '__q') for l in _decompose('__k', st.reduce_axes, '      ')]
-            b.append(f'      __acc = {op}(__acc, ({act})({em.expr(root)}));')
-            b.append('    }')
+            if nlanes == '1':
+                # a thread walks all of the reduce space: one loop per reduce axis, in the same order as the flat walk,
+                # no divisions - a pooling window or a depthwise filter is then a handful of adds per term
+                for d, (ax, _) in enumerate(st.reduce_axes):
+                    if d == len(st.reduce_axes) - 1:
+                        b.append('    ' + '  ' * d + '#pragma unroll 4')
+                    b.append('    ' + '  ' * d + f'for (int {ax} = 0; {ax} < __ext_{ax}; ++{ax})' + (' {' if d == len(st.reduce_axes) - 1 else ''))
+                b.append('    ' + '  ' * len(st.reduce_axes) + f'__acc = {op}(__acc, ({act})({em.expr(root)}));')
+                b.append('    ' + '  ' * (len(st.reduce_axes) - 1) + '}')
+            else:
+                b.append('    #pragma unroll 4')
+                b.append(f'    for (long long __k = {lane}; __k < __red; __k += {nlanes}) {{')
+                b += _decompose('__k', st.reduce_axes, '      ', '__red', tmp='__q')
+                b.append(f'      __acc = {op}(__acc, ({act})({em.expr(root)}));')
+                b.append('    }')
             b += finish
             b += ['  }', '}']
             return '\n'.join(b)
@@ -764,21 +788,28 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
             b.append(f'  const long long __px = __ext_{xa} / {TX}, __py = __ext_{ya} / {TY};')
             b.append(f'  const long long __patches = __total / {TX * TY};')
             b.append('  for (long long __o = __tid; __o < __patches; __o += __nthr) {')
-            b.append('    long long __r = __o;')
-            for ax, _ in reversed(st.data_axes):
-                if ax == ya:
-                    b.append(f'    const int __y0 = (int)(__r % __py) * {TY}; __r /= __py;')
-                elif ax == xa:
-                    b.append(f'    const int __x0 = (int)(__r % __px) * {TX}; __r /= __px;')
-                else:
-                    b.append(f'    const int {ax} = (int)(__r % __ext_{ax}); __r /= __ext_{ax};')
+            others = [ax for ax, _ in st.data_axes if ax not in (xa, ya)]
+            b.append('    int __x0, __y0' + ''.join(f', {ax}' for ax in others) + ';')
+            for small in (True, False):         # 32-bit divisions whenever the patch count fits them
+                b.append('    if (__patches <= 0x7fffffffLL) {' if small else '    } else {')
+                b.append('      unsigned int __r = (unsigned int)__o;' if small else '      long long __r = __o;')
+                cast = '(unsigned int)' if small else ''
+                for ax, _ in reversed(st.data_axes):
+                    if ax == ya:
+                        b.append(f'      __y0 = (int)(__r % {cast}__py) * {TY}; __r /= {cast}__py;')
+                    elif ax == xa:
+                        b.append(f'      __x0 = (int)(__r % {cast}__px) * {TX}; __r /= {cast}__px;')
+                    else:
+                        b.append(f'      {ax} = (int)(__r % {cast}__ext_{ax}); __r /= {cast}__ext_{ax};')
+            b.append('    }')
+            b.append('    ' + ' '.join(f'(void){ax};' for ax in others))
             b.append(f'    {act} __acc[{TX}][{TY}];')
             b.append('    #pragma unroll')
             b.append(f'    for (int __i = 0; __i < {TX}; ++__i)')
             b.append('      #pragma unroll')
             b.append(f'      for (int __j = 0; __j < {TY}; ++__j) __acc[__i][__j] = {ident};')
-            b.append('    for (long long __k = 0; __k < __red; ++__k) {')
-            b += [l.replace('__r', '__q') for l in _decompose('__k', st.reduce_axes, '      ')]
+            for d, (ax, _) in enumerate(st.reduce_axes):       # one loop per reduce axis, in the order of the flat walk
+                b.append('    ' + ' ' * d + f'for (int {ax} = 0; {ax} < __ext_{ax}; ++{ax})' + (' {' if d == len(st.reduce_axes) - 1 else ''))
             b.append('      #pragma unroll')
             b.append(f'      for (int __i = 0; __i < {TX}; ++__i) {{')
             b.append('        #pragma unroll')

@@ -583,6 +583,16 @@ def test_row_vector_maps_match_the_oracle(autort, ir, inputs, shapes, applies):
         assert np.array_equal(got2, got)
 
 
+def dims_of(inputs, shapes):
+    """{named dimension: value} of tensors of these shapes for input specs like `input0=float32[N:8, C:16]`."""
+    env = {}
+    for spec, shape in zip(inputs, shapes):
+        for d, v in zip(spec.split('[', 1)[1].rstrip(']').split(','), shape):
+            if ':' in d:
+                env[d.split(':')[0].strip()] = v
+    return env
+
+
 PATCH_CASES = [
     ('output0[N, M] +=! input0[N, K] * input1[K, M]', ['input0=float32[N:64, K:96]', 'input1=float32[K:96, M:128]'], [(64, 96), (96, 128)]),
     ('output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]', ['input0=float32[B:3, N:32, K:40]', 'input1=float32[B:3, K:40, M:64]'],
@@ -591,6 +601,9 @@ PATCH_CASES = [
     ('output0[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[F, C, KH, KW] where HO in 10, WO in 12',
      ['input0=float32[N:2, C:5, H:12, W:14]', 'input1=float32[F:8, C:5, KH:3, KW:3]'], [(2, 5, 12, 14), (8, 5, 3, 3)]),
     ('output0[N, M] >=! input0[N, K] + input1[K, M]', ['input0=int32[N:16, K:33]', 'input1=int32[K:33, M:20]'], [(16, 33), (33, 20)]),
+    # a depthwise filter whose size comes as named dimensions: the kernels of this call have 3 x 3 written into them
+    ('output0[N, C, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[C, KH, KW] where HO in 12, WO in 16',
+     ['input0=float32[N:3, C:7, H:14, W:18]', 'input1=float32[C:7, KH:3, KW:3]'], [(3, 7, 14, 18), (7, 3, 3)]),
 ]
 
 
@@ -603,7 +616,7 @@ def test_register_tiled_contractions_match_the_oracle(autort, ir, inputs, shapes
     note(f'register-tiled reduce {ir} {shapes}')
     dev = autort.device()
     op = autort.export(ir=ir, inputs=inputs, name='patch_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
-    plan = op.plans[0]
+    plan = op.plans_for(dims_of(inputs, shapes))[0]
     assert 'patch' in plan.variants
     g = torch.Generator().manual_seed(len(ir))
     names = [spec.split('=')[0] for spec in inputs]
@@ -699,11 +712,8 @@ def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, ir, in
     dev = autort.device()
     op = autort.export(ir=ir, inputs=inputs, name='mfma_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
     op.fast_path = None
-    plan = op.plans[-1]
-    env = {}
-    for spec, shape in zip(inputs, shapes):
-        for d, v in zip(spec.split('[', 1)[1].rstrip(']').split(','), shape):
-            env[d.split(':')[0].strip()] = v
+    env = dims_of(inputs, shapes)
+    plan = op.plans_for(env)[-1]                  # a filter of a few named elements gets kernels of its own
     assert plan.choose(env, {n: 0 for n in plan.args})[0] in [v for t, v in plan.variants.items() if t.startswith('matrix')]
     assert plan.row_group is None                 # nothing else takes the statement
     g = torch.Generator().manual_seed(len(ir))

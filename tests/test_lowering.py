@@ -120,3 +120,36 @@ def test_a_padded_convolution_goes_to_the_matrix_kernels_with_its_guards_tabled(
         ir = f'output0[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW].when([{cond}], 0.0) * input1[F, C, KH, KW] where HO in 54, WO in 54'
         g2 = fuse_elementwise(parse_program(ir, ['input0=float32[N:8, C:64, H:56, W:56]', 'input1=float32[F:64, C:64, KH:3, KW:3]']))
         assert hip_codegen._matrix_contraction(g2.statements[0], g2.tensors) is None
+
+
+def test_graph_rewrites_for_one_call_keep_the_program_on_the_oracle():
+    """Two rewrites made per set of dimension values: a reduction over (N, H, W) with few outputs is sliced along all of
+    N, and reduce extents of a few named elements become constants.  Both leave the oracle's results where they were."""
+    import numpy as np
+    from antares_amd.ir.graph import bake_small_reduce_extents, split_wide_reductions
+    from oracle.cpu_backend import CpuModule
+    rng = np.random.default_rng(5)
+    # channel sums: 24 outputs, the outermost reduce axis has 16 values and is sliced into 16
+    prog = parse_program('output0[C] +=! input0[N, C, H, W]', ['input0=float32[N:16, C:24, H:20, W:20]'])
+    env = {'N': 16, 'C': 24, 'H': 20, 'W': 20}
+    sliced = split_wide_reductions(fuse_elementwise(prog), env)
+    assert len(sliced.statements) == 2 and sliced.statements[0].data_axes[0][1] == 16
+    assert [e for _, e in sliced.statements[0].reduce_axes] == [1, 'H', 'W']
+    x = rng.standard_normal((16, 24, 20, 20)).astype(np.float32)
+    assert np.allclose(CpuModule(sliced, fast_math=False)(input0=x)['output0'], x.astype(np.float64).sum((0, 2, 3)), rtol=1e-5, atol=1e-3)
+    # a single reduce axis is never sliced into slices of one element
+    one = split_wide_reductions(fuse_elementwise(parse_program('output0[C] +=! input0[N, C]', ['input0=float32[N:16, C:24]'])), {'N': 16, 'C': 24})
+    assert len(one.statements) == 1
+    # a depthwise filter of named size 3 x 3; a filter of 9 x 9 stays symbolic
+    ir = 'output0[N, C, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[C, KH, KW] where HO in 6, WO in 6'
+    inputs = ['input0=float32[N:2, C:3, H:8, W:8]', 'input1=float32[C:3, KH:3, KW:3]']
+    g = fuse_elementwise(parse_program(ir, inputs))
+    env = {'N': 2, 'C': 3, 'H': 8, 'W': 8, 'KH': 3, 'KW': 3}
+    baked = bake_small_reduce_extents(g, env)
+    assert baked is not g and baked.statements[0].reduce_axes == [('KH', 3), ('KW', 3)] and baked.tensors['input1'].shape == ['C', 3, 3]
+    assert baked.dim_names == g.dim_names                  # the kernels keep every dimension as an argument
+    assert bake_small_reduce_extents(g, {**env, 'KH': 9, 'KW': 9}) is g
+    a, w = rng.standard_normal((2, 3, 8, 8)).astype(np.float32), rng.standard_normal((3, 3, 3)).astype(np.float32)
+    assert np.array_equal(CpuModule(baked, fast_math=False)(input0=a, input1=w)['output0'], CpuModule(g, fast_math=False)(input0=a, input1=w)['output0'])
+    src, plans = hip_codegen.lower_graph(baked)
+    assert 'const int __ext_KH = 3;' in src and 'int __dim_KH' in src
