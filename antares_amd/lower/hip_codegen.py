@@ -868,7 +868,7 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         return f.kind == 'cast' and f.dtype == 'float32' and f.args[0] is ld and tensors[ld.name].dtype == 'float16'
     # fp16 operands that are only cast up: the tiles stay fp16 in LDS and go to v_mfma_f32_32x32x16_f16 - the
     # products of two fp16 values are exact in float32 either way, and the matrix time is a sixteenth
-    HM = half_cast(mc['fa'], la) and half_cast(mc['fb'], lb)
+    HM = (half_cast(mc['fa'], la) and half_cast(mc['fb'], lb)) or st.root.dtype == 'float16'
     BK = 32 if (TS == 64 or HM) else 16               # k per tile: the small blocks take twice the k per barrier
     LD, RS = BK + (8 if HM else 4), BLOCK // BK       # elements per row of a staged tile (16-byte aligned, rows on distinct banks); rows between a lane's elements when lanes walk k
     ET = 'half_t' if HM else 'float'                  # element type of the staged tiles
@@ -1197,7 +1197,7 @@ def _matrix_contraction(st, tensors):
     data axes that only the first load uses are rows (M), those only the second uses are columns (N), those both use
     are a batch, the reduce axes are k.  Every index of a load must split into a part that depends on k axes and a
     part that does not, so that an element's address is a row (column) offset plus a k offset.  -> dict or None."""
-    if st.scatter or st.reduce != '+' or st.root.dtype != 'float32' or not st.reduce_axes or not st.data_axes:
+    if st.scatter or st.reduce != '+' or st.root.dtype not in ('float32', 'float16') or not st.reduce_axes or not st.data_axes:
         return None
     root = st.root
     if root.kind == 'when' or root.kind != 'op' or root.name != '*' or len(root.args) != 2:
@@ -1224,6 +1224,11 @@ def _matrix_contraction(st, tensors):
         return None
     la, lb = la[0], lb[0]
     if any(n.kind in ('load', 'when') for tag in guards for c in guards[tag] for n in walk(c)):
+        return None
+    # A float16 statement (AntaresIR.md:115 with float16 tensors; the reference rounds every product and every partial
+    # sum to float16) is taken only as the product of two float16 loads: the matrix instruction multiplies them
+    # exactly and sums in float32, the result is rounded once - closer to the exact sum than the running float16 sum.
+    if st.root.dtype == 'float16' and not (fa is la and fb is lb and tensors[la.name].dtype == tensors[lb.name].dtype == 'float16'):
         return None
     # axes may be used inside the indices of the two loads and inside the guards only
     inside = sum(1 for n in (la, lb) for a in n.args for m in walk(a) if m.kind == 'axis') + \

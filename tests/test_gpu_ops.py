@@ -748,6 +748,42 @@ def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, ir, in
     assert np.allclose(got, apart, rtol=1e-4, atol=tol)
 
 
+@pytest.mark.parametrize('ir,inputs,shapes', [
+    ('output0[N, M] +=! input0[N, K] * input1[K, M]', ['input0=float16[N:1024, K:512]', 'input1=float16[K:512, M:1000]'], [(1024, 512), (512, 1000)]),
+    ('output0[B, N, M] +=! input0[B, N, K] * input1[B, M, K]', ['input0=float16[B:3, N:300, K:200]', 'input1=float16[B:3, M:260, K:200]'],
+     [(3, 300, 200), (3, 260, 200)]),
+])
+def test_fp16_contractions_sum_in_float32_on_the_matrix_instructions(autort, ir, inputs, shapes):
+    """A float16 sum of products of two float16 loads (AntaresIR.md:115 with float16 tensors) runs on
+    v_mfma_f32_32x32x16_f16: exact products, a float32 sum, one rounding at the end.  The reference rounds every product
+    and every partial sum to float16 (the oracle does the same); the GPU result must be within one float16 rounding
+    of the float64 result, never further from it than the oracle's, and within the oracle's own drift of the oracle."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'fp16 contraction on the matrix instructions {ir} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='mfma_f16_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    op.fast_path = None
+    env = dims_of(inputs, shapes)
+    plan = op.plans_for(env)[-1]
+    g = torch.Generator().manual_seed(len(ir))
+    a, b = [(torch.randn(shape, generator=g) * 0.5).half() for shape in shapes]
+    want = CpuModule(parse_program(ir, inputs), fast_math=False)(input0=a.numpy(), input1=b.numpy())['output0'].astype(np.float64)
+    exact = torch.einsum('...nk,...km->...nm', a.double(), b.double() if ir.endswith('[K, M]') else b.double().transpose(-1, -2)).numpy()
+    drift = np.abs(want - exact).max()
+    M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
+    assert plan.choose(env, {n: 0 for n in plan.args})[0] in (plan.variants['matrixv'], plan.variants['matrix64v'])
+    for tag, side in (('matrix', 128), ('matrix64', 64), ('matrixv', 128), ('matrix64v', 64)):
+        blocks = ((M + side - 1) // side) * ((N + side - 1) // side) * B
+        plan.choose = lambda env_, ptrs, tag=tag, blocks=blocks: (plan.variants[tag], blocks, 256)
+        out = op(a.to(dev), b.to(dev))
+        assert out.dtype == torch.float16 and tuple(out.shape) == exact.shape
+        got = out.cpu().numpy().astype(np.float64)
+        # one float16 rounding of the result, plus what a float32 sum of K terms of this size may be off by
+        assert np.all(np.abs(got - exact) <= 2.0 ** -10 * np.abs(exact) + 2e-4), (tag, np.abs(got - exact).max())
+        assert np.abs(got - exact).max() <= drift and np.abs(got - want).max() <= 2 * drift + 1e-3, (tag, drift)
+
+
 ROW_GROUP_CASES = [
     # program, inputs, shapes, does the row kernel run at these extents
     ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
