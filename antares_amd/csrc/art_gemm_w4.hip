@@ -321,8 +321,9 @@ __global__ __launch_bounds__(256) void gemm_w4a16_combine_kernel(const float* __
 }
 
 // Number of K-splits: as many blocks as the chip holds at once (one per compute unit), but at least
-// two groups per block, no more partial-tile bytes than weight bytes (every split adds an fp32 copy of
-// the output to the traffic), and no more than the scratch space allows.  The rule lands on the measured
+// two groups per block, no more partial-tile bytes than twice the weight bytes (every split adds an fp32 copy of
+// the output to the traffic; 256 rows over 4096 x 4096: 4 splits 23.1 us, the 2 that the weight bytes allow 28.3),
+// and no more than the scratch space allows.  The rule lands on the measured
 // optimum at M = 64 on MI355X: 8 splits for 4096x4096 and 11008x4096 (two 32-row blocks each), 5 for 4096x11008,
 // 2 for 4096x32000.
 int choose_splits(int rows, int N, int K, size_t scratch_bytes, int compute_units) {
@@ -331,7 +332,7 @@ int choose_splits(int rows, int N, int K, size_t scratch_bytes, int compute_unit
   if (s > G / 2) s = G / 2;
   const size_t per_split = (size_t)rows * N * sizeof(float);
   const size_t weight_bytes = (size_t)K * N / 2;
-  if ((size_t)s * per_split > weight_bytes) s = (int)(weight_bytes / per_split);
+  if ((size_t)s * per_split > 2 * weight_bytes) s = (int)(2 * weight_bytes / per_split);
   const int cap = (int)(scratch_bytes / per_split);
   if (s > cap) s = cap;
   return s < 1 ? 1 : s;
@@ -389,10 +390,12 @@ extern "C" int art_gemm_w4a16_residual(const void* x_dev, const void* qweight_de
   ART_REQUIRE(want_rows <= 2, "art_gemm_w4a16: rows-per-block code must be 0, 1 or 2 (got %d)", want_rows);
   int block_rows = BM;
   if (want_rows == 1 || M <= 32) block_rows = 32;
-  else if (want_rows == 0 && M <= 64) {
-    // measured at M = 64 on MI355X: 32-row blocks win where one block per compute unit then covers at least four
-    // K-splits' worth of column tiles (4096 columns), and lose where they would need a second round of blocks
-    if (col_tiles * 2 * 4 <= compute_units) block_rows = 32;
+  else if (want_rows == 0 && (M <= 64 || (M <= 128 && K <= 8192))) {
+    // measured at M = 64 and 128 on MI355X: 32-row blocks win where one block per compute unit then covers at least
+    // four K-splits' worth of (column tile, row block) pairs (M = 64: up to 8192 columns, M = 128: 4096), and lose
+    // where they would need a second round of blocks; beyond 64 rows also where the loop over K is long (128 rows
+    // over 11008 x 4096: 27.2 us against 25.8 with 64-row blocks; over 4096 x 4096: 17.3 against 19.7)
+    if (col_tiles * ((M + 31) / 32) * 4 <= compute_units) block_rows = 32;
   }
   for (int m0 = 0; m0 < M; m0 += block_rows * kMaxRowBlocks) {
     const int rows = M - m0 < block_rows * kMaxRowBlocks ? M - m0 : block_rows * kMaxRowBlocks;
