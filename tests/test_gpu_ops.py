@@ -698,6 +698,10 @@ MATRIX_CASES = [
      ['input0=float16[N:5, C:20, H:30, W:30]', 'input1=float16[F:72, C:20, KH:3, KW:3]'], [(5, 20, 30, 30), (72, 20, 3, 3)]),
     ('output0[N, M] +=! input0[N, K + 5].when([K + 5 < 80], 0.0) * input1[K, M] where K in 80',
      ['input0=float32[N:1024, J:80]', 'input1=float32[K:80, M:1024]'], [(1024, 80), (80, 1024)]),
+    # the guarded factor second: the filter's output channels are the rows, the padded image's positions the columns
+    ('output0[F, N, HO, WO] +=! input1[F, C, KH, KW] * input0[N, C, HO + KH - 2, WO + KW - 2].when([HO + KH - 2 >= 0, HO + KH - 2 < 20, '
+     'WO + KW - 2 >= 0, WO + KW - 2 < 24], 0.0) where HO in 20, WO in 24',
+     ['input0=float32[N:4, C:12, H:20, W:24]', 'input1=float32[F:96, C:12, KH:5, KW:5]'], [(4, 12, 20, 24), (96, 12, 5, 5)]),
 ]
 
 
