@@ -19,7 +19,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from ..ir import Graph, bake_small_reduce_extents, fuse_elementwise, parse_program, split_wide_reductions
-from ..lower import lower_graph
+from ..lower import contraction_slices, lower_graph
 from ..runtime import capi
 
 TORCH_DTYPE = {'float64': torch.float64, 'float32': torch.float32, 'float16': torch.float16,
@@ -84,7 +84,7 @@ class ExportedOp:
         self.fresh_outputs = [o for o in self.graph.outputs if o not in self.declared]
         # what the generic lowering compiles: wide reductions with few outputs become two statements (statically
         # sized ones here; programs with named dimensions get a variant per set of values at call time)
-        self.lowered: Graph = split_wide_reductions(self.fused)
+        self.lowered: Graph = split_wide_reductions(self.fused, wanted=contraction_slices(self.fused.tensors))
         self.source, self.plans = lower_graph(self.lowered, prefix='autort_' + _ident(self.name))
         self._variants: Dict[tuple, dict] = {}
         self._module: Optional[capi.Module] = None
@@ -193,7 +193,7 @@ class ExportedOp:
             # rows that one row kernel reduces and maps in a single launch are not sliced
             in_rows = any(p.row_group is not None and p.row_group.choose(env, {n: 0 for n in p.row_group.args})[1] for p in self.plans)
             g = bake_small_reduce_extents(self.lowered, env) if self.fused.dims else self.lowered
-            g = split_wide_reductions(g, env) if self.fused.dims and not in_rows else g
+            g = split_wide_reductions(g, env, wanted=contraction_slices(g.tensors)) if self.fused.dims and not in_rows else g
             if g is self.lowered:
                 v = {'graph': self.lowered, 'plans': self.plans, 'module': None, 'source': None}
             else:

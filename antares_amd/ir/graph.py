@@ -251,7 +251,7 @@ def bake_small_reduce_extents(graph: Graph, env: Dict[str, int], limit: int = 8)
                  source=graph.source)
 
 
-def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None) -> Graph:
+def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None, wanted=None) -> Graph:
     """A reduction whose outputs are too few to fill the chip is rewritten as
 
         out[D] op= f(D, R)      ->      out__part[S, D] op= f(D, S * chunk + Rc)   (S * chunk = extent of R)
@@ -264,7 +264,12 @@ def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None) ->
     sequential to two-level, as it already does inside a wavefront.
 
     `env` gives the values of named dimensions for one call; the result is then valid for those values only (the
-    slices must tile the axis exactly) and the caller keeps it per shape."""
+    slices must tile the axis exactly) and the caller keeps it per shape.
+
+    `wanted(statement, value)` may name a slice count for a statement that the rule above would leave alone (value(d)
+    is the extent of dimension d in this call): the lowering asks for one when a contraction has too few output tiles
+    to fill the chip.  Such a statement keeps its outputs' order in memory - the slices become the leading dimension
+    of `out__part` - so that it is still a contraction with a batch axis in front."""
     from .nodes import Expr as E
     env = env or {}
 
@@ -289,6 +294,7 @@ def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None) ->
         inner = 1
         for _, d in axes[1:]:
             inner *= value(d)
+        asked = wanted(st, value) if wanted is not None else None
         # which axis walks memory in the biggest operand decides how the lowering maps outputs to lanes
         raxes, daxes, score = {a for a, _ in axes}, {a for a, _ in st.data_axes}, 0
         for n in walk(st.root):
@@ -296,10 +302,10 @@ def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None) ->
                 names = {m.name for m in walk(n.args[-1]) if m.kind == 'axis'}
                 score += len(n.args) if names & raxes else (-len(n.args) if names & daxes else 0)
         want_outputs, min_chunk = (16384, 256) if score >= 0 else (262144, 16)
-        if outputs * 2 > want_outputs or extent * inner < 4 * min_chunk:
+        if asked is None and (outputs * 2 > want_outputs or extent * inner < 4 * min_chunk):
             out.append(st)
             continue
-        target = max(2, min(want_outputs // max(outputs, 1), extent * inner // min_chunk, extent))
+        target = asked if asked is not None else max(2, min(want_outputs // max(outputs, 1), extent * inner // min_chunk, extent))
         S = _divisor_near(extent, target)
         if S < 2 or S > extent or (S == extent and inner == 1):     # a slice per value of the axis: only when other reduce axes remain
             out.append(st)
@@ -315,12 +321,16 @@ def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None) ->
         part = st.output + '__part'
         while part in tensors:
             part += '_'
-        # the slices of one output lie next to each other, so the second statement reduces along memory
-        tensors[part] = TensorInfo(dtype=st.root.dtype, shape=list(st.out_shape) + [S])
-        s1 = replace(st, output=part, out_index=tuple(st.out_index) + (E('axis', 'int32', name=s_ax),), root=root1,
+        s_idx = E('axis', 'int32', name=s_ax)
+        if asked is not None:       # slices in front: statement 1 stays a contraction, statement 2 sums whole planes
+            p_index, p_shape = (s_idx,) + tuple(st.out_index), [S] + list(st.out_shape)
+        else:                       # the slices of one output lie next to each other: statement 2 reduces along memory
+            p_index, p_shape = tuple(st.out_index) + (s_idx,), list(st.out_shape) + [S]
+        tensors[part] = TensorInfo(dtype=st.root.dtype, shape=p_shape)
+        s1 = replace(st, output=part, out_index=p_index, root=root1,
                      data_axes=[(s_ax, S)] + list(st.data_axes), reduce_axes=[(c_ax, chunk)] + list(axes[1:]),
-                     out_dtype=st.root.dtype, out_shape=list(st.out_shape) + [S])
-        load = E('load', st.root.dtype, name=part, args=tuple(st.out_index) + (E('axis', 'int32', name=s_ax),))
+                     out_dtype=st.root.dtype, out_shape=p_shape)
+        load = E('load', st.root.dtype, name=part, args=p_index)
         s2 = replace(st, root=load, reduce_axes=[(s_ax, S)], reads=[part])
         out += [s1, s2]
         changed = True

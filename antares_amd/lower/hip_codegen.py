@@ -269,7 +269,13 @@ class KernelPlan:
         v = ''
         if 'matrixv' in self.variants and pointers is not None and K % self.matrix['vec_width'][0] == 0 and \
                 all(pointers[t] % 16 == 0 for t in self.matrix['vec_tensors']):
-            v = 'v'
+            def whole(dims_):
+                n = 1
+                for d in dims_:
+                    n *= d if isinstance(d, int) else env[d]
+                return n % self.matrix['vec_width'][0] == 0
+            if all(whole(p) for p in self.matrix.get('vec_pitch', [])):
+                v = 'v'
         # ... and when the big tiles are not mostly padding: 64 columns in tiles of 128 multiply twice what they need,
         # which costs more than the small tiles' lower rate (about three quarters of the big ones')
         if big >= 192 and big <= MAX_GRID * 64 and ('matrix64' not in self.variants or small >= 3 * big):
@@ -843,6 +849,7 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
                 wide = [ITEMSIZE[tensors[mc['l' + t].name].dtype] for t in ('a', 'b') if mc['vec'][t]]
                 plan.matrix['vec_tensors'] = [mc['l' + t].name for t in ('a', 'b') if mc['vec'][t]]
                 plan.matrix['vec_width'] = [16 // min(wide)]
+                plan.matrix['vec_pitch'] = [mc['pitch'][t] for t in ('a', 'b') if mc['vec'][t]]     # row lengths, as dimensions to multiply
 
     return '\n\n'.join(src), plan
 
@@ -1272,16 +1279,59 @@ def _matrix_contraction(st, tensors):
     # an operand whose last indices are THE reduce axes, bare and in their order, over dimensions of exactly their
     # extents (`input1[F, C, KH, KW]` of a convolution; the `[N, K]` of a product), lies in memory as rows of k:
     # 16-byte vectors of k can be fetched when k is a multiple of the vector and the tensor is aligned
-    vec = {}
+    # The first of them may be one slice of a longer axis, `S * chunk + Kc` with the slice S a batch axis and chunk the
+    # extent of Kc (what slicing a contraction leaves): a row of the slice is still a run of k, starting a whole number
+    # of slices into a row of the tensor.  `pitch` is the row length of the tensor, which must be whole vectors too.
+    vec, pitch = {}, {}
     red = dict(st.reduce_axes)
+
+    def bare_or_slice(ix, k):
+        if ix.kind == 'axis':
+            return ix.name == k
+        if ix.kind == 'op' and ix.name == '+' and len(ix.args) == 2:
+            sl, ax = ix.args
+            return (ax.kind == 'axis' and ax.name == k and sl.kind == 'op' and sl.name == '*' and len(sl.args) == 2 and
+                    sl.args[0].kind == 'axis' and sl.args[0].name in batch and sl.args[1].kind == 'const' and sl.args[1].value == red[k])
+        return False
     for tag, ld in (('a', la), ('b', lb)):
         nk = len(k_axes)
         tail = ld.args[-nk:] if len(ld.args) >= nk else []
-        vec[tag] = (len(tail) == nk and all(ix.kind == 'axis' and ix.name == k for ix, k in zip(tail, k_axes)) and
+        vec[tag] = (len(tail) == nk and bare_or_slice(tail[0], k_axes[0]) and
+                    all(ix.kind == 'axis' and ix.name == k for ix, k in zip(tail[1:], k_axes[1:])) and
                     not any(set(k_axes) & _axes_of(a) for a in ld.args[:-nk]) and
-                    all(d == red[k] for d, k in zip(tensors[ld.name].shape[-nk:], k_axes)) and not guards[tag])
+                    all(d == red[k] for d, k in zip(tensors[ld.name].shape[-nk + 1:] if nk > 1 else [], k_axes[1:])) and
+                    (tail[0].kind != 'axis' or tensors[ld.name].shape[-nk] == red[k_axes[0]]) and not guards[tag])
+        pitch[tag] = list(tensors[ld.name].shape[-nk:])
     return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts, 'vec': vec,
-            'guards': guards}
+            'guards': guards, 'pitch': pitch}
+
+
+def contraction_slices(tensors):
+    """-> wanted(statement, value) for split_wide_reductions: how many slices of k a contraction on the matrix
+    instructions should be cut into, or None.  Blocks of 64 x 64 outputs that number fewer than two per compute unit
+    leave a wavefront alone on its SIMD with nothing to hide its loads behind; with at least 1024 values of k the
+    product is cut into up to 8 slices (each at least 256 long) that run as a batch and are summed by a second
+    statement - 16 bytes more traffic per output and slice, against a main loop that fills the chip."""
+    def wanted(st, value):
+        if '__part' in st.output:
+            return None
+        mc = _matrix_contraction(st, tensors)
+        if mc is None:
+            return None
+        ext = dict(st.data_axes + st.reduce_axes)
+
+        def prod(names):
+            n = 1
+            for a in names:
+                n *= value(ext[a])
+            return n
+        M, N, B, K = prod(mc['m']), prod(mc['n']), prod(mc['batch']), prod(mc['k'])
+        blocks = ((M + 63) // 64) * ((N + 63) // 64) * B
+        if M < 32 or N < 32 or blocks < 16 or blocks >= 512 or K < 1024:
+            return None
+        slices = min(8, K // 256, (1024 + blocks - 1) // blocks)
+        return slices if slices >= 2 else None
+    return wanted
 
 
 def _row_group_at(graph, i: int) -> int:

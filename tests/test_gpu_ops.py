@@ -788,6 +788,41 @@ def test_fp16_contractions_sum_in_float32_on_the_matrix_instructions(autort, ir,
         assert np.abs(got - exact).max() <= drift and np.abs(got - want).max() <= 2 * drift + 1e-3, (tag, drift)
 
 
+@pytest.mark.parametrize('ir,inputs,shapes,vectors', [
+    ('output0[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[F, C, KH, KW] where HO in 7, WO in 7',
+     ['input0=float32[N:4, C:512, H:9, W:9]', 'input1=float32[F:256, C:512, KH:3, KW:3]'], [(4, 512, 9, 9), (256, 512, 3, 3)], True),
+    ('output0[N, M] +=! input0[N, K] * input1[M, K]', ['input0=float32[N:320, K:4096]', 'input1=float32[M:512, K:4096]'], [(320, 4096), (512, 4096)], True),
+    ('output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]', ['input0=float32[B:2, N:256, K:2048]', 'input1=float32[B:2, K:2048, M:200]'],
+     [(2, 256, 2048), (2, 2048, 200)], True),
+    ('output0[N, M] +=! input0[N, K].to(`float32`) * input1[M, K].to(`float32`)', ['input0=float16[1024, 2048]', 'input1=float16[512, 2048]'],
+     [(1024, 2048), (512, 2048)], True),
+])
+def test_contractions_with_few_output_tiles_are_cut_into_slices_of_k(autort, ir, inputs, shapes, vectors):
+    """A contraction whose 64 x 64 output tiles number fewer than two per compute unit, over at least 1024 values of k,
+    runs as a batch of slices of k on the matrix instructions plus a sum over the slices; an operand that lies as rows
+    of k keeps its 16-byte fetches inside a slice.  Results against the oracle, to the rounding of a float32 sum in
+    another order."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'sliced contraction {ir[:60]} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='sliced_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    op.fast_path = None
+    env = dims_of(inputs, shapes)
+    plans = op.plans_for(env)
+    assert len(plans) == 2 and plans[0].matrix is not None and plans[1].matrix is None
+    sym, blocks, _ = plans[0].choose(env, {n: 0 for n in plans[0].args})
+    assert blocks >= 512 or plans[0].matrix['batch'][0] == 8          # the slices fill the chip, or there are 8 of them
+    assert sym in [v for t, v in plans[0].variants.items() if t.startswith('matrix') and t.endswith('v') == vectors]
+    g = torch.Generator().manual_seed(len(ir))
+    tensors = [torch.randn(shape, generator=g).to(torch.float16 if 'float16' in spec else torch.float32) for spec, shape in zip(inputs, shapes)]
+    names = [spec.split('=')[0] for spec in inputs]
+    want = CpuModule(parse_program(ir, inputs), fast_math=False)(**{n: t.numpy() for n, t in zip(names, tensors)})['output0']
+    K = int(np.prod([e if isinstance(e, int) else env[e] for _, e in parse_program(ir, inputs).statements[0].reduce_axes]))
+    got = op(*[t.to(dev) for t in tensors]).cpu().numpy()
+    assert got.shape == want.shape and np.allclose(got, want, rtol=1e-4, atol=2e-5 * K ** 0.5 * 4), np.abs(got - want).max()
+
+
 ROW_GROUP_CASES = [
     # program, inputs, shapes, does the row kernel run at these extents
     ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '

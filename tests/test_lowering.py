@@ -153,3 +153,41 @@ def test_graph_rewrites_for_one_call_keep_the_program_on_the_oracle():
     assert np.array_equal(CpuModule(baked, fast_math=False)(input0=a, input1=w)['output0'], CpuModule(g, fast_math=False)(input0=a, input1=w)['output0'])
     src, plans = hip_codegen.lower_graph(baked)
     assert 'const int __ext_KH = 3;' in src and 'int __dim_KH' in src
+
+
+def test_contractions_with_few_tiles_are_sliced_along_k_and_keep_their_vector_fetches():
+    """512 x 512 outputs are 64 tiles of 64 x 64: over 8192 values of k the contraction is cut into 8 slices that run as
+    a batch (slices in front, so the statement is still a contraction) and a sum over the slices; each operand is rows
+    of k inside a slice too.  Enough tiles, or a short k, and nothing is cut."""
+    import numpy as np
+    from antares_amd.ir.graph import split_wide_reductions
+    from antares_amd.lower import contraction_slices
+    from oracle.cpu_backend import CpuModule
+    ir, inputs = 'output0[N, M] +=! input0[N, K] * input1[M, K]', ['input0=float32[N:512, K:8192]', 'input1=float32[M:512, K:8192]']
+    g = fuse_elementwise(parse_program(ir, inputs))
+    env = {'N': 512, 'M': 512, 'K': 8192}
+    cut = split_wide_reductions(g, env, wanted=contraction_slices(g.tensors))
+    assert len(cut.statements) == 2
+    s1, s2 = cut.statements
+    assert s1.data_axes[0] == ('KS', 8) and s1.reduce_axes == [('KC', 1024)] and cut.tensors[s1.output].shape == [8, 'N', 'M']
+    assert [a for a, _ in s2.reduce_axes] == ['KS'] and s2.output == 'output0'
+    assert split_wide_reductions(cut, env, wanted=contraction_slices(cut.tensors)) is cut          # not cut twice
+    mc = hip_codegen._matrix_contraction(s1, cut.tensors)
+    assert mc['batch'] == ['KS'] and mc['vec'] == {'a': True, 'b': True} and mc['pitch'] == {'a': ['K'], 'b': ['K']}
+    src, plans = hip_codegen.lower_graph(cut)
+    zero = {n: 0 for n in plans[0].args}
+    assert plans[0]._matrix_choice(env, zero) == ('matrix64v', 512)
+    # a row of the tensor that is no whole number of vectors: element-wise fetches (never the case for a sliced K, but the
+    # launcher checks what it is given)
+    plans[0].matrix['vec_pitch'] = [[8190], ['K']]
+    assert plans[0]._matrix_choice(env, zero) == ('matrix64', 512)
+    for e in ({'N': 2048, 'M': 2048, 'K': 8192}, {'N': 512, 'M': 512, 'K': 512}, {'N': 16, 'M': 4096, 'K': 8192}):
+        assert split_wide_reductions(g, e, wanted=contraction_slices(g.tensors)) is g
+    # the two-statement form computes the same thing
+    small = fuse_elementwise(parse_program(ir, ['input0=float32[N:64, K:2048]', 'input1=float32[M:64, K:2048]']))
+    cut = split_wide_reductions(small, {'N': 64, 'M': 64, 'K': 2048}, wanted=lambda st, value: None if '__part' in st.output else 4)
+    assert len(cut.statements) == 2
+    rng = np.random.default_rng(3)
+    a, b = rng.standard_normal((64, 2048)).astype(np.float32), rng.standard_normal((64, 2048)).astype(np.float32)
+    got = CpuModule(cut, fast_math=False)(input0=a, input1=b)['output0']
+    assert np.allclose(got, a.astype(np.float64) @ b.astype(np.float64).T, rtol=1e-5, atol=1e-3)
