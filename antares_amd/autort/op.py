@@ -243,6 +243,7 @@ class ExportedOp:
                 sym, grid, block = plan.variants[saved['variant']], int(saved['grid']), 256
             else:
                 sym, grid, block = plan.choose(env, ptrs)
+            skip = plan.covers - 1         # a map applied at this reduction's stores
             if grid == 0:
                 continue
             capi.launch(module.function(sym), (grid, 1, 1), (block, 1, 1), stream,

@@ -39,7 +39,12 @@ def emit_evaluator_module(graph, dims: Optional[Dict[str, int]] = None, prefix: 
     head += '// CONFIG: \n// COMPUTE_V1: - einstein_v2(' + repr(' '.join(graph.source.split())) + ')\n'
     out = [head + PRELUDE]
     assert len(pieces) == len(plans) + 1
+    skip = 0
     for plan, piece in zip(plans, pieces[1:]):
+        if skip:                    # a map that the kernels of the reduction before it apply at their stores
+            skip -= 1
+            continue
+        skip = plan.covers - 1
         symbol, grid, block = plan.choose(env, {n: 0 for n in plan.args})      # evaluator buffers are 256-byte aligned
         code = piece.split('\n', 1)[1]                                          # drop lower_graph's own LOCAL line
         ins = ', '.join(disp(n) for n in plan.args[:-1])

@@ -207,6 +207,7 @@ class KernelPlan:
     tile_tensors: List[str] = field(default_factory=list)   # tensors that must be 16-byte aligned for the vector form of it
     row_group: Optional[RowGroup] = None          # set on the first statement of a run that one row kernel can compute
     matrix: Optional[Dict[str, List[object]]] = None   # matrix-instruction variant: extents of its row, column, batch and k axes (and what its vector form needs)
+    covers: int = 1                # statements these kernels compute: 2 when the map behind a reduction is applied at its store
 
     def _tiles(self, env: Dict[str, int]) -> int:
         """64 x 64 tiles of the transposing variant, 0 when it does not apply or an axis is too short to pay."""
@@ -501,11 +502,17 @@ def _is_flat_map(st, tensors) -> bool:
     return all_axes == loads_axes or len(axes) == 1
 
 
-def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
+def lower_statement(st, graph, name: str, tail=None) -> Tuple[str, KernelPlan]:
+    """Kernels of one statement.  `tail`: the map statement behind a reduction that is applied to each result where it
+    is stored (the reference's tail fusion, AntaresIR.md:248-250: `conv_out +=! ...; output0 = f(conv_out, bias)` is
+    one kernel); the reduction's own output is then never written."""
     tensors, dims = graph.tensors, graph.dim_names
     reads = [r for r in st.reads]
     args = sorted(set(reads) - {st.output}) + [st.output]
     written = [st.output]
+    if tail is not None:
+        args = sorted((set(reads) | set(tail.reads)) - {st.output, tail.output}) + [tail.output]
+        written = [tail.output]
 
     def one_touch(n: Expr) -> Optional[str]:
         """A load that reads every element of its tensor exactly once in the whole program - indexed by all axes of
@@ -530,7 +537,7 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
     variants: Dict[str, str] = {}
     plan = KernelPlan(name=name, args=args, dims=dims, variants=variants,
                       kind='scatter' if st.scatter else ('reduce' if st.reduce_axes else 'map'),
-                      output=st.output, data_axes=list(st.data_axes), reduce_axes=list(st.reduce_axes))
+                      output=written[0], data_axes=list(st.data_axes), reduce_axes=list(st.reduce_axes), covers=2 if tail is not None else 1)
 
     def header(sym):
         return [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st) + \
@@ -737,8 +744,18 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
         ident = reduce_identity(st.reduce, root.dtype)
         op = _REDUCE_OP[st.reduce] + '()'
         red_total = ' * '.join(f'(long long)__ext_{ax}' for ax, _ in st.reduce_axes)
-        store = f'{dst} = ({oct_})__acc;'
-        store = f'if ({cond}) {{ {store} }}' if cond else store
+        def result_store(acc):         # C text that stores one result held in `acc`
+            if tail is None:
+                text = f'{dst} = ({oct_}){acc};'
+                return f'if ({cond}) {{ {text} }}' if cond else text
+            # the tail sees the result as the reduction's output would hold it (rounded to its type)
+            tem = ExprEmitter(tensors, load_override=lambda n: '__t' if n.name == st.output else None)
+            troot, tcond = _root_and_cond(tail, tem)
+            tdst = f'{tail.output}[{plain.offset(tail.output, [plain.expr(i) for i in tail.out_index])}]'
+            text = f'{tdst} = ({HIP_TYPE[tail.out_dtype]})({tem.expr(troot)});'
+            text = f'if ({tcond}) {{ {text} }}' if tcond else text
+            return f'{{ const {oct_} __t = ({oct_}){acc}; (void)__t; {text} }}'
+        store = result_store('__acc')
 
         def reduce_body(sym, out_var, out_step, lane, nlanes, finish):
             b = header(sym)
@@ -829,13 +846,14 @@ def lower_statement(st, graph, name: str) -> Tuple[str, KernelPlan]:
             b.append(f'      for (int __j = 0; __j < {TY}; ++__j) {{')
             b.append(f'        const int {xa} = __x0 + __i, {ya} = __y0 + __j; (void){xa}; (void){ya};')
             b.append(f'        const {act} __acc_ = __acc[__i][__j];')
-            pstore = f'{dst} = ({oct_})__acc_;'
-            b.append(f'        if ({cond}) {{ {pstore} }}' if cond else f'        {pstore}')
+            b.append('        ' + result_store('__acc_'))
             b += ['      }', '    }', '  }', '}']
             src.append('\n'.join(b))
             variants['patch'] = sym
             plan.patch, plan.patch_dims = (TX, TY), [ext[xa], ext[ya]]
         mc = _matrix_contraction(st, tensors)
+        if mc is not None and tail is not None:
+            mc['tail'] = (tail, _matrix_tail(st, tail, mc, tensors))      # lower_graph fuses only what these kernels can take
         if mc is not None:
             src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_m', mc))
             src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_m64', mc, TS=64))
@@ -923,18 +941,32 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
                 out.append(f'{indent}const int {a} = (int)(__q % (unsigned int)__ext_{a}); __q /= (unsigned int)__ext_{a}; (void){a};')
         return out
     out_axes = [a for a, _ in st.data_axes]
-    rows_of_out = plain.offset(st.output, [a if (a in mc['m'] or a in mc['batch']) else '0' for a in out_axes])
-    cols_of_out = plain.offset(st.output, [a if a in mc['n'] else '0' for a in out_axes])
+    # With a tail (the map statement behind the reduction, applied where a result is stored) the stores go to the tail's
+    # output, which is indexed by the same axes in the same order; every other tensor the tail reads is addressed as
+    # (row part) + (column part) through two more tables per load.
+    tail, extra = mc.get('tail') or (None, [])
+    out_name = st.output if tail is None else tail.output
+    rows_of_out = plain.offset(out_name, [a if (a in mc['m'] or a in mc['batch']) else '0' for a in out_axes])
+    cols_of_out = plain.offset(out_name, [a if a in mc['n'] else '0' for a in out_axes])
     val_a = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__ra[__S][{j}]').expr(mc['fa']) for j in range(PER)]
     val_b = [ExprEmitter(tensors, load_override=lambda n, j=j: f'__rb[__S][{j}]').expr(mc['fb']) for j in range(PER)]
     if HM:
         val_a, val_b = [f'__ra[__S][{j}]' for j in range(PER)], [f'__rb[__S][{j}]' for j in range(PER)]
+    def stored(acc):                # C text that stores the result held in `acc` at (row __r, column __c) of the tile
+        if tail is None:
+            return f'{st.output}[__cm[__r] + __cn[__c]] = ({oct_}){acc};'
+        where = {i: f'{ld.name}[__xm{q}[__r] + __xn{q}[__c]]' for q, (ld, _, _, ids) in enumerate(extra) for i in ids}
+        tem = ExprEmitter(tensors, load_override=lambda n: '__t' if n.name == st.output else where[id(n)])
+        return (f'{{ const {oct_} __t = ({oct_}){acc}; (void)__t; '
+                f'{tail.output}[__cm[__r] + __cn[__c]] = ({HIP_TYPE[tail.out_dtype]})({tem.expr(tail.root)}); }}')
     b = [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st)
     b += ['  typedef float __f16v __attribute__((ext_vector_type(16)));',
           f'  typedef {ET} __f4 __attribute__((ext_vector_type({VW})));      // 16 bytes of a staged tile',
           f'  __shared__ __attribute__((aligned(16))) {ET} __As[2][{TS} * {LD}];     // [row][k], {BK} k and 16 bytes of padding per row',
           f'  __shared__ __attribute__((aligned(16))) {ET} __Bs[2][{TS} * {LD}];     // [column][k]',
           f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][{BK}], __bk[2][{BK}];'] + \
+         [f'  __shared__ long long __xm{q}[{TS}], __xn{q}[{TS}];      // row and column part of the offsets into {ld.name} (read by the tail)'
+          for q, (ld, _, _, _) in enumerate(extra)] + \
          [f'  __shared__ int __gm{x}[{len(GV[x])}][{TS}], __gk{x}[2][{BK}][{len(GV[x])}];      // the guards of operand {x}: row part and k part of each compared value'
           for x in 'ab' if G[x]] + [
           f'  const long long __M = {prod(mc["m"])}, __N = {prod(mc["n"])}, __B = {prod(mc["batch"])};',
@@ -949,12 +981,14 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           f'      long long __row = __tm * {TS} + __tid;',
           '      if (__row >= __M) __row = __M - 1;']
     b += decompose('__row', mc['m'], '      ')
+    b += [f'      __xm{q}[__tid] = {rowpart};' for q, (_, rowpart, _, _) in enumerate(extra)]
     b += [f'      __gma[{c}][__tid] = {g[0]};' for c, g in enumerate(GV['a'])]
     b += [f'      __am[__tid] = {mc["parts"]["a"][0]};', f'      __cm[__tid] = {rows_of_out};',
           f'    }} else if (__tid < {2 * TS}) {{                  // column offsets of the second operand and of the output',
           f'      long long __colq = __tn * {TS} + (__tid - {TS});',
           '      if (__colq >= __N) __colq = __N - 1;']
     b += decompose('__colq', mc['n'], '      ')
+    b += [f'      __xn{q}[__tid - {TS}] = {colpart};' for q, (_, _, colpart, _) in enumerate(extra)]
     b += [f'      __gmb[{c}][__tid - {TS}] = {g[0]};' for c, g in enumerate(GV['b'])]
     b += [f'      __bn[__tid - {TS}] = {mc["parts"]["b"][0]};', f'      __cn[__tid - {TS}] = {cols_of_out};',
           '    }',
@@ -1112,7 +1146,7 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           '        #pragma unroll',
           '        for (int __e = 0; __e < 16; ++__e) {',
           f'          const int __r = __wm * {HALF} + __i * 32 + (__e >> 2) * 8 + (__lane >> 5) * 4 + (__e & 3);',
-          f'          if (__tm * {TS} + __r < __M && __tn * {TS} + __c < __N) {st.output}[__cm[__r] + __cn[__c]] = ({oct_})__acc[__i][__j][__e];',
+          f'          if (__tm * {TS} + __r < __M && __tn * {TS} + __c < __N) {stored("__acc[__i][__j][__e]")}',
           '        }',
           '      }',
           '    __syncthreads();                               // the tables and buffers are rewritten by the next tile',
@@ -1304,6 +1338,69 @@ def _matrix_contraction(st, tensors):
         pitch[tag] = list(tensors[ld.name].shape[-nk:])
     return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts, 'vec': vec,
             'guards': guards, 'pitch': pitch}
+
+
+def _tail_of(graph, i: int):
+    """The statement behind statement i when it is a map that can be applied where the reduction i stores its results
+    (AntaresIR.md:248-250, tail fusion), else None: same data axes, both outputs indexed by them bare and in order, the
+    reduction's output read at that very position, by this map only, and not wanted by the caller."""
+    if i + 1 >= len(graph.statements):
+        return None
+    st, nx = graph.statements[i], graph.statements[i + 1]
+    if not st.reduce_axes or st.scatter or nx.reduce_axes or nx.scatter or nx.set_op:
+        return None
+    if (st.root.kind == 'when' and len(st.root.args) == 1) or list(st.data_axes) != list(nx.data_axes) or not st.data_axes:
+        return None
+    axes = [a for a, _ in st.data_axes]
+
+    def bare(index):
+        return [x.name if x.kind == 'axis' else None for x in index] == axes
+    t = st.output
+    if not bare(st.out_index) or not bare(nx.out_index) or t in graph.outputs or t in graph.declared or nx.output == t:
+        return None
+    if any(t in s_.reads or s_.output in (t, nx.output) for k, s_ in enumerate(graph.statements) if k not in (i, i + 1)):
+        return None
+    if nx.output in nx.reads or nx.output in st.reads or t in st.reads:
+        return None
+    loads = [n for n in walk(nx.root) if n.kind == 'load' and n.name == t]
+    if not loads or any(not bare(n.args) for n in loads):
+        return None
+    mc = _matrix_contraction(st, graph.tensors)
+    if mc is not None and _matrix_tail(st, nx, mc, graph.tensors) is None:
+        return None                 # the matrix kernels could not take it: two launches beat losing them
+    return nx
+
+
+def _matrix_tail(st, tail, mc, tensors):
+    """What the matrix kernels need to apply `tail` at their stores: [(load, row part, column part)] for every load of
+    another tensor than the reduction's output - its offset must be a sum of a part made of row (and batch) axes and a
+    part made of column axes, like the output's own - or None when the tail cannot be applied there (a conditional
+    store, an axis used as a value, an index that mixes rows and columns, more than four such loads)."""
+    if tail.root.kind == 'when' and len(tail.root.args) == 1:
+        return None
+    plain = ExprEmitter(tensors)
+    loads = [n for n in walk(tail.root) if n.kind == 'load' and n.name != st.output]
+    inside = sum(1 for n in walk(tail.root) if n.kind == 'load' for a in n.args for m in walk(a) if m.kind == 'axis')
+    if sum(1 for m in walk(tail.root) if m.kind == 'axis') != inside:
+        return None
+    if any(m.kind == 'load' for n in loads for a in n.args for m in walk(a)):
+        return None                 # a gathered index would be counted as a load of its own
+    rows, cols = set(mc['m']) | set(mc['batch']), set(mc['n'])
+    out, seen = [], {}
+    for ld in loads:
+        sp = [_split_index(ix, plain, rows, cols) for ix in ld.args]
+        if any(x is None for x in sp):
+            return None
+        entry = (ld, plain.offset(ld.name, [x[0] or '0' for x in sp]), plain.offset(ld.name, [x[1] or '0' for x in sp]))
+        key = (ld.name,) + entry[1:]
+        if key in seen:             # the same element read twice (`x.when(x > 0, 0)`): one pair of tables
+            seen[key].append(id(ld))
+            continue
+        seen[key] = [id(ld)]
+        out.append(entry + (seen[key],))
+    if len(out) > 4:
+        return None
+    return out
 
 
 def contraction_slices(tensors):
@@ -1569,8 +1666,11 @@ def lower_graph(graph, prefix: str = 'autort') -> Tuple[str, List[KernelPlan]]:
     parts, plans = [head + PRELUDE], []
     grouped_until = 0
     for i, st in enumerate(graph.statements):
-        code, plan = lower_statement(st, graph, f'{prefix}_k{i}')
         count = _row_group_at(graph, i) if i >= grouped_until else 0
+        # a map behind a reduction is applied at the reduction's stores (its own kernels stay in the text and are not
+        # launched); not where a row kernel may take the reduction
+        tail = _tail_of(graph, i) if not count and i >= grouped_until else None
+        code, plan = lower_statement(st, graph, f'{prefix}_k{i}', tail=tail)
         if count:
             # the row kernel travels with the first statement's kernels; the per-statement kernels stay for the
             # extents it is not launched at

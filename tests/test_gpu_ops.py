@@ -823,6 +823,59 @@ def test_contractions_with_few_output_tiles_are_cut_into_slices_of_k(autort, ir,
     assert got.shape == want.shape and np.allclose(got, want, rtol=1e-4, atol=2e-5 * K ** 0.5 * 4), np.abs(got - want).max()
 
 
+TAIL_CASES = [
+    # AntaresIR.md:248-250 (ConvBiasRelu tail fusion); a product with a scaled result, a per-column and a per-element
+    # term under a tanh; a float16 result of a float32 sum; a column-wise maximum with a conditional store behind it
+    ('conv_out[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[KH, KW, C, F] where HO in 30, WO in 30; '
+     'conv_bias[N, F, HO, WO] = conv_out[N, F, HO, WO] + input2[0, 0, 0, F]; '
+     'output0[N, F, HO, WO] = conv_bias[N, F, HO, WO].when(conv_bias[N, F, HO, WO] > 0.0, 0.0)',
+     ['input0=float32[N:4, C:16, H:32, W:32]', 'input1=float32[KH:3, KW:3, C:16, F:64]', 'input2=float32[1, 1, 1, F:64]'],
+     [(4, 16, 32, 32), (3, 3, 16, 64), (1, 1, 1, 64)], True),
+    ('acc[N, M] +=! input0[N, K] * input1[M, K]; output0[N, M] = (acc[N, M] * 0.5 + input2[M] + input3[N, M]).call(`tanh`)',
+     ['input0=float32[N:300, K:256]', 'input1=float32[M:200, K:256]', 'input2=float32[M:200]', 'input3=float32[N:300, M:200]'],
+     [(300, 256), (200, 256), (200,), (300, 200)], True),
+    ('acc[B, N, M] +=! input0[B, N, K].to(`float32`) * input1[B, K, M].to(`float32`); output0[B, N, M] = (acc[B, N, M] + input2[B, M]).to(`float16`)',
+     ['input0=float16[B:3, N:128, K:64]', 'input1=float16[B:3, K:64, M:160]', 'input2=float32[B:3, M:160]'], [(3, 128, 64), (3, 64, 160), (3, 160)], True),
+    ('top[C] >=! input0[N, C]; output0[C] = top[C].when(top[C] > input1[C])', ['input0=float32[N:40, C:20000]', 'input1=float32[C:20000]', 'output0=float32[C:20000]'],
+     [(40, 20000), (20000,), (20000,)], False),
+]
+
+
+@pytest.mark.parametrize('ir,inputs,shapes,matrix', TAIL_CASES)
+def test_a_map_behind_a_reduction_is_applied_at_its_stores(autort, ir, inputs, shapes, matrix):
+    """Tail fusion (AntaresIR.md:248-250): the kernels of the reduction store f(result, other tensors) straight into the
+    map's output; the reduction's own output is never written and the map's kernels are not launched.  Every variant of
+    the fused kernels against the oracle, which runs the statements one by one."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'tail fusion {ir[:60]} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='tail_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    op.fast_path = None
+    env = dims_of(inputs, shapes)
+    plans = op.plans_for(env)
+    assert len(plans) == 2 and plans[0].covers == 2 and plans[0].output == 'output0' and plans[0].args[-1] == 'output0'
+    assert not any(a in plans[0].args for a in ('acc', 'conv_out', 'top'))
+    assert ('matrix' in plans[0].variants) == matrix
+    g = torch.Generator().manual_seed(len(ir))
+    tensors = [(torch.randn(shape, generator=g) * 0.5).to(torch.float16 if 'float16' in spec else torch.float32) for spec, shape in zip(inputs, shapes)]
+    names = [spec.split('=')[0] for spec in inputs]
+    want = CpuModule(parse_program(ir, inputs), fast_math=False)(**{n: t.numpy().copy() for n, t in zip(names, tensors)})['output0'].astype(np.float32)
+    plan, total = plans[0], int(np.prod(want.shape))
+    launches = [('thread', (total + 255) // 256), ('wave', (total + 3) // 4), ('block', total)]
+    if 'patch' in plan.variants and plan._patches(env, total):
+        launches.append(('patch', (plan._patches(env, total) + 255) // 256))
+    if matrix:
+        M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
+        launches += [(tag, ((M + side - 1) // side) * ((N + side - 1) // side) * B) for tag, side in (('matrix', 128), ('matrix64', 64)) if tag in plan.variants]
+        launches += [(tag, ((M + side - 1) // side) * ((N + side - 1) // side) * B) for tag, side in (('matrixv', 128), ('matrix64v', 64)) if tag in plan.variants]
+    tol = 1e-2 if want.dtype == np.float16 or 'float16' in ir else 2e-4
+    for tag, grid in launches:
+        plan.choose = lambda env_, ptrs, tag=tag, grid=grid: (plan.variants[tag], min(grid, 65536), 256)
+        got = op(*[t.clone().to(dev) for t in tensors]).float().cpu().numpy()
+        assert got.shape == want.shape and np.allclose(got, want, rtol=tol, atol=tol), (tag, np.abs(got - want).max())
+
+
 ROW_GROUP_CASES = [
     # program, inputs, shapes, does the row kernel run at these extents
     ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
