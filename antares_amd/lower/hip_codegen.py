@@ -1277,6 +1277,12 @@ def _matrix_contraction(st, tensors):
     if sum(1 for m in walk(root) if m.kind == 'axis') != inside:
         return None
     ua, ub = set().union(*[_axes_of(a) for a in la.args]), set().union(*[_axes_of(a) for a in lb.args])
+    # The lanes of a wavefront hold neighbouring COLUMNS of the result: the factor that uses the output's last axis
+    # is made the second one (the product commutes exactly), so that stores run along memory - a convolution's
+    # `output0[N, F, HO, WO]` is then written along WO, not in pieces a feature map apart.
+    if axes[-1] in ua and axes[-1] not in ub:
+        fa, fb, la, lb, ua, ub = fb, fa, lb, la, ub, ua
+        guards = {'a': guards['b'], 'b': guards['a']}
     k_axes = [a for a, _ in st.reduce_axes]
     if not set(k_axes) <= ua or not set(k_axes) <= ub:
         return None

@@ -102,13 +102,15 @@ def test_a_padded_convolution_goes_to_the_matrix_kernels_with_its_guards_tabled(
     from antares_amd.autort.op import compile_cached
     graph = fuse_elementwise(parse_program(PADDED_CONV, ['input0=float32[N:8, C:64, H:56, W:56]', 'input1=float32[F:64, C:64, KH:3, KW:3]']))
     mc = hip_codegen._matrix_contraction(graph.statements[0], graph.tensors)
-    assert [g[2] for g in mc['guards']['a']] == ['<=', '<', '<=', '<'] and mc['guards']['b'] == []
-    assert len({(g[0], g[1]) for g in mc['guards']['a']}) == 2 and not mc['vec']['a']
+    # the image uses the output's last axis: it is made the second factor (columns), so that stores run along WO
+    assert mc['la'].name == 'input1' and mc['lb'].name == 'input0' and mc['n'] == ['N', 'HO', 'WO'] and mc['m'] == ['F']
+    assert [g[2] for g in mc['guards']['b']] == ['<=', '<', '<=', '<'] and mc['guards']['a'] == []
+    assert len({(g[0], g[1]) for g in mc['guards']['b']}) == 2 and not mc['vec']['b']
     src, plans = hip_codegen.lower_graph(graph)
     # the guarded image is fetched element by element; the weights lie as rows of k = (C, KH, KW): 16-byte vectors
-    assert mc['vec']['b'] and {'matrix', 'matrix64', 'matrixv', 'matrix64v'} <= set(plans[0].variants)
+    assert mc['vec']['a'] and {'matrix', 'matrix64', 'matrixv', 'matrix64v'} <= set(plans[0].variants)
     assert plans[0].matrix['vec_tensors'] == ['input1']
-    assert '__gma[2][128]' in src and '__gma[2][64]' in src
+    assert '__gmb[2][128]' in src and '__gmb[2][64]' in src
     # 25088 rows x 64 columns: tiles of 128 columns would be half padding, the small tiles take it
     env = {'N': 8, 'C': 64, 'H': 56, 'W': 56, 'F': 64, 'KH': 3, 'KW': 3}
     assert plans[0]._matrix_choice(env, {n: 0 for n in plans[0].args}) == ('matrix64v', 392)
