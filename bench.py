@@ -71,6 +71,8 @@ def parse_args():
                     help='run only the read-only launch over 32 distinct buffers of the headline weight size, and exit')
     ap.add_argument('--stream-floors', action='store_true',
                     help='run only the read-only, store-only and copy launches (what one launch needs to move bytes), and exit')
+    ap.add_argument('--lowering', action='store_true',
+                    help='run only the generic lowering on a set of programs (products, convolutions, reductions, rows, copies), one JSON line each, and exit')
     ap.add_argument('--phase-chain', action='store_true',
                     help='run only the probe of phases meeting inside one launch (a persistent kernel against dependent launches), and exit')
     return ap.parse_args()
@@ -151,6 +153,113 @@ def bench_stream_floors(torch, capi, steps, warmup, layers=16):
         out.append(row)
         del bufs, dsts
     return out
+
+
+def _conv(n, c, f, hw, dt='float32', pad=False):
+    cast = '.to(`float32`)' if dt == 'float16' else ''
+    if pad:
+        ir = (f'output0[N, F, HO, WO] +=! input0[N, C, HO + KH - 1, WO + KW - 1]{cast}.when([HO + KH - 1 >= 0, HO + KH - 1 < {hw}, '
+              f'WO + KW - 1 >= 0, WO + KW - 1 < {hw}], 0.0) * input1[F, C, KH, KW]{cast} where HO in {hw}, WO in {hw}')
+    else:
+        ir = f'output0[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW]{cast} * input1[F, C, KH, KW]{cast} where HO in {hw - 2}, WO in {hw - 2}'
+    ho = hw if pad else hw - 2
+    return (f'{"padded " if pad else ""}3x3 convolution {dt} {n}x{c}x{hw}x{hw} -> {f} channels', ir,
+            [f'input0={dt}[N:{n}, C:{c}, H:{hw}, W:{hw}]', f'input1={dt}[F:{f}, C:{c}, KH:3, KW:3]'], [(n, c, hw, hw), (f, c, 3, 3)],
+            ('flop', 2 * n * f * ho * ho * c * 9))
+
+
+# Programs of the reference's IR documentation (AntaresIR.md:108-256) and of common networks at sizes that fill the chip,
+# for the generic lowering: (name, program, inputs, shapes, ('flop', count) or ('bytes', count or None = inputs + output)).
+LOWERING_CASES = [
+    ('fp32 product 4096x4096x1024, A stored [K, N]', 'output0[N, M] +=! input0[K, N] * input1[K, M]',
+     ['input0=float32[K:1024, N:4096]', 'input1=float32[K:1024, M:4096]'], [(1024, 4096), (1024, 4096)], ('flop', 2 * 4096 * 4096 * 1024)),
+    ('fp16 A B^T into float32 4096x4096x1024', 'output0[N, M] +=! input0[N, K].to(`float32`) * input1[M, K].to(`float32`)',
+     ['input0=float16[N:4096, K:1024]', 'input1=float16[M:4096, K:1024]'], [(4096, 1024), (4096, 1024)], ('flop', 2 * 4096 * 4096 * 1024)),
+    ('fp16 product 2048^3 (float16 statement)', 'output0[N, M] +=! input0[N, K] * input1[K, M]',
+     ['input0=float16[N:2048, K:2048]', 'input1=float16[K:2048, M:2048]'], [(2048, 2048), (2048, 2048)], ('flop', 2 * 2048 ** 3)),
+    ('batched fp32 product 8 x 512^3', 'output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]',
+     ['input0=float32[B:8, N:512, K:512]', 'input1=float32[B:8, K:512, M:512]'], [(8, 512, 512), (8, 512, 512)], ('flop', 2 * 8 * 512 ** 3)),
+    ('fp32 A B^T 512x512x8192 (sliced along k)', 'output0[N, M] +=! input0[N, K] * input1[M, K]',
+     ['input0=float32[N:512, K:8192]', 'input1=float32[M:512, K:8192]'], [(512, 8192), (512, 8192)], ('flop', 2 * 512 * 512 * 8192)),
+    _conv(8, 64, 64, 56), _conv(32, 128, 128, 30), _conv(32, 128, 128, 28, pad=True), _conv(32, 128, 128, 28, 'float16'),
+    _conv(32, 128, 128, 28, 'float16', pad=True), _conv(8, 512, 512, 9),
+    ('depthwise 3x3 convolution 32x128x56x56', 'output0[N, C, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[C, KH, KW] where HO in 54, WO in 54',
+     ['input0=float32[N:32, C:128, H:56, W:56]', 'input1=float32[C:128, KH:3, KW:3]'], [(32, 128, 56, 56), (128, 3, 3)], ('bytes', None)),
+    ('2x2 max pooling 32x64x112x112', 'output0[N, C, HO, WO] >=! input0[N, C, HO * 2 + KH, WO * 2 + KW] where HO in 56, WO in 56, KH in 2, KW in 2',
+     ['input0=float32[N:32, C:64, H:112, W:112]'], [(32, 64, 112, 112)], ('bytes', None)),
+    ('channel sums of 32x256x56x56', 'output0[C] +=! input0[N, C, H, W]', ['input0=float32[N:32, C:256, H:56, W:56]'], [(32, 256, 56, 56)], ('bytes', None)),
+    ('column sums of 16384x4096', 'output0[C] +=! input0[N, C]', ['input0=float32[N:16384, C:4096]'], [(16384, 4096)], ('bytes', None)),
+    ('sum of 67108864 fp32', 'output0[] +=! input0[N]', ['input0=float32[N:67108864]'], [(67108864,)], ('bytes', None)),
+    ('softmax of 65536 rows of 1024 (AntaresIR.md:226)', 'temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
+     'output0[N, C] = (input0[N, C] - temp0[N]).call(`exp`) / temp1[N]', ['input0=float32[N:65536, C:1024]'], [(65536, 1024)], ('bytes', 65536 * 1024 * 8)),
+    ('layer normalisation of 4096 rows of 4096 (AntaresIR.md:232)', 'temp0[N] +=! input0[N, C]; temp1[N] +=! input0[N, C] * input0[N, C]; '
+     'output0[N, C] = (input0[N, C] * C.val() - temp0[N]) * (temp1[N] * C.val() - temp0[N] * temp0[N] + 1e-5).call(`rsqrt`)',
+     ['input0=float32[N:4096, C:4096]'], [(4096, 4096)], ('bytes', 4096 * 4096 * 8)),
+    ('fp32 transpose 4096x4096', 'output0[C, N] = input0[N, C]', ['input0=float32[N:4096, C:4096]'], [(4096, 4096)], ('bytes', None)),
+    ('fp16 NCHW -> NHWC 8x256x64x64', 'output0[N, H, W, C] = input0[N, C, H, W]', ['input0=float16[N:8, C:256, H:64, W:64]'], [(8, 256, 64, 64)], ('bytes', None)),
+    ('bias add over 32x256x56x56', 'output0[N, C, H, W] = input0[N, C, H, W] + input1[C]',
+     ['input0=float32[N:32, C:256, H:56, W:56]', 'input1=float32[C:256]'], [(32, 256, 56, 56), (256,)], ('bytes', None)),
+    ('gathered rows: 8192 of 32000 x 4096 fp16', 'output0[N, C] = input0[input1[N], C]',
+     ['input0=float16[V:32000, C:4096]', 'input1=int32[N:8192]'], [(32000, 4096), (8192,)], ('bytes', 8192 * 4096 * 2 * 2)),
+    ('convolution + bias + ReLU 32x128x30x30 -> 128 (AntaresIR.md:250, one launch)',
+     'conv_out[N, F, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[F, C, KH, KW] where HO in 28, WO in 28; '
+     'output0[N, F, HO, WO] = (conv_out[N, F, HO, WO] + input2[F]).call(`max`, [0.0])',
+     ['input0=float32[N:32, C:128, H:30, W:30]', 'input1=float32[F:128, C:128, KH:3, KW:3]', 'input2=float32[F:128]'],
+     [(32, 128, 30, 30), (128, 128, 3, 3), (128,)], ('flop', 2 * 32 * 128 * 28 * 28 * 128 * 9)),
+]
+
+
+def bench_lowering(torch, autort, capi, steps, warmup):
+    """The generic lowering on LOWERING_CASES: each program exported as a user would, the hand-written kernels switched
+    off, timed as a graph replay (eight calls on eight copies of the inputs) at the sustained clock; rate in TFLOP/s,
+    or in TB/s of the bytes a single pass over inputs and output moves."""
+    dev = autort.device()
+    out = []
+    for name, ir, inputs, shapes, (kind, count) in LOWERING_CASES:
+        op = autort.export(ir=ir, inputs=inputs, name='bench_lowering_' + ''.join(c for c in name if c.isalnum())[:40])
+        op.fast_path = None
+        g = torch.Generator('cpu').manual_seed(len(name))
+        ts = [torch.randint(0, 32000, shp, generator=g, dtype=torch.int32).to(dev) if 'int32' in spec else
+              torch.randn(shp, generator=g).to(torch.float16 if 'float16' in spec else torch.float32).to(dev) for spec, shp in zip(inputs, shapes)]
+        res = op(*ts)
+        # eight calls per replayed graph, each on its own copy of the inputs: a graph of one short kernel would time
+        # the replay itself (about 17 us), and the same tensors every time would be served by the caches
+        sets = [ts] + [[t.clone() for t in ts] for _ in range(7)]
+
+        def one_pass():
+            for tensors in sets:
+                op(*tensors)
+        sec = time_graph(torch, capi, one_pass, steps, warmup, warm_ms=20.0) / len(sets)
+        row = {'program': name, 'us': round(sec * 1e6, 1), 'launches': sum(1 for _ in _launched(op, inputs, shapes))}
+        if kind == 'flop':
+            row['tflops'] = round(count / sec / 1e12, 1)
+        else:
+            nbytes = count if count is not None else sum(t.numel() * t.element_size() for t in ts) + res.numel() * res.element_size()
+            row['tb_per_s'] = round(nbytes / sec / 1e12, 2)
+        out.append(row)
+        print(json.dumps(row), flush=True)
+        del ts, res, sets
+    return out
+
+
+def _launched(op, inputs, shapes):
+    """The plans a call with these shapes launches from (a plan that covers the statement behind it counts once)."""
+    env = {}
+    for spec, shape in zip(inputs, shapes):
+        for d, v in zip(spec.split('[', 1)[1].rstrip(']').split(','), shape):
+            if ':' in d:
+                env[d.split(':')[0].strip()] = v
+    skip = 0
+    for plan in op.plans_for(env):
+        if skip:
+            skip -= 1
+            continue
+        group = plan.row_group
+        if group is not None and group.choose(env, {n: 0 for n in group.args})[1]:
+            skip = group.count - 1
+        else:
+            skip = plan.covers - 1
+        yield plan
 
 
 def bench_phase_chain(torch, capi, phases=32, nbytes=2048 * 11008, runs=5):
@@ -481,6 +590,9 @@ def main():
         return
     if args.phase_chain:
         print(json.dumps(bench_phase_chain(torch, capi)), flush=True)
+        return
+    if args.lowering:
+        bench_lowering(torch, autort, capi, args.steps, args.warmup)
         return
     K, N, M = 4096, 11008, 1
     head = bench_gemv(torch, autort, capi, workloads, K, N, M, args.steps, args.warmup, args.seed)

@@ -193,3 +193,19 @@ def test_contractions_with_few_tiles_are_sliced_along_k_and_keep_their_vector_fe
     a, b = rng.standard_normal((64, 2048)).astype(np.float32), rng.standard_normal((64, 2048)).astype(np.float32)
     got = CpuModule(cut, fast_math=False)(input0=a, input1=b)['output0']
     assert np.allclose(got, a.astype(np.float64) @ b.astype(np.float64).T, rtol=1e-5, atol=1e-3)
+
+
+def test_the_programs_of_the_lowering_benchmark_lower_and_take_the_kernels_they_are_listed_for():
+    """`bench.py --lowering` times these programs on the GPU; here: each parses and lowers, the contractions have
+    matrix-instruction kernels, the two row programs are one row group each, and the fused tail is one launch."""
+    import bench
+    for name, ir, inputs, shapes, (kind, count) in bench.LOWERING_CASES:
+        graph = fuse_elementwise(parse_program(ir, inputs))
+        src, plans = hip_codegen.lower_graph(graph)
+        assert len(plans) == len(graph.statements) and src
+        if kind == 'flop':
+            assert 'matrix' in plans[0].variants, name
+        if 'AntaresIR.md:226' in name or 'AntaresIR.md:232' in name:
+            assert plans[0].row_group is not None and plans[0].row_group.count == 3, name
+        if 'one launch' in name:
+            assert plans[0].covers == 2, name
