@@ -18,7 +18,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..ir import Graph, bake_small_reduce_extents, fuse_elementwise, parse_program, split_wide_reductions
+from ..ir import Graph, bake_small_reduce_extents, fuse_elementwise, pad_guarded_factors, parse_program, split_wide_reductions
 from ..lower import contraction_slices, lower_graph
 from ..runtime import capi
 
@@ -84,7 +84,8 @@ class ExportedOp:
         self.fresh_outputs = [o for o in self.graph.outputs if o not in self.declared]
         # what the generic lowering compiles: wide reductions with few outputs become two statements (statically
         # sized ones here; programs with named dimensions get a variant per set of values at call time)
-        self.lowered: Graph = split_wide_reductions(self.fused, wanted=contraction_slices(self.fused.tensors))
+        padded = pad_guarded_factors(self.fused)
+        self.lowered: Graph = split_wide_reductions(padded, wanted=contraction_slices(padded.tensors))
         self.source, self.plans = lower_graph(self.lowered, prefix='autort_' + _ident(self.name))
         self._variants: Dict[tuple, dict] = {}
         self._module: Optional[capi.Module] = None
@@ -185,14 +186,16 @@ class ExportedOp:
 
     def _variant(self, env: Dict[str, int]) -> dict:
         """Graph, plans and module for these values of the named dimensions: the default ones, unless a reduction
-        of the program is worth slicing at these sizes (split_wide_reductions) or runs over a window of a few elements
-        given by named dimensions (bake_small_reduce_extents), which need their own kernels."""
+        of the program is worth slicing at these sizes (split_wide_reductions), runs over a window of a few elements
+        given by named dimensions (bake_small_reduce_extents) or multiplies a zero-padded operand
+        (pad_guarded_factors), which need their own kernels."""
         key = tuple(env[d] for d in self.fused.dim_names)
         v = self._variants.get(key)
         if v is None:
             # rows that one row kernel reduces and maps in a single launch are not sliced
             in_rows = any(p.row_group is not None and p.row_group.choose(env, {n: 0 for n in p.row_group.args})[1] for p in self.plans)
             g = bake_small_reduce_extents(self.lowered, env) if self.fused.dims else self.lowered
+            g = pad_guarded_factors(g, env) if self.fused.dims else g
             g = split_wide_reductions(g, env, wanted=contraction_slices(g.tensors)) if self.fused.dims and not in_rows else g
             if g is self.lowered:
                 v = {'graph': self.lowered, 'plans': self.plans, 'module': None, 'source': None}

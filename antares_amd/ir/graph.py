@@ -251,6 +251,127 @@ def bake_small_reduce_extents(graph: Graph, env: Dict[str, int], limit: int = 8)
                  source=graph.source)
 
 
+def _interval(e: Expr, extent) -> Optional[Tuple[int, int]]:
+    """[lowest, highest] value of an index expression made of axes, integer constants, + - and *; None for anything
+    else.  extent(axis name) -> int or None."""
+    if e.kind == 'const' and isinstance(e.value, int) and not isinstance(e.value, bool):
+        return e.value, e.value
+    if e.kind == 'axis':
+        n = extent(e.name)
+        return (0, n - 1) if n else None
+    if e.kind == 'cast' and e.dtype in ('int32', 'int64'):
+        return _interval(e.args[0], extent)
+    if e.kind == 'op' and e.name in ('+', '-', '*') and len(e.args) == 2:
+        a, b = _interval(e.args[0], extent), _interval(e.args[1], extent)
+        if a is None or b is None:
+            return None
+        if e.name == '+':
+            return a[0] + b[0], a[1] + b[1]
+        if e.name == '-':
+            return a[0] - b[1], a[1] - b[0]
+        c = [x * y for x in a for y in b]
+        return min(c), max(c)
+    return None
+
+
+def pad_guarded_factors(graph: Graph, env: Optional[Dict[str, int]] = None) -> Graph:
+    """A sum of products in which one factor is a guarded load, `x[..., HO + KH - 1, ...].when([HO + KH - 1 >= 0,
+    HO + KH - 1 < 32, ...], 0)` (the zero padding of a convolution, AntaresIR.md:166), is rewritten as
+
+        x__pad[P0, P1, ...] = x[P0 + lo0, P1 + lo1, ...].when([the same conditions on P + lo], 0)
+        out[...] +=! x__pad[..., HO + KH - 1 - lo, ...] * w[...]
+
+    where [lo, hi] is the interval each index takes: the guards are evaluated once per element of the padded copy
+    instead of once per term of the sum (nine times per element for a 3 x 3 filter, and in the inner loop of the
+    contraction).  Only when every condition compares one of the load's own index expressions with a constant, the
+    unguarded indices provably stay inside the tensor, the copy is at most four times the tensor, and the sum has at
+    least 64 terms.  `env`: values of named dimensions for one call (the result is then valid for those only)."""
+    from .nodes import Expr as E
+    from .printer import to_ir
+    env = env or {}
+
+    def value(d):
+        return d if isinstance(d, int) else env.get(d)
+    out: List[Statement] = []
+    tensors = dict(graph.tensors)
+    changed = False
+    for st in graph.statements:
+        done = False
+        root = st.root
+        terms = 1
+        for _, d in st.reduce_axes:
+            terms *= value(d) or 0
+        if st.reduce == '+' and not st.scatter and root.kind == 'op' and root.name == '*' and len(root.args) == 2 and terms >= 64 and \
+                all(value(d) for _, d in st.data_axes):
+            ext = {a: value(d) for a, d in st.data_axes + st.reduce_axes}
+            for which in (0, 1):
+                f = root.args[which]
+                if f.kind != 'when' or len(f.args) != 2 or f.merge != 'all' or not (f.args[1].kind == 'const' and f.args[1].value == 0):
+                    continue
+                loads = [n for n in walk(f.args[0]) if n.kind == 'load']
+                if len(loads) != 1 or not loads[0].args or loads[0].name == st.output or loads[0].name + '__pad' in tensors:
+                    continue
+                ld = loads[0]
+                if any(n.kind in ('load', 'when') for c in f.conds for n in walk(c)):
+                    continue
+                shape = [value(d) for d in tensors[ld.name].shape]
+                spans = [_interval(ix, ext.get) for ix in ld.args]
+                if any(sp is None for sp in spans) or any(n is None for n in shape):
+                    continue
+                texts = [to_ir(ix) for ix in ld.args]
+                # every condition: (index expression of the load) compared with an integer constant
+                guarded, ok = set(), True
+                for c in f.conds:
+                    sides = [to_ir(a) for a in c.args] if c.kind == 'op' and len(c.args) == 2 and c.name in ('<', '<=', '>', '>=', '==', '!=') else []
+                    hit = [k for k, t in enumerate(sides) if t in texts]
+                    other = c.args[1 - hit[0]] if len(hit) == 1 else None
+                    if other is None or not (other.kind == 'const' and isinstance(other.value, int)):
+                        ok = False
+                        break
+                    guarded.add(texts.index(sides[hit[0]]))
+                if not ok or not guarded:
+                    continue
+                if any(d not in guarded and not (0 <= sp[0] and sp[1] < n) for d, (sp, n) in enumerate(zip(spans, shape))):
+                    continue
+                size, numel = 1, 1
+                for sp, n in zip(spans, shape):
+                    size *= sp[1] - sp[0] + 1
+                    numel *= n
+                if size > 4 * numel:
+                    continue
+                # the padded copy
+                pad = ld.name + '__pad'
+                axes = []
+                for d in range(len(spans)):
+                    ax = f'P{d}'
+                    while ax in ext or any(ax == a for a, _ in axes):
+                        ax += 'p'
+                    axes.append((ax, spans[d][1] - spans[d][0] + 1))
+                moved = [E('op', 'int32', name='+', args=(E('axis', 'int32', name=ax), E('const', 'int32', value=sp[0]))) if sp[0] else E('axis', 'int32', name=ax)
+                         for (ax, _), sp in zip(axes, spans)]
+                by_text = dict(zip(texts, moved))
+                conds = tuple(E(c.kind, c.dtype, name=c.name, args=tuple(by_text.get(to_ir(a), a) for a in c.args)) for c in f.conds)
+                dt = tensors[ld.name].dtype
+                fill = E('when', dt, args=(E('load', dt, name=ld.name, args=tuple(moved)), E('const', dt, value=0 if dt.startswith('int') else 0.0)),
+                         conds=conds, merge='all')
+                tensors[pad] = TensorInfo(dtype=dt, shape=[n for _, n in axes])
+                s0 = Statement(output=pad, out_index=tuple(E('axis', 'int32', name=ax) for ax, _ in axes), root=fill, reduce=None, set_op=None,
+                               data_axes=list(axes), reduce_axes=[], out_dtype=dt, out_shape=[n for _, n in axes], scatter=False, reads=[ld.name])
+                shifted = tuple(E('op', 'int32', name='-', args=(ix, E('const', 'int32', value=sp[0]))) if sp[0] else ix for ix, sp in zip(ld.args, spans))
+                inner = rewrite(f.args[0], lambda n: E('load', dt, name=pad, args=shifted) if n is ld else None)
+                new_root = E(root.kind, root.dtype, name=root.name, args=(inner, root.args[1]) if which == 0 else (root.args[0], inner))
+                reads = [r for r in st.reads if r != ld.name or any(n.kind == 'load' and n.name == ld.name for n in walk(new_root))] + [pad]
+                out += [s0, replace(st, root=new_root, reads=reads)]
+                done = changed = True
+                break
+        if not done:
+            out.append(st)
+    if not changed:
+        return graph
+    return Graph(statements=out, tensors=tensors, declared=graph.declared, outputs=graph.outputs, dims=graph.dims,
+                 source=graph.source)
+
+
 def split_wide_reductions(graph: Graph, env: Optional[Dict[str, int]] = None, wanted=None) -> Graph:
     """A reduction whose outputs are too few to fill the chip is rewritten as
 

@@ -705,19 +705,28 @@ MATRIX_CASES = [
 ]
 
 
-@pytest.mark.parametrize('ir,inputs,shapes', MATRIX_CASES)
-def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, ir, inputs, shapes):
+@pytest.mark.parametrize('ir,inputs,shapes,how', [c + (None,) for c in MATRIX_CASES] +
+                         [c + ('guards in the kernel',) for c in MATRIX_CASES if '.when(' in c[0]])
+def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, monkeypatch, ir, inputs, shapes, how):
     """Sums of products of two loads whose indices split into a row (or column) part and a k part run on
     v_mfma_f32_32x32x2_f32 when k is a multiple of 16 and there are enough tiles; results are the oracle's to the
-    rounding of a float32 sum in another order, and the register-tiled variant gives the same to that rounding."""
+    rounding of a float32 sum in another order, and the register-tiled variant gives the same to that rounding.
+    A zero-padded factor is normally copied into a padded tensor first (one more statement in front); the cases marked
+    'guards in the kernel' switch that off, so that the contraction itself evaluates the conditions - what a program
+    gets whose conditions the rewrite does not take."""
     from antares_amd.ir import parse_program
     from oracle.cpu_backend import CpuModule
-    note(f'matrix-instruction contraction {ir[:60]} {shapes}')
+    note(f'matrix-instruction contraction {ir[:60]} {shapes} {how or ""}')
     dev = autort.device()
-    op = autort.export(ir=ir, inputs=inputs, name='mfma_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    if how:
+        monkeypatch.setattr('antares_amd.autort.op.pad_guarded_factors', lambda graph, env=None: graph)
+    op = autort.export(ir=ir, inputs=inputs, name='mfma_' + str(abs(hash((ir, tuple(inputs), how))) % 10 ** 8))
     op.fast_path = None
     env = dims_of(inputs, shapes)
     plan = op.plans_for(env)[-1]                  # a filter of a few named elements gets kernels of its own
+    if '.when(' in ir:
+        padded = any(n.endswith('__pad') for n in plan.args)
+        assert padded == (how is None) and len(op.plans_for(env)) == (2 if padded else 1)
     assert plan.choose(env, {n: 0 for n in plan.args})[0] in [v for t, v in plan.variants.items() if t.startswith('matrix')]
     assert plan.row_group is None                 # nothing else takes the statement
     g = torch.Generator().manual_seed(len(ir))

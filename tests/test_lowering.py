@@ -209,3 +209,35 @@ def test_the_programs_of_the_lowering_benchmark_lower_and_take_the_kernels_they_
             assert plans[0].row_group is not None and plans[0].row_group.count == 3, name
         if 'one launch' in name:
             assert plans[0].covers == 2, name
+
+
+def test_a_zero_padded_factor_is_copied_into_a_padded_tensor_once():
+    """`x[.., HO * 2 + KH - 1, WO + KW - 1].when([bounds], 0) * w[...]`: the guards are evaluated once per element of a
+    padded copy, the contraction reads the copy unguarded; the rewrite is refused when it cannot prove what it needs."""
+    import numpy as np
+    from antares_amd.ir.graph import pad_guarded_factors
+    from oracle.cpu_backend import CpuModule
+    conv = ('output0[N, F, HO, WO] +=! input0[N, C, HO * 2 + KH - 1, WO + KW - 1].when([HO * 2 + KH - 1 >= 0, HO * 2 + KH - 1 < 32, '
+            'WO + KW - 1 >= 0, WO + KW - 1 < 32], 0.0) * input1[F, C, KH, KW] where HO in 16, WO in 32')
+    inputs = ['input0=float32[N:2, C:8, H:32, W:32]', 'input1=float32[F:8, C:8, KH:3, KW:3]']
+    g = fuse_elementwise(parse_program(conv, inputs))
+    env = {'N': 2, 'C': 8, 'H': 32, 'W': 32, 'F': 8, 'KH': 3, 'KW': 3}
+    padded = pad_guarded_factors(g, env)
+    assert [s.output for s in padded.statements] == ['input0__pad', 'output0'] and padded.tensors['input0__pad'].shape == [2, 8, 33, 34]
+    assert pad_guarded_factors(padded, env) is padded and pad_guarded_factors(g, {}) is g        # once; and not without the extents
+    mc = hip_codegen._matrix_contraction(padded.statements[1], padded.tensors)
+    assert mc is not None and mc['guards'] == {'a': [], 'b': []}
+    rng = np.random.default_rng(1)
+    x, w = rng.standard_normal((2, 8, 32, 32)).astype(np.float32), rng.standard_normal((8, 8, 3, 3)).astype(np.float32)
+    assert np.array_equal(CpuModule(padded, fast_math=False)(input0=x, input1=w)['output0'], CpuModule(g, fast_math=False)(input0=x, input1=w)['output0'])
+    refused = [
+        # a condition on something that is no index of the load; an unguarded index that may leave the tensor; too few terms
+        conv.replace('WO + KW - 1 < 32]', 'WO + KW - 1 < 32, HO < 9]'),
+        conv.replace('input0[N, C,', 'input0[N + 1, C,').replace('WO in 32', 'WO in 32, N in 2'),
+        'output0[N, M] +=! input0[N, K + 5].when([K + 5 < 40], 0.0) * input1[K, M] where K in 40',
+    ]
+    for ir in refused[:2]:
+        g2 = fuse_elementwise(parse_program(ir, inputs))
+        assert pad_guarded_factors(g2, env) is g2, ir
+    g3 = fuse_elementwise(parse_program(refused[2], ['input0=float32[N:64, J:40]', 'input1=float32[K:40, M:64]']))
+    assert pad_guarded_factors(g3, {'N': 64, 'J': 40, 'K': 40, 'M': 64}) is g3
