@@ -893,11 +893,14 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         return f.kind == 'cast' and f.dtype == 'float32' and f.args[0] is ld and tensors[ld.name].dtype == 'float16'
     # fp16 operands that are only cast up: the tiles stay fp16 in LDS and go to v_mfma_f32_32x32x16_f16 - the
     # products of two fp16 values are exact in float32 either way, and the matrix time is a sixteenth
-    HM = (half_cast(mc['fa'], la) and half_cast(mc['fb'], lb)) or st.root.dtype == 'float16'
-    BK = 32 if (TS == 64 or HM) else 16               # k per tile: the small blocks take twice the k per barrier
-    LD, RS = BK + (8 if HM else 4), BLOCK // BK       # elements per row of a staged tile (16-byte aligned, rows on distinct banks); rows between a lane's elements when lanes walk k
-    ET = 'half_t' if HM else 'float'                  # element type of the staged tiles
-    VW = 8 if HM else 4                               # elements per 16-byte vector of them
+    IM = st.root.dtype == 'int32'                     # int8 operands cast to int32: int8 tiles, v_mfma_i32_32x32x32_i8, int32 accumulators
+    HM = (half_cast(mc['fa'], la) and half_cast(mc['fb'], lb)) or st.root.dtype == 'float16' or IM      # operands staged as loaded
+    BK = 64 if IM else (32 if (TS == 64 or HM) else 16)   # k per tile: the small blocks take twice the k per barrier
+    LD, RS = BK + (16 if IM else (8 if HM else 4)), BLOCK // BK       # elements per row of a staged tile (16-byte aligned, rows on distinct banks); rows between a lane's elements when lanes walk k
+    ET = 'signed char' if IM else ('half_t' if HM else 'float')      # element type of the staged tiles
+    VW = 16 if IM else (8 if HM else 4)               # elements per 16-byte vector of them
+    KG = 32 if IM else (16 if HM else 8)              # k one round of matrix instructions multiplies
+    ZERO = '0' if IM else '0.f'
     # how an operand travels: 'rows' (lanes along rows, PER k each), 'k' (lanes along k, PER rows each), or 'kvec' (a
     # lane fetches 16 bytes of k of PER / VL rows: rows of k in memory, whole vectors, aligned - the launcher checks)
     def vector_ok(x, ld):       # the staged value must be the loaded one, in the tile's element type
@@ -960,7 +963,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         return (f'{{ const {oct_} __t = ({oct_}){acc}; (void)__t; '
                 f'{tail.output}[__cm[__r] + __cn[__c]] = ({HIP_TYPE[tail.out_dtype]})({tem.expr(tail.root)}); }}')
     b = [_signature(sym, args, tensors, dims, written) + ' {'] + _extents(st)
-    b += ['  typedef float __f16v __attribute__((ext_vector_type(16)));',
+    b += [f'  typedef {"int" if IM else "float"} __f16v __attribute__((ext_vector_type(16)));',
+          '  typedef int __i4 __attribute__((ext_vector_type(4)));',
           f'  typedef {ET} __f4 __attribute__((ext_vector_type({VW})));      // 16 bytes of a staged tile',
           f'  __shared__ __attribute__((aligned(16))) {ET} __As[2][{TS} * {LD}];     // [row][k], {BK} k and 16 bytes of padding per row',
           f'  __shared__ __attribute__((aligned(16))) {ET} __Bs[2][{TS} * {LD}];     // [column][k]',
@@ -1073,18 +1077,24 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           '      #pragma unroll',
           f'      for (int __j = 0; __j < {NT}; ++__j)',
           '        #pragma unroll',
-          '        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = 0.f;',
+          f'        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = {ZERO};',
           f'    const int __row0 = __wm * {HALF} + (__lane & 31), __col0 = __wn * {HALF} + (__lane & 31), __kq = (__lane >> 5) * {VW};',
           '    auto __multiply = [&](int __buf) {',
           '      #pragma unroll',
-          f'      for (int __g = 0; __g < {BK // (16 if HM else 8)}; ++__g) {{',
+          f'      for (int __g = 0; __g < {BK // KG}; ++__g) {{',
           f'        __f4 __a[{NT}], __b[{NT}];',
           '        #pragma unroll',
           f'        for (int __i = 0; __i < {NT}; ++__i) {{',
-          f'          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * {LD} + __g * {16 if HM else 8} + __kq];',
-          f'          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * {LD} + __g * {16 if HM else 8} + __kq];',
+          f'          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * {LD} + __g * {KG} + __kq];',
+          f'          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * {LD} + __g * {KG} + __kq];',
           '        }']
-    if HM:      # a lane supplies 8 consecutive k of its row (column): k = (lane / 32) * 8 .. + 7 of the 16
+    if IM:      # a lane supplies 16 consecutive k of its row (column), the same ones for both operands
+        b += ['        #pragma unroll',
+              f'        for (int __i = 0; __i < {NT}; ++__i)',
+              '          #pragma unroll',
+              f'          for (int __j = 0; __j < {NT}; ++__j)',
+              '            __acc[__i][__j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(__i4, __a[__i]), __builtin_bit_cast(__i4, __b[__j]), __acc[__i][__j], 0, 0, 0);']
+    elif HM:    # a lane supplies 8 consecutive k of its row (column): k = (lane / 32) * 8 .. + 7 of the 16
         b += ['        #pragma unroll',
               f'        for (int __i = 0; __i < {NT}; ++__i)',
               '          #pragma unroll',
@@ -1238,7 +1248,7 @@ def _matrix_contraction(st, tensors):
     data axes that only the first load uses are rows (M), those only the second uses are columns (N), those both use
     are a batch, the reduce axes are k.  Every index of a load must split into a part that depends on k axes and a
     part that does not, so that an element's address is a row (column) offset plus a k offset.  -> dict or None."""
-    if st.scatter or st.reduce != '+' or st.root.dtype not in ('float32', 'float16') or not st.reduce_axes or not st.data_axes:
+    if st.scatter or st.reduce != '+' or st.root.dtype not in ('float32', 'float16', 'int32') or not st.reduce_axes or not st.data_axes:
         return None
     root = st.root
     if root.kind == 'when' or root.kind != 'op' or root.name != '*' or len(root.args) != 2:
@@ -1271,6 +1281,11 @@ def _matrix_contraction(st, tensors):
     # exactly and sums in float32, the result is rounded once - closer to the exact sum than the running float16 sum.
     if st.root.dtype == 'float16' and not (fa is la and fb is lb and tensors[la.name].dtype == tensors[lb.name].dtype == 'float16'):
         return None
+    # An int32 statement is taken as the product of two int8 loads cast to int32: v_mfma_i32_32x32x32_i8 multiplies and
+    # sums them exactly, and integer sums do not depend on their order - the result is the reference's, bit for bit.
+    if st.root.dtype == 'int32' and not all(f.kind == 'cast' and f.dtype == 'int32' and f.args[0] is ld and tensors[ld.name].dtype == 'int8'
+                                            for f, ld in ((fa, la), (fb, lb))):
+        return None
     # axes may be used inside the indices of the two loads and inside the guards only
     inside = sum(1 for n in (la, lb) for a in n.args for m in walk(a) if m.kind == 'axis') + \
         sum(1 for tag in guards for c in guards[tag] for m in walk(c) if m.kind == 'axis')
@@ -1291,7 +1306,7 @@ def _matrix_contraction(st, tensors):
     batch = [a for a in axes if a in ua and a in ub]
     if not m_axes or not n_axes or len(m_axes) + len(n_axes) + len(batch) != len(axes):
         return None
-    if ITEMSIZE[tensors[la.name].dtype] not in (2, 4) or ITEMSIZE[tensors[lb.name].dtype] not in (2, 4):
+    if any(ITEMSIZE[tensors[ld.name].dtype] not in ((1,) if st.root.dtype == 'int32' else (2, 4)) for ld in (la, lb)):
         return None
     plain = ExprEmitter(tensors)
     parts = {}

@@ -177,6 +177,8 @@ LOWERING_CASES = [
      ['input0=float16[N:4096, K:1024]', 'input1=float16[M:4096, K:1024]'], [(4096, 1024), (4096, 1024)], ('flop', 2 * 4096 * 4096 * 1024)),
     ('fp16 product 2048^3 (float16 statement)', 'output0[N, M] +=! input0[N, K] * input1[K, M]',
      ['input0=float16[N:2048, K:2048]', 'input1=float16[K:2048, M:2048]'], [(2048, 2048), (2048, 2048)], ('flop', 2 * 2048 ** 3)),
+    ('int8 A B^T into int32 4096^3', 'output0[N, M] +=! input0[N, K].cast(`int32`) * input1[M, K].cast(`int32`)',
+     ['input0=int8[N:4096, K:4096]', 'input1=int8[M:4096, K:4096]'], [(4096, 4096), (4096, 4096)], ('flop', 2 * 4096 ** 3)),
     ('batched fp32 product 8 x 512^3', 'output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]',
      ['input0=float32[B:8, N:512, K:512]', 'input1=float32[B:8, K:512, M:512]'], [(8, 512, 512), (8, 512, 512)], ('flop', 2 * 8 * 512 ** 3)),
     ('fp32 A B^T 512x512x8192 (sliced along k)', 'output0[N, M] +=! input0[N, K] * input1[M, K]',
@@ -220,7 +222,8 @@ def bench_lowering(torch, autort, capi, steps, warmup):
         op.fast_path = None
         g = torch.Generator('cpu').manual_seed(len(name))
         ts = [torch.randint(0, 32000, shp, generator=g, dtype=torch.int32).to(dev) if 'int32' in spec else
-              torch.randn(shp, generator=g).to(torch.float16 if 'float16' in spec else torch.float32).to(dev) for spec, shp in zip(inputs, shapes)]
+              (torch.randint(-128, 128, shp, generator=g, dtype=torch.int8).to(dev) if 'int8' in spec else
+               torch.randn(shp, generator=g).to(torch.float16 if 'float16' in spec else torch.float32).to(dev)) for spec, shp in zip(inputs, shapes)]
         res = op(*ts)
         # eight calls per replayed graph, each on its own copy of the inputs: a graph of one short kernel would time
         # the replay itself (about 17 us), and the same tensors every time would be served by the caches

@@ -832,6 +832,43 @@ def test_contractions_with_few_output_tiles_are_cut_into_slices_of_k(autort, ir,
     assert got.shape == want.shape and np.allclose(got, want, rtol=1e-4, atol=2e-5 * K ** 0.5 * 4), np.abs(got - want).max()
 
 
+@pytest.mark.parametrize('ir,inputs,shapes', [
+    ('output0[N, M] +=! input0[N, K].cast(`int32`) * input1[M, K].cast(`int32`)', ['input0=int8[N:1000, K:528]', 'input1=int8[M:1024, K:528]'],
+     [(1000, 528), (1024, 528)]),
+    ('output0[N, M] +=! input0[N, K].cast(`int32`) * input1[K, M].cast(`int32`)', ['input0=int8[N:300, K:200]', 'input1=int8[K:200, M:260]'],
+     [(300, 200), (200, 260)]),
+    ('output0[B, N, M] +=! input0[B, N, K].cast(`int32`) * input1[B, M, K].cast(`int32`)', ['input0=int8[B:2, N:256, K:4096]', 'input1=int8[B:2, M:192, K:4096]'],
+     [(2, 256, 4096), (2, 192, 4096)]),
+])
+def test_int8_contractions_are_bit_exact_on_the_matrix_instructions(autort, ir, inputs, shapes):
+    """An int32 sum of products of two int8 loads cast to int32 runs on v_mfma_i32_32x32x32_i8: exact products, exact
+    sums, and integer sums do not depend on their order - every kernel gives the integers of a 64-bit product (and the
+    oracle's), bit for bit; the third case is also cut into slices of k."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'int8 contraction on the matrix instructions {ir} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='mfma_i8_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    op.fast_path = None
+    env = dims_of(inputs, shapes)
+    plan = op.plans_for(env)[0]
+    assert plan.matrix is not None and len(op.plans_for(env)) == (2 if 'B:2' in inputs[0] else 1)
+    g = torch.Generator().manual_seed(len(ir))
+    a, b = [torch.randint(-128, 128, shape, generator=g, dtype=torch.int8) for shape in shapes]
+    exact = torch.einsum('...nk,...km->...nm', a.long(), b.long() if ir.split('input1')[1].startswith('[K, M]') else b.long().transpose(-1, -2)).to(torch.int32).numpy()
+    if a.numel() <= 1 << 20:
+        want = CpuModule(parse_program(ir, inputs), fast_math=False)(input0=a.numpy(), input1=b.numpy())['output0']
+        assert np.array_equal(want, exact)
+    M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
+    for tag, side in (('matrix', 128), ('matrix64', 64), ('matrixv', 128), ('matrix64v', 64)):
+        if tag not in plan.variants or (tag.endswith('v') and shapes[0][-1] % plan.matrix['vec_width'][0]):
+            continue                # the vector kernels are launched for whole vectors of k only
+        blocks = ((M + side - 1) // side) * ((N + side - 1) // side) * B
+        plan.choose = lambda env_, ptrs, tag=tag, blocks=blocks: (plan.variants[tag], blocks, 256)
+        got = op(a.to(dev), b.to(dev))
+        assert got.dtype == torch.int32 and np.array_equal(got.cpu().numpy(), exact), tag
+
+
 TAIL_CASES = [
     # AntaresIR.md:248-250 (ConvBiasRelu tail fusion); a product with a scaled result, a per-column and a per-element
     # term under a tanh; a float16 result of a float32 sum; a column-wise maximum with a conditional store behind it
