@@ -860,14 +860,15 @@ def lower_statement(st, graph, name: str, tail=None) -> Tuple[str, KernelPlan]:
             variants['matrix'], variants['matrix64'] = name + '_m', name + '_m64'
             ext = dict(st.data_axes + st.reduce_axes)
             plan.matrix = {key: [ext[a] for a in mc[key]] for key in ('m', 'n', 'batch', 'k')}
-            if mc['vec']['a'] or mc['vec']['b']:
+            wide_ok = {t: mc['vec'][t] or mc['rowrun'][t] for t in ('a', 'b')}
+            if wide_ok['a'] or wide_ok['b']:
                 src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_mv', mc, vectors=True))
                 src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_m64v', mc, TS=64, vectors=True))
                 variants['matrixv'], variants['matrix64v'] = name + '_mv', name + '_m64v'
-                wide = [ITEMSIZE[tensors[mc['l' + t].name].dtype] for t in ('a', 'b') if mc['vec'][t]]
-                plan.matrix['vec_tensors'] = [mc['l' + t].name for t in ('a', 'b') if mc['vec'][t]]
+                wide = [ITEMSIZE[tensors[mc['l' + t].name].dtype] for t in ('a', 'b') if wide_ok[t]]
+                plan.matrix['vec_tensors'] = [mc['l' + t].name for t in ('a', 'b') if wide_ok[t]]
                 plan.matrix['vec_width'] = [16 // min(wide)]
-                plan.matrix['vec_pitch'] = [mc['pitch'][t] for t in ('a', 'b') if mc['vec'][t]]     # row lengths, as dimensions to multiply
+                plan.matrix['vec_pitch'] = [mc['pitch'][t] for t in ('a', 'b') if wide_ok[t]]     # row lengths, as dimensions to multiply
 
     return '\n\n'.join(src), plan
 
@@ -905,7 +906,11 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     # lane fetches 16 bytes of k of PER / VL rows: rows of k in memory, whole vectors, aligned - the launcher checks)
     def vector_ok(x, ld):       # the staged value must be the loaded one, in the tile's element type
         return vectors and mc['vec'][x] and (HM or (tensors[ld.name].dtype == 'float32' and mc['f' + x] is ld))
-    mode = {x: ('kvec' if vector_ok(x, ld) else ('k' if mc['parts'][x][2] else 'rows')) for x, ld in (('a', la), ('b', lb))}
+    mode = {x: ('kvec' if vector_ok(x, ld) else ('tr' if (vectors and mc['rowrun'][x]) else ('k' if mc['parts'][x][2] else 'rows')))
+            for x, ld in (('a', la), ('b', lb))}
+    PT = TS + 32                                      # halves per k row of a tile staged as it lies, [k][row]: 64 bytes past a multiple of 256
+    CG = TS // 8                                      # 16-byte groups of rows in such a tile
+    KP = BLOCK // CG                                  # k rows of it that one pass of the 256 threads covers
     VL = 16 // ITEMSIZE[tensors[la.name].dtype] if mode['a'] == 'kvec' else (16 // ITEMSIZE[tensors[lb.name].dtype] if mode['b'] == 'kvec' else VW)
     VPR = BK // VL                                    # vectors per row of a tile
     RV = BLOCK // VPR                                 # rows a pass of the 256 threads covers
@@ -966,8 +971,10 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
     b += [f'  typedef {"int" if IM else "float"} __f16v __attribute__((ext_vector_type(16)));',
           '  typedef int __i4 __attribute__((ext_vector_type(4)));',
           f'  typedef {ET} __f4 __attribute__((ext_vector_type({VW})));      // 16 bytes of a staged tile',
-          f'  __shared__ __attribute__((aligned(16))) {ET} __As[2][{TS} * {LD}];     // [row][k], {BK} k and 16 bytes of padding per row',
-          f'  __shared__ __attribute__((aligned(16))) {ET} __Bs[2][{TS} * {LD}];     // [column][k]',
+          f'  __shared__ __attribute__((aligned(16))) {ET} __As[2][{BK * PT if mode["a"] == "tr" else TS * LD}];     // [row][k], {BK} k and 16 bytes of padding per row ([k][row] when staged as it lies)',
+          f'  __shared__ __attribute__((aligned(16))) {ET} __Bs[2][{BK * PT if mode["b"] == "tr" else TS * LD}];     // [column][k]',
+          '  typedef short __s4 __attribute__((ext_vector_type(4)));',
+          '  typedef __attribute__((address_space(3))) __s4 __lds_s4;',
           f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][{BK}], __bk[2][{BK}];'] + \
          [f'  __shared__ long long __xm{q}[{TS}], __xn{q}[{TS}];      // row and column part of the offsets into {ld.name} (read by the tail)'
           for q, (ld, _, _, _) in enumerate(extra)] + \
@@ -1019,6 +1026,13 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
                   f'    for (int __j = 0; __j < {TS // RV}; ++__j) __p{x}[__j] = {ld.name} + {tab}[__tid / {VPR} + {RV} * __j];',
                   f'    __v{x} __r{x}[{DEPTH}][{TS // RV}];']
             continue
+        if mode[x] == 'tr':
+            # a lane owns 8 neighbouring rows (a whole vector: all inside the extents or all past them) and every KP-th k;
+            # the last of them names the address, so that a group past the end re-reads the last whole vector
+            b += [f'    typedef {ct} __w{x} __attribute__((ext_vector_type(8)));',
+                  f'    const {ct}* __p{x} = {ld.name} + ({tab}[(__tid % {CG}) * 8 + 7] - 7);',
+                  f'    __w{x} __r{x}[{DEPTH}][{BK // KP}];']
+            continue
         if mode[x] == 'k':
             b += [f'    const {ct}* __p{x}[{PER}];', '    #pragma unroll',
                   f'    for (int __j = 0; __j < {PER}; ++__j) __p{x}[__j] = {ld.name} + {tab}[__rw + {RS} * __j];']
@@ -1033,6 +1047,10 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
             b += [f'      {{ const long long __k0 = (long long)__ktile * {BK} + (__tid % {VPR}) * {VL};',
                   f'        const long long __ko = __k0 + {VL} <= __K ? __k0 : 0;', '        #pragma unroll',
                   f'        for (int __j = 0; __j < {TS // RV}; ++__j) __r{x}[__S][__j] = *(const __v{x}*)(__p{x}[__j] + __ko); }}']
+            continue
+        if mode[x] == 'tr':
+            b += ['      #pragma unroll',
+                  f'      for (int __j = 0; __j < {BK // KP}; ++__j) __r{x}[__S][__j] = *(const __w{x}*)(__p{x} + {ktab_}[__buf][__tid / {CG} + {KP} * __j]);']
             continue
         if G[x]:
             row, k = (f'__rw + {RS} * __j', '__kl') if mode[x] == 'k' else ('__ml', '__kh + __j')
@@ -1057,6 +1075,11 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
                 b += [f'        *(__v{x}*){dst} = __in ? __r{x}[__S][{j}] : (__v{x})(0);']
             b += ['      }']
             continue
+        if mode[x] == 'tr':
+            for j in range(BK // KP):
+                b += [f'      {{ const int __ks = __tid / {CG} + {KP * j};',
+                      f'        *(__w{x}*)&{lds}[__buf][__ks * {PT} + (__tid % {CG}) * 8] = (long long)__kt * {BK} + __ks < __K ? __r{x}[__S][{j}] : (__w{x})(0); }}']
+            continue
         def inside(j, x=x):
             return f' && ((__g{x}[__S] >> {j}) & 1u)' if G[x] else ''
         if mode[x] == 'k':
@@ -1070,6 +1093,18 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
             for q in range(PER // VW):
                 b += [f'        *(__f4*)&{lds}[__buf][__ml * {LD} + __kh + {VW * q}] = __f4{{' + ', '.join(guarded(VW * q + e) for e in range(VW)) + '};']
             b += ['      }']
+    def feed(x, lds, w):            # C text that fetches operand x of accumulator tile __i for round __g
+        if mode[x] != 'tr':
+            base = '__row0' if x == 'a' else '__col0'
+            return f'          __{x}[__i] = *(const __f4*)&{lds}[__buf][({base} + 32 * __i) * {LD} + __g * {KG} + __kq];'
+        # 16 lanes read a patch of 4 k x 16 rows and each receives the four k of one row; two patches, 4 k apart, make
+        # the 8 consecutive k a lane supplies: k = (lane / 32) * 8 .. + 7, row = lane % 32 of the tile - as above
+        at = f'&{lds}[__buf][(__g * 16 + __tq) * {PT} + {w} * {HALF} + 32 * __i + __tc]'
+        return (f'          {{ const __s4 __lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__lds_s4*)({at})), '
+                f'__hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__lds_s4*)({at} + 4 * {PT}));\n'
+                f'            typedef half_t __h4 __attribute__((ext_vector_type(4)));\n'
+                f'            const __h4 __l = __builtin_bit_cast(__h4, __lo), __h = __builtin_bit_cast(__h4, __hi);\n'
+                f'            __{x}[__i] = __f4{{__l[0], __l[1], __l[2], __l[3], __h[0], __h[1], __h[2], __h[3]}}; }}')
     b += ['    };',
           f'    __f16v __acc[{NT}][{NT}];',
           '    #pragma unroll',
@@ -1079,14 +1114,15 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           '        #pragma unroll',
           f'        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = {ZERO};',
           f'    const int __row0 = __wm * {HALF} + (__lane & 31), __col0 = __wn * {HALF} + (__lane & 31), __kq = (__lane >> 5) * {VW};',
+          '    const int __tq = (__lane >> 5) * 8 + ((__lane & 15) >> 2), __tc = ((__lane & 31) >> 4) * 16 + (__lane & 3) * 4; (void)__tq; (void)__tc;',
           '    auto __multiply = [&](int __buf) {',
           '      #pragma unroll',
           f'      for (int __g = 0; __g < {BK // KG}; ++__g) {{',
           f'        __f4 __a[{NT}], __b[{NT}];',
           '        #pragma unroll',
           f'        for (int __i = 0; __i < {NT}; ++__i) {{',
-          f'          __a[__i] = *(const __f4*)&__As[__buf][(__row0 + 32 * __i) * {LD} + __g * {KG} + __kq];',
-          f'          __b[__i] = *(const __f4*)&__Bs[__buf][(__col0 + 32 * __i) * {LD} + __g * {KG} + __kq];',
+          feed('a', '__As', '__wm'),
+          feed('b', '__Bs', '__wn'),
           '        }']
     if IM:      # a lane supplies 16 consecutive k of its row (column), the same ones for both operands
         b += ['        #pragma unroll',
@@ -1357,8 +1393,22 @@ def _matrix_contraction(st, tensors):
                     all(d == red[k] for d, k in zip(tensors[ld.name].shape[-nk + 1:] if nk > 1 else [], k_axes[1:])) and
                     (tail[0].kind != 'axis' or tensors[ld.name].shape[-nk] == red[k_axes[0]]) and not guards[tag])
         pitch[tag] = list(tensors[ld.name].shape[-nk:])
+    # The other way round, for fp16 tiles: an operand whose last index is its fastest row (column) axis, bare, over a
+    # dimension of exactly that extent (`input1[K, M]` of a product, V of an attention) has neighbouring rows next to
+    # each other in memory.  It is fetched in 16-byte vectors of rows, staged as it lies ([k][row]) and transposed on
+    # its way out of LDS (ds_read_b64_tr_b16), when that extent is whole vectors.
+    half = st.root.dtype == 'float16' or all(f.kind == 'cast' and f.dtype == 'float32' and f.args[0] is ld and tensors[ld.name].dtype == 'float16'
+                                             for f, ld in ((fa, la), (fb, lb)))
+    rowrun = {}
+    for tag, ld, own in (('a', la, m_axes), ('b', lb, n_axes)):
+        last = ld.args[-1]
+        ext_own = dict(st.data_axes)[own[-1]]
+        rowrun[tag] = (half and not vec[tag] and not guards[tag] and not parts[tag][2] and last.kind == 'axis' and last.name == own[-1] and
+                       not any(own[-1] in _axes_of(a) for a in ld.args[:-1]) and tensors[ld.name].shape[-1] == ext_own)
+        if rowrun[tag]:
+            pitch[tag] = [ext_own]
     return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts, 'vec': vec,
-            'guards': guards, 'pitch': pitch}
+            'guards': guards, 'pitch': pitch, 'rowrun': rowrun}
 
 
 def _tail_of(graph, i: int):

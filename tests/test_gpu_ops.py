@@ -741,7 +741,7 @@ def test_contractions_on_the_matrix_instructions_match_the_oracle(autort, monkey
     M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
     rule = plan.choose
     sizes = [('matrix', 128), ('matrix64', 64)]                # blocks of 128 x 128 and of 64 x 64 outputs
-    if 'matrixv' in plan.variants and K % plan.matrix['vec_width'][0] == 0:
+    if 'matrixv' in plan.variants and (plan._matrix_choice(env, {n: 0 for n in plan.args})[0] or '').endswith('v'):
         sizes += [('matrixv', 128), ('matrix64v', 64)]          # ... and their forms that fetch rows of k in 16-byte vectors
         ptrs = {n: 0 for n in plan.args}
         assert plan.choose(env, ptrs)[0] in (plan.variants['matrixv'], plan.variants['matrix64v'])
@@ -833,6 +833,43 @@ def test_contractions_with_few_output_tiles_are_cut_into_slices_of_k(autort, ir,
 
 
 @pytest.mark.parametrize('ir,inputs,shapes', [
+    # both operands stored along rows; the second one only, batched (the V of an attention), ragged tiles, k = 2.5 tiles
+    ('output0[N, M] +=! input0[K, N].to(`float32`) * input1[K, M].to(`float32`)', ['input0=float16[K:96, N:1000]', 'input1=float16[K:96, M:520]'],
+     [(96, 1000), (96, 520)]),
+    ('output0[B, S, D] +=! input0[B, S, T].to(`float32`) * input1[B, T, D].to(`float32`)', ['input0=float16[B:3, S:300, T:80]', 'input1=float16[B:3, T:80, D:128]'],
+     [(3, 300, 80), (3, 80, 128)]),
+])
+def test_fp16_operands_stored_along_rows_are_staged_as_they_lie(autort, ir, inputs, shapes):
+    """An fp16 operand whose neighbouring rows (columns) are neighbours in memory - `input1[K, M]` - is fetched in 16-byte
+    vectors of rows, staged in LDS as [k][row] and transposed on its way to the matrix instruction by
+    ds_read_b64_tr_b16; the result is that of the kernels that stage it row by row, and the oracle's."""
+    from antares_amd.ir import parse_program
+    from oracle.cpu_backend import CpuModule
+    note(f'fp16 operands staged as they lie {ir} {shapes}')
+    dev = autort.device()
+    op = autort.export(ir=ir, inputs=inputs, name='mfma_tr_' + str(abs(hash((ir, tuple(inputs)))) % 10 ** 8))
+    op.fast_path = None
+    env = dims_of(inputs, shapes)
+    plan = op.plans_for(env)[-1]
+    zero = {n: 0 for n in plan.args}
+    assert plan.choose(env, zero)[0] in (plan.variants['matrixv'], plan.variants['matrix64v'])
+    odd = {k: (v + 4 if k in ('M', 'D') else v) for k, v in env.items()}          # a row length that is no whole number of vectors
+    assert plan.choose(odd, zero)[0] in (plan.variants['matrix'], plan.variants['matrix64'])
+    g = torch.Generator().manual_seed(len(ir))
+    a, b = [(torch.randn(shape, generator=g) * 0.5).half() for shape in shapes]
+    want = CpuModule(parse_program(ir, inputs), fast_math=False)(input0=a.numpy(), input1=b.numpy())['output0']
+    M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
+    got = {}
+    for tag, side in (('matrix', 128), ('matrix64', 64), ('matrixv', 128), ('matrix64v', 64)):
+        blocks = ((M + side - 1) // side) * ((N + side - 1) // side) * B
+        plan.choose = lambda env_, ptrs, tag=tag, blocks=blocks: (plan.variants[tag], blocks, 256)
+        got[tag] = op(a.to(dev), b.to(dev)).cpu().numpy()
+        assert np.allclose(got[tag], want, rtol=1e-4, atol=1e-3), (tag, np.abs(got[tag] - want).max())
+    # the same products in the same order of k inside a tile: the bits agree between the two ways of staging
+    assert np.array_equal(got['matrix'], got['matrixv']) and np.array_equal(got['matrix64'], got['matrix64v'])
+
+
+@pytest.mark.parametrize('ir,inputs,shapes', [
     ('output0[N, M] +=! input0[N, K].cast(`int32`) * input1[M, K].cast(`int32`)', ['input0=int8[N:1000, K:528]', 'input1=int8[M:1024, K:528]'],
      [(1000, 528), (1024, 528)]),
     ('output0[N, M] +=! input0[N, K].cast(`int32`) * input1[K, M].cast(`int32`)', ['input0=int8[N:300, K:200]', 'input1=int8[K:200, M:260]'],
@@ -914,7 +951,8 @@ def test_a_map_behind_a_reduction_is_applied_at_its_stores(autort, ir, inputs, s
     if matrix:
         M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
         launches += [(tag, ((M + side - 1) // side) * ((N + side - 1) // side) * B) for tag, side in (('matrix', 128), ('matrix64', 64)) if tag in plan.variants]
-        launches += [(tag, ((M + side - 1) // side) * ((N + side - 1) // side) * B) for tag, side in (('matrixv', 128), ('matrix64v', 64)) if tag in plan.variants]
+        if (plan._matrix_choice(env, {n: 0 for n in plan.args})[0] or '').endswith('v'):       # whole vectors everywhere they are fetched
+            launches += [(tag, ((M + side - 1) // side) * ((N + side - 1) // side) * B) for tag, side in (('matrixv', 128), ('matrix64v', 64))]
     tol = 1e-2 if want.dtype == np.float16 or 'float16' in ir else 2e-4
     for tag, grid in launches:
         plan.choose = lambda env_, ptrs, tag=tag, grid=grid: (plan.variants[tag], min(grid, 65536), 256)
