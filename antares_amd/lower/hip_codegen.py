@@ -908,8 +908,9 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         return vectors and mc['vec'][x] and (HM or (tensors[ld.name].dtype == 'float32' and mc['f' + x] is ld))
     mode = {x: ('kvec' if vector_ok(x, ld) else ('tr' if (vectors and mc['rowrun'][x]) else ('k' if mc['parts'][x][2] else 'rows')))
             for x, ld in (('a', la), ('b', lb))}
-    PT = TS + 32                                      # halves per k row of a tile staged as it lies, [k][row]: 64 bytes past a multiple of 256
-    CG = TS // 8                                      # 16-byte groups of rows in such a tile
+    PT = TS + 32                                      # elements per k row of a tile staged as it lies, [k][row]: its k rows start on different banks
+    VR = 16 if IM else 8                              # rows per 16-byte vector of it
+    CG = TS // VR                                     # 16-byte groups of rows in such a tile
     KP = BLOCK // CG                                  # k rows of it that one pass of the 256 threads covers
     VL = 16 // ITEMSIZE[tensors[la.name].dtype] if mode['a'] == 'kvec' else (16 // ITEMSIZE[tensors[lb.name].dtype] if mode['b'] == 'kvec' else VW)
     VPR = BK // VL                                    # vectors per row of a tile
@@ -975,6 +976,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           f'  __shared__ __attribute__((aligned(16))) {ET} __Bs[2][{BK * PT if mode["b"] == "tr" else TS * LD}];     // [column][k]',
           '  typedef short __s4 __attribute__((ext_vector_type(4)));',
           '  typedef __attribute__((address_space(3))) __s4 __lds_s4;',
+          '  typedef int __i2 __attribute__((ext_vector_type(2)));',
+          '  typedef __attribute__((address_space(3))) __i2 __lds_i2;',
           f'  __shared__ long long __am[{TS}], __bn[{TS}], __cm[{TS}], __cn[{TS}], __ak[2][{BK}], __bk[2][{BK}];'] + \
          [f'  __shared__ long long __xm{q}[{TS}], __xn{q}[{TS}];      // row and column part of the offsets into {ld.name} (read by the tail)'
           for q, (ld, _, _, _) in enumerate(extra)] + \
@@ -1029,8 +1032,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         if mode[x] == 'tr':
             # a lane owns 8 neighbouring rows (a whole vector: all inside the extents or all past them) and every KP-th k;
             # the last of them names the address, so that a group past the end re-reads the last whole vector
-            b += [f'    typedef {ct} __w{x} __attribute__((ext_vector_type(8)));',
-                  f'    const {ct}* __p{x} = {ld.name} + ({tab}[(__tid % {CG}) * 8 + 7] - 7);',
+            b += [f'    typedef {ct} __w{x} __attribute__((ext_vector_type({VR})));',
+                  f'    const {ct}* __p{x} = {ld.name} + ({tab}[(__tid % {CG}) * {VR} + {VR - 1}] - {VR - 1});',
                   f'    __w{x} __r{x}[{DEPTH}][{BK // KP}];']
             continue
         if mode[x] == 'k':
@@ -1078,7 +1081,7 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         if mode[x] == 'tr':
             for j in range(BK // KP):
                 b += [f'      {{ const int __ks = __tid / {CG} + {KP * j};',
-                      f'        *(__w{x}*)&{lds}[__buf][__ks * {PT} + (__tid % {CG}) * 8] = (long long)__kt * {BK} + __ks < __K ? __r{x}[__S][{j}] : (__w{x})(0); }}']
+                      f'        *(__w{x}*)&{lds}[__buf][__ks * {PT} + (__tid % {CG}) * {VR}] = (long long)__kt * {BK} + __ks < __K ? __r{x}[__S][{j}] : (__w{x})(0); }}']
             continue
         def inside(j, x=x):
             return f' && ((__g{x}[__S] >> {j}) & 1u)' if G[x] else ''
@@ -1099,6 +1102,11 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
             return f'          __{x}[__i] = *(const __f4*)&{lds}[__buf][({base} + 32 * __i) * {LD} + __g * {KG} + __kq];'
         # 16 lanes read a patch of 4 k x 16 rows and each receives the four k of one row; two patches, 4 k apart, make
         # the 8 consecutive k a lane supplies: k = (lane / 32) * 8 .. + 7, row = lane % 32 of the tile - as above
+        if IM:      # 16 lanes read a patch of 8 k x 16 rows (a lane supplies 8 bytes of one k) and each receives the 8 k of one row
+            at = f'&{lds}[__buf][(__g * 32 + __tq) * {PT} + {w} * {HALF} + 32 * __i + __tc]'
+            return (f'          {{ const __i2 __lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__lds_i2*)({at})), '
+                    f'__hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__lds_i2*)({at} + 8 * {PT}));\n'
+                    f'            __{x}[__i] = __builtin_bit_cast(__f4, __i4{{__lo[0], __lo[1], __hi[0], __hi[1]}}); }}')
         at = f'&{lds}[__buf][(__g * 16 + __tq) * {PT} + {w} * {HALF} + 32 * __i + __tc]'
         return (f'          {{ const __s4 __lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__lds_s4*)({at})), '
                 f'__hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__lds_s4*)({at} + 4 * {PT}));\n'
@@ -1114,7 +1122,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           '        #pragma unroll',
           f'        for (int __e = 0; __e < 16; ++__e) __acc[__i][__j][__e] = {ZERO};',
           f'    const int __row0 = __wm * {HALF} + (__lane & 31), __col0 = __wn * {HALF} + (__lane & 31), __kq = (__lane >> 5) * {VW};',
-          '    const int __tq = (__lane >> 5) * 8 + ((__lane & 15) >> 2), __tc = ((__lane & 31) >> 4) * 16 + (__lane & 3) * 4; (void)__tq; (void)__tc;',
+          ('    const int __tq = (__lane >> 5) * 16 + ((__lane & 15) >> 1), __tc = ((__lane & 31) >> 4) * 16 + (__lane & 1) * 8; (void)__tq; (void)__tc;' if IM else
+           '    const int __tq = (__lane >> 5) * 8 + ((__lane & 15) >> 2), __tc = ((__lane & 31) >> 4) * 16 + (__lane & 3) * 4; (void)__tq; (void)__tc;'),
           '    auto __multiply = [&](int __buf) {',
           '      #pragma unroll',
           f'      for (int __g = 0; __g < {BK // KG}; ++__g) {{',
@@ -1403,7 +1412,7 @@ def _matrix_contraction(st, tensors):
     for tag, ld, own in (('a', la, m_axes), ('b', lb, n_axes)):
         last = ld.args[-1]
         ext_own = dict(st.data_axes)[own[-1]]
-        rowrun[tag] = (half and not vec[tag] and not guards[tag] and not parts[tag][2] and last.kind == 'axis' and last.name == own[-1] and
+        rowrun[tag] = ((half or st.root.dtype == 'int32') and not vec[tag] and not guards[tag] and not parts[tag][2] and last.kind == 'axis' and last.name == own[-1] and
                        not any(own[-1] in _axes_of(a) for a in ld.args[:-1]) and tensors[ld.name].shape[-1] == ext_own)
         if rowrun[tag]:
             pitch[tag] = [ext_own]

@@ -876,6 +876,9 @@ def test_fp16_operands_stored_along_rows_are_staged_as_they_lie(autort, ir, inpu
      [(300, 200), (200, 260)]),
     ('output0[B, N, M] +=! input0[B, N, K].cast(`int32`) * input1[B, M, K].cast(`int32`)', ['input0=int8[B:2, N:256, K:4096]', 'input1=int8[B:2, M:192, K:4096]'],
      [(2, 256, 4096), (2, 192, 4096)]),
+    # the second operand stored along its columns, whole vectors of them: staged as it lies, transposed by ds_read_b64_tr_b8
+    ('output0[N, M] +=! input0[N, K].cast(`int32`) * input1[K, M].cast(`int32`)', ['input0=int8[N:200, K:160]', 'input1=int8[K:160, M:272]'],
+     [(200, 160), (160, 272)]),
 ])
 def test_int8_contractions_are_bit_exact_on_the_matrix_instructions(autort, ir, inputs, shapes):
     """An int32 sum of products of two int8 loads cast to int32 runs on v_mfma_i32_32x32x32_i8: exact products, exact
@@ -898,8 +901,8 @@ def test_int8_contractions_are_bit_exact_on_the_matrix_instructions(autort, ir, 
         assert np.array_equal(want, exact)
     M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
     for tag, side in (('matrix', 128), ('matrix64', 64), ('matrixv', 128), ('matrix64v', 64)):
-        if tag not in plan.variants or (tag.endswith('v') and shapes[0][-1] % plan.matrix['vec_width'][0]):
-            continue                # the vector kernels are launched for whole vectors of k only
+        if tag not in plan.variants or (tag.endswith('v') and not (plan._matrix_choice(env, {n: 0 for n in plan.args})[0] or '').endswith('v')):
+            continue                # the vector kernels are launched for whole vectors only
         blocks = ((M + side - 1) // side) * ((N + side - 1) // side) * B
         plan.choose = lambda env_, ptrs, tag=tag, blocks=blocks: (plan.variants[tag], blocks, 256)
         got = op(a.to(dev), b.to(dev))
