@@ -908,8 +908,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
         return vectors and mc['vec'][x] and (HM or (tensors[ld.name].dtype == 'float32' and mc['f' + x] is ld))
     mode = {x: ('kvec' if vector_ok(x, ld) else ('tr' if (vectors and mc['rowrun'][x]) else ('k' if mc['parts'][x][2] else 'rows')))
             for x, ld in (('a', la), ('b', lb))}
-    PT = TS + 32                                      # elements per k row of a tile staged as it lies, [k][row]: its k rows start on different banks
-    VR = 16 if IM else 8                              # rows per 16-byte vector of it
+    PT = TS + (32 if HM else 8)                       # elements per k row of a tile staged as it lies, [k][row]: the k rows a wavefront reads together start on different banks
+    VR = 16 if IM else (8 if HM else 4)               # rows per 16-byte vector of it
     CG = TS // VR                                     # 16-byte groups of rows in such a tile
     KP = BLOCK // CG                                  # k rows of it that one pass of the 256 threads covers
     VL = 16 // ITEMSIZE[tensors[la.name].dtype] if mode['a'] == 'kvec' else (16 // ITEMSIZE[tensors[lb.name].dtype] if mode['b'] == 'kvec' else VW)
@@ -1102,6 +1102,9 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
             return f'          __{x}[__i] = *(const __f4*)&{lds}[__buf][({base} + 32 * __i) * {LD} + __g * {KG} + __kq];'
         # 16 lanes read a patch of 4 k x 16 rows and each receives the four k of one row; two patches, 4 k apart, make
         # the 8 consecutive k a lane supplies: k = (lane / 32) * 8 .. + 7, row = lane % 32 of the tile - as above
+        if not HM:  # float32 needs no transposing read: four 4-byte reads, k = g * 8 + (lane / 32) * 4 + m for instruction m
+            at = f'{lds}[__buf][(__g * 8 + __kq + %d) * {PT} + {w} * {HALF} + 32 * __i + (__lane & 31)]'
+            return f'          __{x}[__i] = __f4{{' + ', '.join(at % m for m in range(4)) + '};'
         if IM:      # 16 lanes read a patch of 8 k x 16 rows (a lane supplies 8 bytes of one k) and each receives the 8 k of one row
             at = f'&{lds}[__buf][(__g * 32 + __tq) * {PT} + {w} * {HALF} + 32 * __i + __tc]'
             return (f'          {{ const __i2 __lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__lds_i2*)({at})), '
@@ -1412,7 +1415,8 @@ def _matrix_contraction(st, tensors):
     for tag, ld, own in (('a', la, m_axes), ('b', lb, n_axes)):
         last = ld.args[-1]
         ext_own = dict(st.data_axes)[own[-1]]
-        rowrun[tag] = ((half or st.root.dtype == 'int32') and not vec[tag] and not guards[tag] and not parts[tag][2] and last.kind == 'axis' and last.name == own[-1] and
+        plain32 = (fa if tag == 'a' else fb) is ld and tensors[ld.name].dtype == 'float32' and not half
+        rowrun[tag] = ((half or st.root.dtype == 'int32' or plain32) and not vec[tag] and not guards[tag] and not parts[tag][2] and last.kind == 'axis' and last.name == own[-1] and
                        not any(own[-1] in _axes_of(a) for a in ld.args[:-1]) and tensors[ld.name].shape[-1] == ext_own)
         if rowrun[tag]:
             pitch[tag] = [ext_own]

@@ -838,11 +838,16 @@ def test_contractions_with_few_output_tiles_are_cut_into_slices_of_k(autort, ir,
      [(96, 1000), (96, 520)]),
     ('output0[B, S, D] +=! input0[B, S, T].to(`float32`) * input1[B, T, D].to(`float32`)', ['input0=float16[B:3, S:300, T:80]', 'input1=float16[B:3, T:80, D:128]'],
      [(3, 300, 80), (3, 80, 128)]),
+    # float32: both operands along rows; the second one only, batched, k = 2.5 tiles of the big blocks
+    ('output0[N, M] +=! input0[K, N] * input1[K, M]', ['input0=float32[K:72, N:1000]', 'input1=float32[K:72, M:516]'], [(72, 1000), (72, 516)]),
+    ('output0[B, S, D] +=! input0[B, S, T] * input1[B, T, D]', ['input0=float32[B:3, S:300, T:40]', 'input1=float32[B:3, T:40, D:128]'],
+     [(3, 300, 40), (3, 40, 128)]),
 ])
-def test_fp16_operands_stored_along_rows_are_staged_as_they_lie(autort, ir, inputs, shapes):
-    """An fp16 operand whose neighbouring rows (columns) are neighbours in memory - `input1[K, M]` - is fetched in 16-byte
-    vectors of rows, staged in LDS as [k][row] and transposed on its way to the matrix instruction by
-    ds_read_b64_tr_b16; the result is that of the kernels that stage it row by row, and the oracle's."""
+def test_operands_stored_along_rows_are_staged_as_they_lie(autort, ir, inputs, shapes):
+    """An operand whose neighbouring rows (columns) are neighbours in memory - `input1[K, M]` - is fetched in 16-byte
+    vectors of rows and staged in LDS as [k][row]; fp16 tiles are transposed on their way to the matrix instruction by
+    ds_read_b64_tr_b16, float32 ones are read element by element.  The result is that of the kernels that stage it row
+    by row, bit for bit, and the oracle's."""
     from antares_amd.ir import parse_program
     from oracle.cpu_backend import CpuModule
     note(f'fp16 operands staged as they lie {ir} {shapes}')
@@ -853,10 +858,10 @@ def test_fp16_operands_stored_along_rows_are_staged_as_they_lie(autort, ir, inpu
     plan = op.plans_for(env)[-1]
     zero = {n: 0 for n in plan.args}
     assert plan.choose(env, zero)[0] in (plan.variants['matrixv'], plan.variants['matrix64v'])
-    odd = {k: (v + 4 if k in ('M', 'D') else v) for k, v in env.items()}          # a row length that is no whole number of vectors
+    odd = {k: (v + 2 if k in ('M', 'D') else v) for k, v in env.items()}          # a row length that is no whole number of vectors
     assert plan.choose(odd, zero)[0] in (plan.variants['matrix'], plan.variants['matrix64'])
     g = torch.Generator().manual_seed(len(ir))
-    a, b = [(torch.randn(shape, generator=g) * 0.5).half() for shape in shapes]
+    a, b = [(torch.randn(shape, generator=g) * 0.5).to(torch.float16 if 'float16' in inputs[0] else torch.float32) for shape in shapes]
     want = CpuModule(parse_program(ir, inputs), fast_math=False)(input0=a.numpy(), input1=b.numpy())['output0']
     M, N, B = (int(np.prod([e if isinstance(e, int) else env[e] for e in plan.matrix[k]])) for k in ('m', 'n', 'batch'))
     got = {}
