@@ -277,11 +277,19 @@ class KernelPlan:
                 return n % self.matrix['vec_width'][0] == 0
             if all(whole(p) for p in self.matrix.get('vec_pitch', [])):
                 v = 'v'
-        # ... and when the big tiles are not mostly padding: 64 columns in tiles of 128 multiply twice what they need,
-        # which costs more than the small tiles' lower rate (about three quarters of the big ones')
-        if big >= 192 and big <= MAX_GRID * 64 and ('matrix64' not in self.variants or small >= 3 * big):
+        # Which block size: the big blocks run in rounds - a compute unit holds one of them with float32 tiles, two with
+        # fp16 or int8 tiles, and a round takes as long whether it is full or not - while the small blocks share compute
+        # units and take time in proportion to their number, about a 900th of a round each (a 700th with fp16 tiles;
+        # measured on squares of 1664 to 4096 with k = 1024 - fp32 2176^2 145 us in big blocks, 104 in small ones, fp16 29
+        # against 36 - and on 3 x 3 convolutions of 25088 x 128 outputs).  Tiles
+        # that are mostly padding (64 columns in tiles of 128) count as whole blocks on both sides, which settles them.
+        half = self.matrix.get('half_tiles')
+        rounds = -(-big // (512 if half else 256))
+        if 'matrix64' in self.variants and 16 <= small <= MAX_GRID * 64 and small < (700 if half else 900) * rounds:
+            return 'matrix64' + v, small
+        if big >= 16 and big <= MAX_GRID * 64:
             return 'matrix' + v, big
-        if 'matrix64' in self.variants and small >= 16 and small <= MAX_GRID * 64:
+        if 'matrix64' in self.variants and 16 <= small <= MAX_GRID * 64:
             return 'matrix64' + v, small
         return None, 0
 
@@ -860,6 +868,7 @@ def lower_statement(st, graph, name: str, tail=None) -> Tuple[str, KernelPlan]:
             variants['matrix'], variants['matrix64'] = name + '_m', name + '_m64'
             ext = dict(st.data_axes + st.reduce_axes)
             plan.matrix = {key: [ext[a] for a in mc[key]] for key in ('m', 'n', 'batch', 'k')}
+            plan.matrix['half_tiles'] = bool(mc['half'])      # fp16 or int8 tiles: two of the big blocks fit a compute unit
             wide_ok = {t: mc['vec'][t] or mc['rowrun'][t] for t in ('a', 'b')}
             if wide_ok['a'] or wide_ok['b']:
                 src.append(_matrix_kernel(st, tensors, dims, args, written, name + '_mv', mc, vectors=True))
@@ -868,7 +877,8 @@ def lower_statement(st, graph, name: str, tail=None) -> Tuple[str, KernelPlan]:
                 wide = [ITEMSIZE[tensors[mc['l' + t].name].dtype] for t in ('a', 'b') if wide_ok[t]]
                 plan.matrix['vec_tensors'] = [mc['l' + t].name for t in ('a', 'b') if wide_ok[t]]
                 plan.matrix['vec_width'] = [16 // min(wide)]
-                plan.matrix['vec_pitch'] = [mc['pitch'][t] for t in ('a', 'b') if wide_ok[t]]     # row lengths, as dimensions to multiply
+                plan.matrix['vec_pitch'] = [mc['pitch'][t] for t in ('a', 'b') if wide_ok[t]] + \
+                    [mc['pitch'][t + '_run'] for t in ('a', 'b') if wide_ok[t] and t + '_run' in mc['pitch']]     # row and run lengths, as dimensions to multiply
 
     return '\n\n'.join(src), plan
 
@@ -1046,9 +1056,8 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
             b.append(f'    unsigned int __g{x}[{DEPTH}];              // bit j: element j of the set is inside its guards')
     b += ['    auto __load = [&](auto __set, int __buf, int __ktile) {', '      constexpr int __S = decltype(__set)::value; (void)__ktile;']
     for x, ktab_ in (('a', '__ak'), ('b', '__bk')):
-        if mode[x] == 'kvec':       # the k offset of a row of k is k itself; a vector past the end re-reads the row's first
-            b += [f'      {{ const long long __k0 = (long long)__ktile * {BK} + (__tid % {VPR}) * {VL};',
-                  f'        const long long __ko = __k0 + {VL} <= __K ? __k0 : 0;', '        #pragma unroll',
+        if mode[x] == 'kvec':       # a vector starts where its first k does (the table; k past the end wraps to valid ones, staged as zeros)
+            b += [f'      {{ const long long __ko = {ktab_}[__buf][(__tid % {VPR}) * {VL}];', '        #pragma unroll',
                   f'        for (int __j = 0; __j < {TS // RV}; ++__j) __r{x}[__S][__j] = *(const __v{x}*)(__p{x}[__j] + __ko); }}']
             continue
         if mode[x] == 'tr':
@@ -1405,6 +1414,15 @@ def _matrix_contraction(st, tensors):
                     all(d == red[k] for d, k in zip(tensors[ld.name].shape[-nk + 1:] if nk > 1 else [], k_axes[1:])) and
                     (tail[0].kind != 'axis' or tensors[ld.name].shape[-nk] == red[k_axes[0]]) and not guards[tag])
         pitch[tag] = list(tensors[ld.name].shape[-nk:])
+        # ... or at least its last index is the fastest reduce axis, bare (the channels of an image stored
+        # `[N, H, W, C]`): a vector is then a run of that axis, which the launcher wants in whole vectors, like the rows
+        if not vec[tag] and not guards[tag] and ld.args[-1].kind == 'axis' and ld.args[-1].name == k_axes[-1] and \
+                not any(k_axes[-1] in _axes_of(a) for a in ld.args[:-1]):
+            vec[tag] = True
+            pitch[tag] = [tensors[ld.name].shape[-1]]
+            runs = [red[k_axes[-1]]]
+            if runs != pitch[tag]:
+                pitch[tag + '_run'] = runs
     # The other way round, for fp16 tiles: an operand whose last index is its fastest row (column) axis, bare, over a
     # dimension of exactly that extent (`input1[K, M]` of a product, V of an attention) has neighbouring rows next to
     # each other in memory.  It is fetched in 16-byte vectors of rows, staged as it lies ([k][row]) and transposed on
@@ -1421,7 +1439,7 @@ def _matrix_contraction(st, tensors):
         if rowrun[tag]:
             pitch[tag] = [ext_own]
     return {'fa': fa, 'fb': fb, 'la': la, 'lb': lb, 'm': m_axes, 'n': n_axes, 'batch': batch, 'k': k_axes, 'parts': parts, 'vec': vec,
-            'guards': guards, 'pitch': pitch, 'rowrun': rowrun}
+            'guards': guards, 'pitch': pitch, 'rowrun': rowrun, 'half': half or st.root.dtype == 'int32'}
 
 
 def _tail_of(graph, i: int):

@@ -185,6 +185,14 @@ LOWERING_CASES = [
      ['input0=float32[N:512, K:8192]', 'input1=float32[M:512, K:8192]'], [(512, 8192), (512, 8192)], ('flop', 2 * 512 * 512 * 8192)),
     _conv(8, 64, 64, 56), _conv(32, 128, 128, 30), _conv(32, 128, 128, 28, pad=True), _conv(32, 128, 128, 28, 'float16'),
     _conv(32, 128, 128, 28, 'float16', pad=True), _conv(8, 512, 512, 9),
+    ('3x3 convolution float32, channels last, 32x30x30x128 -> 128 channels',
+     'output0[N, HO, WO, F] +=! input0[N, HO + KH, WO + KW, C] * input1[KH, KW, C, F] where HO in 28, WO in 28',
+     ['input0=float32[N:32, H:30, W:30, C:128]', 'input1=float32[KH:3, KW:3, C:128, F:128]'], [(32, 30, 30, 128), (3, 3, 128, 128)],
+     ('flop', 2 * 32 * 128 * 28 * 28 * 128 * 9)),
+    ('3x3 convolution float16, channels last, 32x30x30x128 -> 128 channels',
+     'output0[N, HO, WO, F] +=! input0[N, HO + KH, WO + KW, C].to(`float32`) * input1[KH, KW, C, F].to(`float32`) where HO in 28, WO in 28',
+     ['input0=float16[N:32, H:30, W:30, C:128]', 'input1=float16[KH:3, KW:3, C:128, F:128]'], [(32, 30, 30, 128), (3, 3, 128, 128)],
+     ('flop', 2 * 32 * 128 * 28 * 28 * 128 * 9)),
     ('depthwise 3x3 convolution 32x128x56x56', 'output0[N, C, HO, WO] +=! input0[N, C, HO + KH, WO + KW] * input1[C, KH, KW] where HO in 54, WO in 54',
      ['input0=float32[N:32, C:128, H:56, W:56]', 'input1=float32[C:128, KH:3, KW:3]'], [(32, 128, 56, 56), (128, 3, 3)], ('bytes', None)),
     ('2x2 max pooling 32x64x112x112', 'output0[N, C, HO, WO] >=! input0[N, C, HO * 2 + KH, WO * 2 + KW] where HO in 56, WO in 56, KH in 2, KW in 2',

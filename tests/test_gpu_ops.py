@@ -698,6 +698,12 @@ MATRIX_CASES = [
      ['input0=float16[N:5, C:20, H:30, W:30]', 'input1=float16[F:72, C:20, KH:3, KW:3]'], [(5, 20, 30, 30), (72, 20, 3, 3)]),
     ('output0[N, M] +=! input0[N, K + 5].when([K + 5 < 80], 0.0) * input1[K, M] where K in 80',
      ['input0=float32[N:1024, J:80]', 'input1=float32[K:80, M:1024]'], [(1024, 80), (80, 1024)]),
+    # channels last (image `[N, H, W, C]`, filter `[KH, KW, C, F]`): the image in 16-byte vectors of channels, the filter staged as it
+    # lies; the same with fp16 operands and 24 channels (k = 216: 6.75 tiles)
+    ('output0[N, HO, WO, F] +=! input0[N, HO + KH, WO + KW, C] * input1[KH, KW, C, F] where HO in 20, WO in 20',
+     ['input0=float32[N:5, H:22, W:22, C:16]', 'input1=float32[KH:3, KW:3, C:16, F:72]'], [(5, 22, 22, 16), (3, 3, 16, 72)]),
+    ('output0[N, HO, WO, F] +=! input0[N, HO + KH, WO + KW, C].to(`float32`) * input1[KH, KW, C, F].to(`float32`) where HO in 20, WO in 20',
+     ['input0=float16[N:5, H:22, W:22, C:24]', 'input1=float16[KH:3, KW:3, C:24, F:72]'], [(5, 22, 22, 24), (3, 3, 24, 72)]),
     # the guarded factor second: the filter's output channels are the rows, the padded image's positions the columns
     ('output0[F, N, HO, WO] +=! input1[F, C, KH, KW] * input0[N, C, HO + KH - 2, WO + KW - 2].when([HO + KH - 2 >= 0, HO + KH - 2 < 20, '
      'WO + KW - 2 >= 0, WO + KW - 2 < 24], 0.0) where HO in 20, WO in 24',

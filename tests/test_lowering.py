@@ -114,7 +114,10 @@ def test_a_padded_convolution_goes_to_the_matrix_kernels_with_its_guards_tabled(
     # 25088 rows x 64 columns: tiles of 128 columns would be half padding, the small tiles take it
     env = {'N': 8, 'C': 64, 'H': 56, 'W': 56, 'F': 64, 'KH': 3, 'KW': 3}
     assert plans[0]._matrix_choice(env, {n: 0 for n in plans[0].args}) == ('matrix64v', 392)
-    assert plans[0]._matrix_choice({**env, 'F': 128}, {n: 0 for n in plans[0].args}) == ('matrixv', 196)
+    # 196 big blocks would be one round that is three quarters full: the small ones fill the chip; 3136 big blocks are
+    # thirteen rounds of 256, less than 12544 small blocks at a 900th of a round each
+    assert plans[0]._matrix_choice({**env, 'F': 128}, {n: 0 for n in plans[0].args}) == ('matrix64v', 784)
+    assert plans[0]._matrix_choice({**env, 'N': 32, 'F': 512}, {n: 0 for n in plans[0].args}) == ('matrixv', 3136)
     assert plans[0]._matrix_choice(env, {**{n: 0 for n in plans[0].args}, 'input1': 4}) == ('matrix64', 392)
     assert len(compile_cached(src)) > 1000
     # a guard that mixes rows and k in a product, or reads a tensor, leaves the statement to the other variants
