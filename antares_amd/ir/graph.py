@@ -252,13 +252,21 @@ def bake_small_reduce_extents(graph: Graph, env: Dict[str, int], limit: int = 8)
 
 
 def _interval(e: Expr, extent) -> Optional[Tuple[int, int]]:
-    """[lowest, highest] value of an index expression made of axes, integer constants, + - and *; None for anything
-    else.  extent(axis name) -> int or None."""
+    """[lowest, highest] value of an index expression made of axes, their extents, integer constants, + - * and the
+    division of something non-negative by a positive constant; None for anything else.  extent(axis name) -> int or None."""
     if e.kind == 'const' and isinstance(e.value, int) and not isinstance(e.value, bool):
         return e.value, e.value
     if e.kind == 'axis':
         n = extent(e.name)
         return (0, n - 1) if n else None
+    if e.kind == 'axis_range':                      # `KH.val()`: the extent itself
+        n = extent(e.name)
+        return (n, n) if n else None
+    if e.kind == 'op' and e.name == '//' and len(e.args) == 2:     # a non-negative value divided by a positive constant
+        a, b = _interval(e.args[0], extent), _interval(e.args[1], extent)
+        if a is None or b is None or a[0] < 0 or b[0] != b[1] or b[0] <= 0:
+            return None
+        return a[0] // b[0], a[1] // b[0]
     if e.kind == 'cast' and e.dtype in ('int32', 'int64'):
         return _interval(e.args[0], extent)
     if e.kind == 'op' and e.name in ('+', '-', '*') and len(e.args) == 2:

@@ -974,6 +974,33 @@ def test_a_map_behind_a_reduction_is_applied_at_its_stores(autort, ir, inputs, s
         assert got.shape == want.shape and np.allclose(got, want, rtol=tol, atol=tol), (tag, np.abs(got - want).max())
 
 
+def test_one_operator_called_at_several_sizes_gets_the_rewrites_of_each(autort):
+    """A padded convolution with bias and ReLU exported once with named dimensions and called with three batch sizes and
+    two filter sizes: every call finds (or builds) the kernels of its own dimension values - filter size written in,
+    operand padded by a statement in front, tail applied at the stores - and gives torch's result."""
+    note('padded conv + bias + relu at several sizes through one operator')
+    dev = autort.device()
+    ir = ('conv[N, F, HO, WO] +=! input0[N, C, HO + KH - KH.val() / 2, WO + KW - KW.val() / 2].when([HO + KH - KH.val() / 2 >= 0, '
+          'HO + KH - KH.val() / 2 < 24, WO + KW - KW.val() / 2 >= 0, WO + KW - KW.val() / 2 < 24], 0.0) * input1[F, C, KH, KW] where HO in 24, WO in 24; '
+          'output0[N, F, HO, WO] = (conv[N, F, HO, WO] + input2[F]).call(`max`, [0.0])')
+    op = autort.export(ir=ir, inputs=['input0=float32[N:4, C:16, H:24, W:24]', 'input1=float32[F:64, C:16, KH:3, KW:3]', 'input2=float32[F:64]'],
+                       name='conv_bias_relu_sizes')
+    g = torch.Generator().manual_seed(5)
+    seen = set()
+    for n, k in ((4, 3), (2, 3), (7, 5), (4, 3)):
+        x, w, b = torch.randn(n, 16, 24, 24, generator=g), torch.randn(64, 16, k, k, generator=g) * 0.1, torch.randn(64, generator=g)
+        got = op(x.to(dev), w.to(dev), b.to(dev)).cpu()
+        want = torch.relu(torch.nn.functional.conv2d(x.double(), w.double(), b.double(), padding=k // 2)).float()
+        assert got.shape == want.shape and torch.allclose(got, want, rtol=1e-4, atol=1e-3), (n, k, (got - want).abs().max())
+        seen.add((n, k))
+        assert len(op._variants) == len(seen)
+    env = {'N': 7, 'C': 16, 'H': 24, 'W': 24, 'F': 64, 'KH': 5, 'KW': 5}
+    plans = op.plans_for(env)
+    # the copy padded by two on each side, then the contraction with the tail at its stores (the map's own plan is not launched)
+    assert [p.output for p in plans] == ['input0__pad', 'output0', 'output0'] and plans[1].covers == 2 and plans[1].matrix is not None
+    assert dict(plans[1].reduce_axes)['KH'] == 5
+
+
 ROW_GROUP_CASES = [
     # program, inputs, shapes, does the row kernel run at these extents
     ('temp0[N] >=! input0[N, C]; temp1[N] +=! (input0[N, C] - temp0[N]).call(`exp`); '
