@@ -179,6 +179,10 @@ LOWERING_CASES = [
      ['input0=float16[N:2048, K:2048]', 'input1=float16[K:2048, M:2048]'], [(2048, 2048), (2048, 2048)], ('flop', 2 * 2048 ** 3)),
     ('int8 A B^T into int32 4096^3', 'output0[N, M] +=! input0[N, K].cast(`int32`) * input1[M, K].cast(`int32`)',
      ['input0=int8[N:4096, K:4096]', 'input1=int8[M:4096, K:4096]'], [(4096, 4096), (4096, 4096)], ('flop', 2 * 4096 ** 3)),
+    ('attention scores: 256 fp16 products of 1024 x 1024 x 128 into float32 (a 1 GiB result)',
+     'output0[B, H, S, T] +=! input0[B, H, S, D].to(`float32`) * input1[B, H, T, D].to(`float32`)',
+     ['input0=float16[B:8, H:32, S:1024, D:128]', 'input1=float16[B:8, H:32, T:1024, D:128]'], [(8, 32, 1024, 128), (8, 32, 1024, 128)],
+     ('bytes', None)),
     ('batched fp32 product 8 x 512^3', 'output0[B, N, M] +=! input0[B, N, K] * input1[B, K, M]',
      ['input0=float32[B:8, N:512, K:512]', 'input1=float32[B:8, K:512, M:512]'], [(8, 512, 512), (8, 512, 512)], ('flop', 2 * 8 * 512 ** 3)),
     ('fp32 A B^T 512x512x8192 (sliced along k)', 'output0[N, M] +=! input0[N, K] * input1[M, K]',
