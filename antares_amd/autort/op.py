@@ -197,6 +197,8 @@ class ExportedOp:
             g = bake_small_reduce_extents(self.lowered, env) if self.fused.dims else self.lowered
             g = pad_guarded_factors(g, env) if self.fused.dims else g
             g = split_wide_reductions(g, env, wanted=contraction_slices(g.tensors)) if self.fused.dims and not in_rows else g
+            if g is not self.lowered:      # kernels of this call's own anyway: every reduce extent a constant (divisions by constants)
+                g = bake_small_reduce_extents(g, env, limit=1 << 30)
             if g is self.lowered:
                 v = {'graph': self.lowered, 'plans': self.plans, 'module': None, 'source': None}
             else:
