@@ -204,8 +204,9 @@ class ExportedOp:
             else:
                 source, plans = lower_graph(g, prefix='autort_' + _ident(self.name) + '_s' + '_'.join(str(k) for k in key))
                 v = {'graph': g, 'plans': plans, 'module': None, 'source': source}
-            if len(self._variants) < 64:
-                self._variants[key] = v
+            if len(self._variants) >= 64:          # the oldest set of values goes (its code object stays in the cache on disk)
+                self._variants.pop(next(iter(self._variants)))
+            self._variants[key] = v
         if v['module'] is None:
             v['module'] = self._load() if v['source'] is None else capi.Module(compile_cached(v['source']))
         return v
