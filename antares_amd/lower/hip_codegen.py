@@ -1004,18 +1004,18 @@ def _matrix_kernel(st, tensors, dims, args, written, sym: str, mc, TS: int = 128
           '  const int __tid = threadIdx.x, __lane = __tid & 63, __wave = __tid >> 6, __wm = __wave >> 1, __wn = __wave & 1;',
           '  for (long long __blk = blockIdx.x; __blk < __tiles * __B; __blk += gridDim.x) {',
           '    const long long __t0 = __blk % __tiles, __tm = __t0 / __tn_n, __tn = __t0 % __tn_n;']
-    b += decompose('__blk / __tiles', mc['batch'], '    ')
+    b += _decompose('__blk / __tiles', [(a, None) for a in mc['batch']], '    ', '__B', tmp='__q') if mc['batch'] else []
     b += [f'    if (__tid < {TS}) {{                            // row offsets of the first operand and of the output',
           f'      long long __row = __tm * {TS} + __tid;',
           '      if (__row >= __M) __row = __M - 1;']
-    b += decompose('__row', mc['m'], '      ')
+    b += _decompose('__row', [(a, None) for a in mc['m']], '      ', '__M', tmp='__q')       # 32-bit divisions whenever the count fits
     b += [f'      __xm{q}[__tid] = {rowpart};' for q, (_, rowpart, _, _) in enumerate(extra)]
     b += [f'      __gma[{c}][__tid] = {g[0]};' for c, g in enumerate(GV['a'])]
     b += [f'      __am[__tid] = {mc["parts"]["a"][0]};', f'      __cm[__tid] = {rows_of_out};',
           f'    }} else if (__tid < {2 * TS}) {{                  // column offsets of the second operand and of the output',
           f'      long long __colq = __tn * {TS} + (__tid - {TS});',
           '      if (__colq >= __N) __colq = __N - 1;']
-    b += decompose('__colq', mc['n'], '      ')
+    b += _decompose('__colq', [(a, None) for a in mc['n']], '      ', '__N', tmp='__q')
     b += [f'      __xn{q}[__tid - {TS}] = {colpart};' for q, (_, _, colpart, _) in enumerate(extra)]
     b += [f'      __gmb[{c}][__tid - {TS}] = {g[0]};' for c, g in enumerate(GV['b'])]
     b += [f'      __bn[__tid - {TS}] = {mc["parts"]["b"][0]};', f'      __cn[__tid - {TS}] = {cols_of_out};',
