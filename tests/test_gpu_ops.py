@@ -920,6 +920,27 @@ def test_int8_contractions_are_bit_exact_on_the_matrix_instructions(autort, ir, 
         assert got.dtype == torch.int32 and np.array_equal(got.cpu().numpy(), exact), tag
 
 
+@pytest.mark.parametrize('in_kernel', [False, True])
+def test_int8_padded_convolution_is_bit_exact(autort, monkeypatch, in_kernel):
+    """A zero-padded 3 x 3 convolution of int8 images and filters into int32 on v_mfma_i32_32x32x32_i8, with the image
+    copied into a padded tensor first and with the conditions evaluated in the contraction: torch's integers both ways."""
+    note(f'int8 padded convolution, guards {"in the kernel" if in_kernel else "in a padded copy"}')
+    dev = autort.device()
+    if in_kernel:
+        monkeypatch.setattr('antares_amd.autort.op.pad_guarded_factors', lambda graph, env=None: graph)
+    ir = ('output0[N, F, HO, WO] +=! input0[N, C, HO + KH - 1, WO + KW - 1].cast(`int32`).when([HO + KH - 1 >= 0, HO + KH - 1 < 20, '
+          'WO + KW - 1 >= 0, WO + KW - 1 < 20], 0) * input1[F, C, KH, KW].cast(`int32`) where HO in 20, WO in 20')
+    op = autort.export(ir=ir, inputs=['input0=int8[N:3, C:24, H:20, W:20]', 'input1=int8[F:72, C:24, KH:3, KW:3]'], name=f'conv_i8_{int(in_kernel)}')
+    env = {'N': 3, 'C': 24, 'H': 20, 'W': 20, 'F': 72, 'KH': 3, 'KW': 3}
+    plans = op.plans_for(env)
+    assert len(plans) == (1 if in_kernel else 2) and plans[-1].matrix is not None and plans[-1].matrix['half_tiles']
+    g = torch.Generator().manual_seed(9)
+    x, w = torch.randint(-128, 128, (3, 24, 20, 20), generator=g, dtype=torch.int8), torch.randint(-128, 128, (72, 24, 3, 3), generator=g, dtype=torch.int8)
+    want = torch.nn.functional.conv2d(x.double(), w.double(), padding=1).to(torch.int32)        # sums below 2^53: exact
+    got = op(x.to(dev), w.to(dev)).cpu()
+    assert got.dtype == torch.int32 and torch.equal(got, want)
+
+
 TAIL_CASES = [
     # AntaresIR.md:248-250 (ConvBiasRelu tail fusion); a product with a scaled result, a per-column and a per-element
     # term under a tanh; a float16 result of a float32 sum; a column-wise maximum with a conditional store behind it
