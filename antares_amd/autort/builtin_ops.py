@@ -312,6 +312,86 @@ class GemvW4Fused:
         return out
 
 
+class W4Prepack:
+    """``w4_prepack(qweight[K/2, N], scales[K/128, N], qzeros[K/128, N/2]) -> packed``: the one-time repacking of an
+    int4 matrix for ``gemv_w4p`` - tiles of 16 columns over all of K stored contiguously, in the order the kernel's
+    wavefronts read them (the load-time weight preparation of samples/05_llama2_7b_int4.py:34-66).  ``packed`` is a
+    uint8 tensor that remembers K and N (``packed.w4_shape``)."""
+    name = 'w4_prepack'
+
+    def __call__(self, qweight, scales, qzeros, out=None, extra=None):
+        K, N = qweight.shape[0] * 2, qweight.shape[1]
+        if qweight.dtype != torch.uint8 or qzeros.dtype != torch.uint8 or scales.dtype != torch.float16:
+            raise TypeError('w4_prepack: qweight and qzeros must be uint8, scales float16')
+        if scales.shape != (K // 128, N) or qzeros.shape != (K // 128, N // 2):
+            raise ValueError('w4_prepack: operand shapes do not match K, N')
+        nbytes = capi.lib().art_w4_prepack_bytes(K, N)
+        if nbytes == 0:
+            raise ValueError(f'w4_prepack: unsupported shape K={K} N={N} (K % 128 == 0, K <= 16384, N % 16 == 0)')
+        if out is None:
+            out = torch.empty(nbytes, dtype=torch.uint8, device=qweight.device)
+        elif out.dtype != torch.uint8 or out.numel() != nbytes or not out.is_contiguous():
+            raise TypeError(f'w4_prepack: out must be a contiguous uint8 tensor of {nbytes} bytes')
+        for t in (qweight, scales, qzeros):
+            if not t.is_contiguous():
+                raise ValueError('w4_prepack: operands must be contiguous')
+        _require_cuda(qweight, scales, qzeros, out)
+        capi.check(capi.lib().art_w4_prepack(c_void_p(qweight.data_ptr()), c_void_p(scales.data_ptr()), c_void_p(qzeros.data_ptr()),
+                                            c_void_p(out.data_ptr()), K, N, c_void_p(current_stream_handle())))
+        out.w4_shape = (K, N)
+        return out
+
+
+class GemvW4Packed:
+    """``gemv_w4p(x[K], packed, out=None, norm_weight=None, residual=None, eps=1e-5, swiglu_out=False, shape=None)``:
+    the int4 GEMV over weights repacked by ``w4_prepack`` - one block per 16 columns over all of K, no K-splits.
+    ``norm_weight``: RMSNorm of x folded in; ``residual``: added to the rounded product (``out`` may be the residual);
+    ``swiglu_out``: the matrix holds gate and up columns interleaved in blocks of 8 (``interleave_gate_up``) and
+    ``out[N/2]`` receives fp16(silu(gate) * up).  ``shape`` = (K, N) when ``packed`` does not carry ``w4_shape``."""
+    name = 'gemv_w4p'
+
+    def __call__(self, x, packed, out=None, norm_weight=None, residual=None, eps=RMS_EPS, swiglu_out=False, shape=None, extra=None):
+        K, N = shape if shape is not None else getattr(packed, 'w4_shape', (None, None))
+        if K is None:
+            raise ValueError('gemv_w4p: pass shape=(K, N) or a tensor returned by w4_prepack')
+        if x.dtype != torch.float16 or x.numel() != K:
+            raise TypeError(f'gemv_w4p: x must be float16 of {K} values')
+        if packed.dtype != torch.uint8 or packed.numel() != capi.lib().art_w4_prepack_bytes(K, N):
+            raise ValueError('gemv_w4p: packed does not have the size of a repacked K x N matrix')
+        n_out = N // 2 if swiglu_out else N
+        if out is None:
+            out = torch.empty(n_out, dtype=torch.float16, device=x.device)
+        elif out.dtype != torch.float16 or out.numel() != n_out:
+            raise TypeError(f'gemv_w4p: out must be float16 of {n_out} values')
+        tensors = [x, packed, out]
+        for t, what, n in ((norm_weight, 'norm_weight', K), (residual, 'residual', N)):
+            if t is not None:
+                if t.dtype != torch.float16 or t.numel() != n:
+                    raise TypeError(f'gemv_w4p: {what} must be float16 of {n} values')
+                tensors.append(t)
+        _require_cuda(*tensors)
+        capi.check(capi.lib().art_gemv_w4p(c_void_p(x.data_ptr()), c_void_p(packed.data_ptr()), c_void_p(out.data_ptr()), K, N,
+                                          _ptr_or_null(norm_weight), float(eps), _ptr_or_null(residual), int(bool(swiglu_out)),
+                                          c_void_p(current_stream_handle())))
+        return out
+
+
+def interleave_gate_up(gate: dict, up: dict) -> dict:
+    """Columns of two int4 matrices of the same shape (dicts of qweight / scales / qzeros) interleaved in blocks of 8:
+    g0..g7 u0..u7 g8..g15 u8..u15 ... - the column order ``gemv_w4p(swiglu_out=True)`` expects, so that a block of 16
+    columns holds 8 gate columns and the matching 8 up columns."""
+    def mix(a, b, cols_per_elem):
+        blk = 8 // cols_per_elem          # elements of the last axis that make 8 columns
+        rows, n = a.shape
+        return torch.stack([a.view(rows, n // blk, blk), b.view(rows, n // blk, blk)], dim=2).reshape(rows, 2 * n).contiguous()
+    return {'qweight': mix(gate['qweight'], up['qweight'], 1), 'scales': mix(gate['scales'], up['scales'], 1),
+            'qzeros': mix(gate['qzeros'], up['qzeros'], 2)}
+
+
+builtin('w4_prepack')(lambda: W4Prepack())
+builtin('gemv_w4p')(lambda: GemvW4Packed())
+
+
 class AttentionRope:
     """``attention_rope_f16(qkv[3*H*D], inv_freq[D], key_cache[S,H*D], val_cache[S,H*D], att_f[1], out[H,D], extra=[pos_tensor])``:
     rotary embedding of q and k, both cache writes and the attention over rows 0..pos, one launch per layer."""

@@ -94,9 +94,18 @@ class LlamaInt4Decoder:
     """One-token-per-step decoder.  ``step()`` enqueues a whole forward pass on the
     current stream; ``capture()`` records it once in a HIP graph."""
 
-    def __init__(self, cfg: LlamaConfig, weights: Dict[str, object], device=None, fused: bool = True, att_parts: int = 8):
+    def __init__(self, cfg: LlamaConfig, weights: Dict[str, object], device=None, fused: bool = True, att_parts: int = 8,
+                 packed: Optional[bool] = None):
+        """``packed`` (default: with ``fused``): the projections whose input needs no merging (q|k|v, gate|up, down,
+        lm_head) run over weights repacked once here (``autort.ops.w4_prepack``, the counterpart of the sample's
+        load-time repacking, samples/05_llama2_7b_int4.py:34-66) with ``autort.ops.gemv_w4p``: one block per 16
+        columns over all of K, no K-splits.  The benchmark-format tensors stay for the o-projection (which merges the
+        split attention's records while it loads x) and for the batched passes of ``prefill``."""
         import autort
         self.fused = fused
+        self.packed = fused if packed is None else bool(packed)
+        if self.packed and not fused:
+            raise ValueError('the packed projections come with the fused decoder')
         self.att_parts = att_parts if fused else 1     # blocks per head in the decode attention (1 = unsplit)
         self.autort = autort
         self.cfg = cfg
@@ -110,7 +119,8 @@ class LlamaInt4Decoder:
         self.inv_freq = torch.cat([inv, inv]).view(D).to(self.dev)
         self.att_f = torch.tensor([1 / math.sqrt(D)], dtype=torch.float32, device=self.dev)
         # sum(x^2) of the residual stream, handed from the projection that writes it to the one that normalises it
-        self.hand_sumsq = fused and d <= 8192
+        # (the packed projections own all of K and sum the squares of x themselves)
+        self.hand_sumsq = fused and d <= 8192 and not self.packed
         self.sumsq = torch.zeros(2, 256, dtype=torch.int64, device=self.dev)
         # device-side step state
         self.token = torch.zeros(1, dtype=torch.int32, device=self.dev)
@@ -131,6 +141,28 @@ class LlamaInt4Decoder:
         self._prefill_graphs: Dict[int, tuple] = {}                  # prompt length -> (recorded pass, its token buffer)
         self._stream: Optional[torch.cuda.Stream] = None             # the one side stream recordings are made on
         self._ops()
+        self.pw: Dict[str, object] = {}
+        if self.packed:
+            self._prepack()
+
+    def _prepack(self):
+        """One-time repacking of the matrices the packed GEMV reads; gate and up are interleaved in blocks of 8
+        columns first, so that a block of the GEMV holds matching gate / up columns and can apply SwiGLU itself."""
+        from .autort.builtin_ops import interleave_gate_up
+        pack = self.autort.ops.w4_prepack
+        F = self.cfg.ffn
+
+        def packed(lin):
+            return pack(lin['qweight'], lin['scales'], lin['qzeros'])
+        layers = []
+        for lw in self.w['layers']:
+            gu = lw['gate_up']
+            gate = {'qweight': gu['qweight'][:, :F].contiguous(), 'scales': gu['scales'][:, :F].contiguous(),
+                    'qzeros': gu['qzeros'][:, :F // 2].contiguous()}
+            up = {'qweight': gu['qweight'][:, F:].contiguous(), 'scales': gu['scales'][:, F:].contiguous(),
+                  'qzeros': gu['qzeros'][:, F // 2:].contiguous()}
+            layers.append({'qkv': packed(lw['qkv']), 'gate_up': packed(interleave_gate_up(gate, up)), 'down': packed(lw['down'])})
+        self.pw = {'layers': layers, 'lm_head': packed(self.w['lm_head'])}
 
     def _ops(self):
         a = self.autort
@@ -159,6 +191,8 @@ class LlamaInt4Decoder:
         gemv = ops.gemv_w4a16_fused
         if embed:
             self.embed(self.w['embed'], self.token, out=self.x)
+        if self.packed:
+            return self._step_packed()
         # The projections that write the residual stream (o, down) leave sum(x^2) of what they wrote in a buffer, and the
         # projection that normalises the stream next reads it there instead of re-reading x in every block.  Two
         # buffers alternate: a writer adds into one and zeroes the other for the writer after it.  Only the first
@@ -185,6 +219,28 @@ class LlamaInt4Decoder:
         h = self.w['lm_head']
         gemv(self.x, h['qweight'], h['scales'], h['qzeros'], self.logits, norm_weight=self.w['final_norm'], eps=cfg.rms_eps,
              sumsq_in=after_down)
+        return self.logits
+
+    def _step_packed(self) -> torch.Tensor:
+        """The fused step over repacked weights: q|k|v (RMSNorm folded in), attention, o (merge + residual, benchmark
+        layout), gate|up (RMSNorm in, SwiGLU out), down (residual), five launches per layer."""
+        cfg, ops = self.cfg, self.autort.ops
+        d, F = cfg.dim, cfg.ffn
+        gemv = ops.gemv_w4p
+        for l, (lw, pw) in enumerate(zip(self.w['layers'], self.pw['layers'])):
+            o = lw['o']
+            gemv(self.x, pw['qkv'], self.qkv, norm_weight=lw['att_norm'], eps=cfg.rms_eps, shape=(d, 3 * d))
+            if self.att_parts > 1:
+                ops.attention_rope_split_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f,
+                                             self.att_partial, extra=[self.pos])
+                ops.gemv_w4a16_attn(self.att_partial, o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
+            else:
+                ops.attention_rope_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f, self.att,
+                                       extra=[self.pos])
+                ops.gemv_w4a16_fused(self.att.view(-1), o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
+            gemv(self.x, pw['gate_up'], self.hb, norm_weight=lw['ffn_norm'], eps=cfg.rms_eps, swiglu_out=True, shape=(d, 2 * F))
+            gemv(self.hb, pw['down'], self.x, residual=self.x, shape=(F, d))
+        gemv(self.x, self.pw['lm_head'], self.logits, norm_weight=self.w['final_norm'], eps=cfg.rms_eps, shape=(d, cfg.vocab))
         return self.logits
 
     def step_plain(self) -> torch.Tensor:

@@ -379,6 +379,30 @@ def bench_gemv(torch, autort, capi, workloads, K, N, M, steps, warmup, seed, lay
             'sec_per_step': sec, 'us_per_launch': per_launch * 1e6, 'gbps': by / per_launch / 1e9}
 
 
+def bench_gemv_packed(torch, autort, capi, workloads, K, N, steps, warmup, seed, layers=LAYERS):
+    """The same GEMV over weights repacked once by `autort.ops.w4_prepack` (tiles of 16 columns over all of K, one block
+    per tile, no K-splits), timed exactly as `bench_gemv`: `layers` distinct weight sets per replayed graph.  The
+    algorithmic bytes are those of the benchmark format (the packed form is 0.75 % larger)."""
+    dev = autort.device()
+    p = workloads.w4_problem(seed, 1, K, N)
+    packs = []
+    for l in range(layers):
+        qw, sc, qz = (torch.roll(p[k], l, 0).to(dev) for k in ('qweight', 'scales', 'qzeros'))
+        packs.append(autort.ops.w4_prepack(qw, sc, qz))
+        del qw, sc, qz
+    x = p['x'].to(dev).view(-1)
+    ys = [torch.empty(N, dtype=torch.float16, device=dev) for _ in range(layers)]
+
+    def one_pass():
+        for pk, y in zip(packs, ys):
+            autort.ops.gemv_w4p(x, pk, y, shape=(K, N))
+    sec = time_graph(torch, capi, one_pass, steps, warmup) / layers
+    by = workloads.w4_bytes(1, K, N)
+    return {'workload': f'int4 g128 GEMV M=1 K={K} N={N}, weights repacked once (16 columns x K per block)',
+            'us_per_launch': round(sec * 1e6, 3), 'gbps': round(by / sec / 1e9, 1), 'roofline_frac': round(by / sec / 1e9 / HBM_PEAK_GBPS, 4),
+            'packed_bytes': int(packs[0].numel())}
+
+
 def bench_gemm_f16(torch, autort, capi, workloads, steps, warmup, seed, n):
     from antares_amd.autort import patterns
     dev = autort.device()
@@ -449,10 +473,23 @@ def bench_decode(torch, autort, capi, seed, prompt_len=128, decode_steps=256, cp
     prompt = torch.randint(0, cfg.vocab, (prompt_len,), generator=g, dtype=torch.int64).to(torch.int32)
     prompt_dev = prompt.to(dec.dev)
     dec.capture(greedy=True, prompt=prompt_dev)
+    stream = side_stream(torch)
+    # the first greedy tokens of the replayed graph, to be compared with the eager 13-launch form further down
+    check_steps = 8
     dec.key_cache.zero_()
     dec.val_cache.zero_()
     dec.reset(int(prompt[0]), 0)
-    stream = side_stream(torch)
+    graph_tokens = []
+    with torch.cuda.stream(stream):
+        for _ in range(prompt_len - 1):
+            dec.graph.replay()
+        for _ in range(check_steps):
+            dec.graph.replay()
+            stream.synchronize()
+            graph_tokens.append(int(dec.token.item()))
+    dec.key_cache.zero_()
+    dec.val_cache.zero_()
+    dec.reset(int(prompt[0]), 0)
     tokens = []
     with torch.cuda.stream(stream):
         for _ in range(prompt_len - 1):          # positions 0 .. prompt_len-2 consume the prompt
@@ -480,7 +517,21 @@ def bench_decode(torch, autort, capi, seed, prompt_len=128, decode_steps=256, cp
     dec.prefill(prompt_dev)
     torch.cuda.synchronize()
     prefill_ms = (time.perf_counter() - t0) * 1e3
+    # the same prompt and the first greedy steps through the decoder that mirrors the sample line by line (thirteen
+    # launches per layer, one Python call per operator, no graph, split-K kernels over the benchmark layout)
+    plain = LlamaInt4Decoder(cfg, weights, fused=False)
+    plain.reset(int(prompt[0]), 0)
+    eager_tokens = []
+    for i in range(prompt_len - 1 + check_steps):
+        plain.step()
+        plain.advance(prompt_dev)
+        if i >= prompt_len - 1:
+            eager_tokens.append(int(plain.token.item()))
+    del plain
     out = {'workload': f'Llama-2-7B-shaped int4 decode, {cfg.n_layers} layers, batch 1, prompt {prompt_len} + {decode_steps} greedy steps',
+           'projections': 'q|k|v, gate|up, down, lm_head over weights repacked once (16 columns x K per block); o over the benchmark layout'
+           if dec.packed else 'benchmark layout, split-K',
+           'greedy_tokens_first_8': {'replayed_graph': graph_tokens, 'eager_13_launch_form': eager_tokens, 'equal': graph_tokens == eager_tokens},
            'tokens_per_s': round(1.0 / sec_per_token, 2), 'ms_per_token': round(sec_per_token * 1e3, 4),
            'weight_bytes_per_token': cfg.weight_bytes_per_token(), 'mean_kv_bytes_per_token': int(kv_bytes),
            'hbm_gbps': round(bytes_per_token / sec_per_token / 1e9, 1),
@@ -633,7 +684,13 @@ def main():
         result['roofline']['same_tensors_every_launch'] = {
             'us_per_launch': round(same['us_per_launch'], 3), 'algorithmic_gbps': round(same['gbps'], 1),
             'note': 'weights served by the caches; not an HBM rate'}
+        # the headline shape over weights repacked once (layout named in the row): reported beside the headline, which
+        # stays on the benchmark's [K/2, N] layout
+        result['roofline']['repacked_weights'] = bench_gemv_packed(torch, autort, capi, workloads, K, N, args.steps, args.warmup, args.seed)
         extra = []
+        for (k, n) in [(4096, 4096), (11008, 4096), (4096, 32000)]:
+            extra.append(bench_gemv_packed(torch, autort, capi, workloads, k, n, max(10, args.steps // 2), args.warmup, args.seed,
+                                           layers=32 if n < 32000 else 8))
         for (k, n) in [(4096, 4096), (11008, 4096), (4096, 32000)]:
             r = bench_gemv(torch, autort, capi, workloads, k, n, 1, max(10, args.steps // 2), args.warmup, args.seed,
                            layers=32 if n < 32000 else 8)

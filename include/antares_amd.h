@@ -218,6 +218,27 @@ int art_gemv_w4a16_fused_sumsq(const void* x_dev, const void* qweight_dev, const
                                int swiglu_input, const void* sumsq_in_dev, void* sumsq_out_dev, void* sumsq_clear_dev,
                                void* stream);
 
+/* The int4 GEMV (M = 1) over weights repacked once, when they are loaded - as the reference repacks its checkpoint
+ * when it loads it (samples/05_llama2_7b_int4.py:34-66).  The packed form stores a tile of 16 columns over all of K
+ * contiguously (records of 1024 values of k: weights in the order a wavefront reads them, then the scales and zero
+ * points of the record's 8 groups), so one block owns its columns over the whole of K: no K-splits, no atomics,
+ * no workspace.  Same arithmetic as art_gemv_w4a16 (fp32 accumulation in another order).  K % 128 == 0, K <= 16384,
+ * N % 16 == 0.
+ *   art_w4_prepack_bytes: size of the packed form (0 for a shape that is not supported).
+ *   art_w4_prepack:       qweight / scales / qzeros as for art_gemv_w4a16 -> packed_dev (256-byte aligned).
+ *   art_gemv_w4p:         y = x @ dequant(W), with the operators around a projection folded in as in
+ *                         art_gemv_w4a16_fused: norm_weight_dev != NULL normalises x first (RMSNorm, lines :128-131),
+ *                         residual_dev != NULL adds it to the rounded product (lines :168,:173; may alias y), and
+ *                         swiglu_out != 0 takes columns 16t..16t+7 of the matrix as gate columns and 16t+8..16t+15
+ *                         as the matching up columns and writes y[8t + j] = fp16(silu(gate) * up) (line :171; N/2
+ *                         outputs; the caller interleaves the two matrices in blocks of 8 columns before packing).
+ * Replaces the kernel the reference generates from samples/05_llama2_7b_int4.py:135-144. */
+size_t art_w4_prepack_bytes(int K, int N);
+int art_w4_prepack(const void* qweight_dev, const void* scales_dev, const void* qzeros_dev, void* packed_dev, int K, int N,
+                   void* stream);
+int art_gemv_w4p(const void* x_dev, const void* packed_dev, void* y_dev, int K, int N, const void* norm_weight_dev, float eps,
+                 const void* residual_dev, int swiglu_out, void* stream);
+
 /* The reference's own weight format (samples/05_llama2_7b_int4.py:135-139):
  * qweight int32 [K/8,N], eight nibbles per word along K (least significant
  * first), zero point fixed at 8, scales fp32 or fp16 [K/128,N], x and y fp32
