@@ -191,6 +191,8 @@ class ExportedOp:
         (pad_guarded_factors), which need their own kernels."""
         key = tuple(env[d] for d in self.fused.dim_names)
         v = self._variants.get(key)
+        if v is not None and len(self._variants) > 1:
+            self._variants[key] = self._variants.pop(key)      # most recently used last
         if v is None:
             # rows that one row kernel reduces and maps in a single launch are not sliced
             in_rows = any(p.row_group is not None and p.row_group.choose(env, {n: 0 for n in p.row_group.args})[1] for p in self.plans)
@@ -204,11 +206,11 @@ class ExportedOp:
             else:
                 source, plans = lower_graph(g, prefix='autort_' + _ident(self.name) + '_s' + '_'.join(str(k) for k in key))
                 v = {'graph': g, 'plans': plans, 'module': None, 'source': source}
-            if len(self._variants) >= 64:          # the oldest set of values goes (its code object stays in the cache on disk)
-                self._variants.pop(next(iter(self._variants)))
+            if len(self._variants) >= 64:          # the set of values used longest ago goes; its code object stays loaded
+                self._variants.pop(next(iter(self._variants)))      # (capi.shared_module) and is found again by its text
             self._variants[key] = v
         if v['module'] is None:
-            v['module'] = self._load() if v['source'] is None else capi.Module(compile_cached(v['source']))
+            v['module'] = self._load() if v['source'] is None else capi.shared_module(compile_cached(v['source']))
         return v
 
     def plans_for(self, env: Dict[str, int]) -> list:

@@ -34,10 +34,33 @@ def match(fused: Graph) -> Optional[Tuple[Callable, Dict[str, str]]]:
     """(handler, roles) for a recognised program, else None.  ``roles`` maps the registered program's tensor names
     to the names the caller's program uses for the tensors in the same places."""
     hit = _TABLE.get(fused.canonical_key())
-    if hit is None:
+    if hit is None or not _axes_span_their_dimensions(fused):
         return None
     handler, registered = hit
     return handler, dict(zip(registered, fused.canonical_tensor_order()))
+
+
+def _axes_span_their_dimensions(fused: Graph) -> bool:
+    """The canonical key drops extents, and the handlers take every size from the operands' shapes: a program that
+    restricts an axis (`... where K in 100`, `... where M in 100`) spells the same statements but computes something
+    else - a shorter sum, a smaller output.  Such a program is left to the generic lowering: a hand kernel is taken
+    only when every axis that indexes a tensor dimension directly runs over exactly that dimension."""
+    from ..ir.nodes import walk
+    for st in fused.statements:
+        extent = dict(st.data_axes + st.reduce_axes)
+        uses = [(st.output, st.out_index)]
+        uses += [(n.name, n.args) for n in walk(st.root) if n.kind == 'load']
+        for name, index in uses:
+            info = fused.tensors.get(name)
+            if info is None:
+                continue
+            shape = list(info.shape)
+            if len(index) != len(shape):
+                continue                          # scalars (`[]` against `[1]`) carry no axis
+            for ix, dim in zip(index, shape):
+                if ix.kind == 'axis' and ix.name in extent and extent[ix.name] != dim:
+                    return False
+    return True
 
 
 # ---------------------------------------------------------------------------

@@ -21,6 +21,7 @@ struct Workspace {
 // the first time the stream is seen (up to kMaxStreamsPerDevice streams per device; that first use must not happen
 // while the stream is being captured into a graph, because it allocates).  Returns nullptr with the error set.
 Workspace* workspace(hipStream_t stream);
+int release_stream(hipStream_t stream);
 constexpr int kMaxStreamsPerDevice = 40;      // torch hands out 32 pooled streams per device besides the default one
 
 // Looks up, for the current device, the address of the scratch array built into the code object (used by

@@ -79,10 +79,14 @@ Workspace* workspace(hipStream_t stream) {
     fail("call art_init first");
     return nullptr;
   }
-  for (int i = 0; i < d.used; ++i)
-    if (d.slot[i].stream == stream) return &d.slot[i].ws;
-  if (d.used == kMaxStreamsPerDevice) {
-    fail("more than %d streams use split-K / two-pass kernels on device %d; order them on fewer streams", kMaxStreamsPerDevice, dev);
+  int free_slot = -1;
+  for (int i = 0; i < d.used; ++i) {
+    if (d.slot[i].ws.base != nullptr && d.slot[i].stream == stream) return &d.slot[i].ws;
+    if (d.slot[i].ws.base == nullptr && free_slot < 0) free_slot = i;        // released by art_release_stream
+  }
+  if (free_slot < 0 && d.used == kMaxStreamsPerDevice) {
+    fail("more than %d streams use split-K / two-pass kernels on device %d; order them on fewer streams, or hand the "
+         "workspaces of destroyed streams back with art_release_stream", kMaxStreamsPerDevice, dev);
     return nullptr;
   }
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
@@ -91,12 +95,36 @@ Workspace* workspace(hipStream_t stream) {
          "run the operator once on this stream before capturing");
     return nullptr;
   }
-  StreamWorkspace& sw = d.slot[d.used];
+  StreamWorkspace& sw = d.slot[free_slot >= 0 ? free_slot : d.used];
   sw.stream = stream;
   sw.ws = Workspace{};
   if (allocate_workspace(&sw.ws)) return nullptr;
-  ++d.used;
+  if (free_slot < 0) ++d.used;
   return &sw.ws;
+}
+
+// Frees the workspace of (current device, stream) after the stream's work has finished; the slot can be taken by
+// another stream afterwards.  A stream without a workspace is no error.
+int release_stream(hipStream_t stream) {
+  int dev = 0;
+  ART_HIP(hipGetDevice(&dev));
+  ART_REQUIRE(dev >= 0 && dev < kMaxDevices, "art_release_stream: bad device %d", dev);
+  ART_REQUIRE(stream != nullptr, "art_release_stream: the default stream keeps its workspace");
+  void* base = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_mu);
+    DeviceState& d = g_dev[dev];
+    for (int i = 0; i < d.used; ++i)
+      if (d.slot[i].ws.base != nullptr && d.slot[i].stream == stream) {
+        base = d.slot[i].ws.base;
+        d.slot[i].ws = Workspace{};
+        d.slot[i].stream = nullptr;
+      }
+  }
+  if (base == nullptr) return 0;
+  ART_HIP(hipStreamSynchronize(stream));       // outside the lock: launches on other streams go on meanwhile
+  ART_HIP(hipFree(base));
+  return 0;
 }
 
 static std::string& compile_log() {
@@ -118,6 +146,7 @@ extern "C" {
 const char* art_last_error(void) { return art::last_error().c_str(); }
 const char* art_compile_log(void) { return art::compile_log().c_str(); }
 size_t art_workspace_bytes(void) { return art::kWorkspaceBytes; }
+int art_release_stream(void* stream) { return art::release_stream((hipStream_t)stream); }
 
 int art_init(int device) {
   int count = 0;

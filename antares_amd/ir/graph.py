@@ -291,7 +291,8 @@ def pad_guarded_factors(graph: Graph, env: Optional[Dict[str, int]] = None) -> G
 
     where [lo, hi] is the interval each index takes: the guards are evaluated once per element of the padded copy
     instead of once per term of the sum (nine times per element for a 3 x 3 filter, and in the inner loop of the
-    contraction).  Only when every condition compares one of the load's own index expressions with a constant, the
+    contraction).  Only when the guarded value is the load itself (or casts of it: g(0) must be 0 for what stays
+    around the padded load), every condition compares one of the load's own index expressions with a constant, the
     unguarded indices provably stay inside the tensor, the copy is at most four times the tensor, and the sum has at
     least 64 terms.  `env`: values of named dimensions for one call (the result is then valid for those only)."""
     from .nodes import Expr as E
@@ -316,10 +317,15 @@ def pad_guarded_factors(graph: Graph, env: Optional[Dict[str, int]] = None) -> G
                 f = root.args[which]
                 if f.kind != 'when' or len(f.args) != 2 or f.merge != 'all' or not (f.args[1].kind == 'const' and f.args[1].value == 0):
                     continue
-                loads = [n for n in walk(f.args[0]) if n.kind == 'load']
-                if len(loads) != 1 or not loads[0].args or loads[0].name == st.output or loads[0].name + '__pad' in tensors:
+                # The guarded value must be the load itself or casts of it: the contraction then reads the padded copy
+                # through the same casts, and a cast maps the copy's zeros to zeros.  Anything else around the load
+                # (`(x[..] + 1).when(..)`, `x[..].call(exp)`) would turn the border's 0 into g(0).
+                bare = f.args[0]
+                while bare.kind == 'cast' and len(bare.args) == 1:
+                    bare = bare.args[0]
+                if bare.kind != 'load' or not bare.args or bare.name == st.output or bare.name + '__pad' in tensors:
                     continue
-                ld = loads[0]
+                ld = bare
                 if any(n.kind in ('load', 'when') for c in f.conds for n in walk(c)):
                     continue
                 shape = [value(d) for d in tensors[ld.name].shape]

@@ -46,6 +46,7 @@ _SIGNATURES = {
     'art_stream_synchronize': (c_int, [c_void_p]),
     'art_copy_bytes': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     'art_workspace_bytes': (c_size_t, []),
+    'art_release_stream': (c_int, [c_void_p]),
     'art_alloc': (c_int, [c_size_t, POINTER(c_void_p)]),
     'art_free': (c_int, [c_void_p]),
     'art_memcpy_htod': (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -156,6 +157,22 @@ class Module:
             check(lib().art_get_function(self.handle, name.encode(), byref(f)))
             self._funcs[name] = f
         return f
+
+
+_loaded_modules = {}
+
+
+def shared_module(image: bytes) -> Module:
+    """The loaded code object for this image, loaded once per process: an operator that drops a per-shape kernel set
+    from its table and meets the shape again gets the module that is already on the device instead of loading a
+    second copy.  Modules stay loaded for the life of the process (a recorded graph may still launch from them), as the
+    reference's do (graph_evaluator/execute_module.hpp:274-319)."""
+    import hashlib
+    key = hashlib.sha256(image).digest()
+    m = _loaded_modules.get(key)
+    if m is None:
+        m = _loaded_modules[key] = Module(image)
+    return m
 
 
 def launch(func, grid, block, stream: int, args, lds: int = 0):

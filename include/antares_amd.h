@@ -368,6 +368,15 @@ int art_greedy_next(const void* logits_dev, int vocab, const void* prompt_dev, i
 /* Bytes of one library workspace (one per stream that launches split-K / two-pass kernels). */
 size_t art_workspace_bytes(void);
 
+/* Hands back the workspace the library allocated for `stream` on the current device (waits for the stream's work
+ * first), so that a process that creates and destroys streams does not run out of the 40 slots: call it before
+ * destroying a stream that launched a split-K / two-pass kernel.  A stream that has none is no error; the default
+ * stream keeps its workspace.  A HIP graph recorded on a stream has that stream's workspace baked into its kernel
+ * arguments: replay it on the stream it was recorded on (or order it there), and do not release that stream while
+ * the graph is alive.  The reference frees nothing either way (its allocation cache never shrinks,
+ * backends/c-rocm/include/backend.hpp:78-114). */
+int art_release_stream(void* stream);
+
 #ifdef __cplusplus
 }
 #endif

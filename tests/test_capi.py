@@ -126,3 +126,35 @@ def test_store_only_launch_and_phases_meeting_inside_one_launch():
                                    c_void_p(status.data_ptr()), None) != 0
     assert l.art_phase_chain_probe(c_void_p(src.data_ptr()), src.numel(), 1000, 1, 1, c_void_p(sink.data_ptr()),
                                    c_void_p(status.data_ptr()), None) != 0
+
+
+@pytest.mark.gpu
+def test_a_released_stream_gives_its_workspace_back():
+    """A process that creates and destroys streams: every stream that launches a split-K kernel gets a 64 MiB
+    workspace (40 slots per device); `art_release_stream` hands it back, so the 41st, 42nd ... stream still works, and
+    a released stream that launches again simply gets a new one."""
+    import numpy as np
+    import torch
+    from ctypes import c_void_p
+    from antares_amd import workloads
+    from antares_amd.runtime import capi
+    capi.init(0)
+    lib = capi.lib()
+    p = {k: v.cuda() for k, v in workloads.w4_problem(5, 1, 1024, 256).items()}
+    want = None
+    for i in range(48):
+        s = torch.cuda.Stream()
+        y = torch.zeros(1, 256, dtype=torch.float16, device='cuda')
+        s.wait_stream(torch.cuda.current_stream())
+        capi.check(lib.art_gemv_w4a16(c_void_p(p['x'].data_ptr()), c_void_p(p['qweight'].data_ptr()), c_void_p(p['scales'].data_ptr()),
+                                      c_void_p(p['qzeros'].data_ptr()), c_void_p(y.data_ptr()), 1, 1024, 256, c_void_p(s.cuda_stream)))
+        if i % 7 == 0:            # a stream that is released and used again
+            capi.check(lib.art_release_stream(c_void_p(s.cuda_stream)))
+            capi.check(lib.art_gemv_w4a16(c_void_p(p['x'].data_ptr()), c_void_p(p['qweight'].data_ptr()), c_void_p(p['scales'].data_ptr()),
+                                          c_void_p(p['qzeros'].data_ptr()), c_void_p(y.data_ptr()), 1, 1024, 256, c_void_p(s.cuda_stream)))
+        capi.check(lib.art_release_stream(c_void_p(s.cuda_stream)))          # waits for the stream's work
+        got = y.cpu().numpy()
+        want = got if want is None else want
+        assert np.array_equal(got, want), i
+    capi.check(lib.art_release_stream(c_void_p(torch.cuda.Stream().cuda_stream)))      # a stream with no workspace: no error
+    assert lib.art_release_stream(c_void_p(0)) != 0 and b'default stream' in lib.art_last_error()

@@ -244,3 +244,45 @@ def test_a_zero_padded_factor_is_copied_into_a_padded_tensor_once():
         assert pad_guarded_factors(g2, env) is g2, ir
     g3 = fuse_elementwise(parse_program(refused[2], ['input0=float32[N:64, J:40]', 'input1=float32[K:40, M:64]']))
     assert pad_guarded_factors(g3, {'N': 64, 'J': 40, 'K': 40, 'M': 64}) is g3
+
+
+def test_the_padding_rewrite_leaves_guarded_values_that_do_not_map_zero_to_zero():
+    """`g(x[..]).when(conds, 0) * w`: the border contributes 0, not g(0) * w.  The rewrite into a padded copy is only
+    taken for a bare load or casts of it; whatever the rewrite returns must compute what the program as written does
+    (both run through the CPU oracle, before and after)."""
+    import numpy as np
+    from antares_amd.ir.graph import pad_guarded_factors
+    from oracle.cpu_backend import CpuModule
+    guards = '.when([HO + KH - 1 >= 0, HO + KH - 1 < 16, WO + KW - 1 >= 0, WO + KW - 1 < 16], 0.0)'
+    idx = 'input0[N, C, HO + KH - 1, WO + KW - 1]'
+    env = {'N': 2, 'C': 8, 'H': 16, 'W': 16, 'F': 4, 'KH': 3, 'KW': 3}
+    rng = np.random.default_rng(2)
+    w = rng.standard_normal((4, 8, 3, 3)).astype(np.float32)
+    cases = [
+        (f'({idx} + 1.0)', 'float32', False),                        # g(0) = 1
+        (f'{idx}.call(`exp`)', 'float32', False),                    # g(0) = 1
+        (f'({idx} * 2.0)', 'float32', False),                        # maps 0 to 0, but not proved: left alone
+        (idx, 'float32', True),
+        (f'{idx}.cast(`float32`)', 'float16', True),                 # a cast stays around the padded load
+    ]
+    for factor, dt, rewritten in cases:
+        ir = f'output0[N, F, HO, WO] +=! {factor}{guards} * input1[F, C, KH, KW] where HO in 16, WO in 16'
+        g = fuse_elementwise(parse_program(ir, [f'input0={dt}[N:2, C:8, H:16, W:16]', 'input1=float32[F:4, C:8, KH:3, KW:3]']))
+        after = pad_guarded_factors(g, env)
+        assert (after is not g) == rewritten, factor
+        x = rng.standard_normal((2, 8, 16, 16)).astype(np.float16 if dt == 'float16' else np.float32)
+        want = CpuModule(g, fast_math=False)(input0=x, input1=w)['output0']
+        got = CpuModule(after, fast_math=False)(input0=x, input1=w)['output0']
+        assert np.array_equal(got, want), factor
+    # what the refused rewrite would have done wrong: the border of the `+ 1.0` case is not the interior's formula
+    ir = f'output0[N, F, HO, WO] +=! ({idx} + 1.0){guards} * input1[F, C, KH, KW] where HO in 16, WO in 16'
+    g = fuse_elementwise(parse_program(ir, ['input0=float32[N:2, C:8, H:16, W:16]', 'input1=float32[F:4, C:8, KH:3, KW:3]']))
+    x = rng.standard_normal((2, 8, 16, 16)).astype(np.float32)
+    out = CpuModule(g, fast_math=False)(input0=x, input1=w)['output0']
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1))) + 1.0                 # the wrong reading: g applied to the padding
+    wrong = np.einsum('nchw,fc->nfhw', xp[:, :, 0:16, 0:16], w[:, :, 0, 0])
+    for kh in range(3):
+        for kw in range(3):
+            if kh or kw:
+                wrong += np.einsum('nchw,fc->nfhw', xp[:, :, kh:kh + 16, kw:kw + 16], w[:, :, kh, kw])
+    assert np.abs(out - wrong)[:, :, 0, :].max() > 0.5 and np.allclose(out[:, :, 1:15, 1:15], wrong[:, :, 1:15, 1:15], atol=1e-4)

@@ -206,3 +206,32 @@ def test_hand_kernel_roles_follow_the_program_not_the_names():
     # the registered spelling maps to itself
     own = ExportedOp(patterns.GEMM_F16_IR, patterns.GEMM_F16_INPUTS)
     assert own.fast_roles['a'] == 'a' and own.fast_roles['c'] == 'c'
+
+
+def test_programs_that_restrict_an_axis_do_not_take_a_hand_kernel():
+    """The hand kernels take every size from the operands' shapes; `where K in 100` or `where M in 100` spell the same
+    statements as the full product but compute a shorter sum or a smaller output, so they must go to the generic
+    lowering (the canonical key alone cannot tell them apart)."""
+    from antares_amd.autort import patterns
+    from antares_amd.autort.op import ExportedOp
+    from antares_amd.ir import fuse_elementwise, parse_program
+    cases = [(patterns.GEMM_F32_IR, patterns.GEMM_F32_INPUTS), (patterns.BATCH_GEMM_F32_IR, patterns.BATCH_GEMM_F32_INPUTS),
+             ('c[M, N] +=! a[K, M] * b[K, N]', ['a=float32[K:512, M:512]', 'b=float32[K:512, N:512]']),
+             ('c[M, N] +=! a[M, K] * b[N, K]', ['a=float32[M:512, K:512]', 'b=float32[N:512, K:512]']),
+             ('c[M, N] +=! a[K, M] * b[N, K]', ['a=float32[K:512, M:512]', 'b=float32[N:512, K:512]'])]
+    for ir, inputs in cases:
+        assert patterns.match(fuse_elementwise(parse_program(ir, inputs))) is not None, ir
+        for clause in ('K in 100', 'M in 100', 'N in 8'):
+            g = fuse_elementwise(parse_program(f'{ir} where {clause}', inputs))
+            assert patterns.match(g) is None, (ir, clause)
+            assert ExportedOp(f'{ir} where {clause}', list(inputs)).fast_path is None
+    # the two-statement programs: a restricted reduce axis in the first statement
+    f16 = patterns.GEMM_F16_IR.strip().split('\n')
+    restricted = f16[0] + ' where K in 64\n' + f16[1]
+    assert patterns.match(fuse_elementwise(parse_program(patterns.GEMM_F16_IR, patterns.GEMM_F16_INPUTS))) is not None
+    assert patterns.match(fuse_elementwise(parse_program(restricted, patterns.GEMM_F16_INPUTS))) is None
+    w4 = patterns.W4A16_IR.strip().split('\n')
+    assert patterns.match(fuse_elementwise(parse_program(w4[0] + ' where N in 16\n' + w4[1] + ' where N in 16', patterns.W4A16_INPUTS))) is None
+    # a `where` that only repeats the dimension, or static shapes of the full extent, still match
+    assert patterns.match(fuse_elementwise(parse_program('c[M, N] +=! a[M, K] * b[K, N] where K in 4096',
+                                                         ['a=float32[4096, 4096]', 'b=float32[4096, 4096]']))) is not None
