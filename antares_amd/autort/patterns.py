@@ -194,8 +194,18 @@ def _gemm_f16_handler(op, bound, env, stream) -> bool:
     N = b.shape[1]
     if N % 8 or K % 64 or a.data_ptr() % 16 or b.data_ptr() % 16 or c.data_ptr() % 16:
         return False
-    capi.check(capi.lib().art_gemm_f16(c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()), M, N, K,
-                                      c_void_p(stream)))
+
+    def run(value, t, st=None):
+        capi.check(capi.lib().art_gemm_f16_tuned(c_void_p(t[0].data_ptr()), c_void_p(t[1].data_ptr()), c_void_p(t[2].data_ptr()), M, N, K,
+                                                 int(value), c_void_p(stream if st is None else st)))
+    # the launch parameter: threads per block (2 x 2 wavefronts of 128 x 128 outputs, or 2 x 4 of 128 x 64)
+    key = f'gemm_f16.threads|{M},{K},{N}'
+    saved = op.tuned.get(key)
+    trials = op.config.get('tune')
+    if saved is None and isinstance(trials, int) and trials > 0 and not torch.cuda.is_current_stream_capturing():
+        saved = tune_hand_kernel(op, key, [256, 512], lambda v, t: run(v, t, torch.cuda.current_stream().cuda_stream), trials,
+                                 [(a, b, torch.empty_like(c))])
+    run(saved['value'] if saved is not None else 0, (a, b, c))
     return True
 
 

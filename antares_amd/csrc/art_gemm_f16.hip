@@ -8,7 +8,9 @@
 // Design for MI355X:
 //   * block tile 256 x 256 x 32, 256 threads = 2 x 2 wavefronts, each wavefront owns 128 x 128 of C as
 //     4 x 4 accumulator tiles of v_mfma_f32_32x32x16_f16 (256 accumulator registers per lane, one
-//     wavefront per SIMD); 16 MFMAs (512 matrix-core cycles) per 8 KiB of LDS reads;
+//     wavefront per SIMD); 16 MFMAs (512 matrix-core cycles) per 8 KiB of LDS reads.  The same tile can be worked
+//     by 512 threads = 2 x 4 wavefronts of 128 x 64 (two wavefronts per SIMD): a launch parameter for tuning runs,
+//     not the default - measured side by side it is 3 % slower at 4096^3 and 8 % slower at 8192^3;
 //   * A tile in LDS as [m][k] (k contiguous, rows padded by 16 bytes): one ds_read_b128 gives a lane
 //     its 8 consecutive k of one row;
 //   * B tile in LDS exactly as it lies in memory, [k][n] (n contiguous, rows padded by 64 bytes); the
@@ -51,14 +53,19 @@ __device__ __forceinline__ int xcd_tile(int b, int nb) {
 
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
-__global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
-                                                        _Float16* __restrict__ C, int M, int N, int K) {
+template <int WN>      // wavefronts along n: 2 (256 threads, 128 x 128 per wavefront) or 4 (512 threads, 128 x 64)
+__global__ __launch_bounds__(128 * WN) void gemm_f16_kernel(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
+                                                           _Float16* __restrict__ C, int M, int N, int K) {
+  constexpr int NT_ = 128 * WN;            // threads
+  constexpr int CH = 1024 / NT_;           // 16-byte chunks per thread, operand and stage
+  constexpr int NJ = 8 / WN;               // 32-column accumulator tiles per wavefront
+  constexpr int WCOLS = 256 / WN;          // columns per wavefront
   extern __shared__ __align__(16) _Float16 smem[];
   _Float16* As = smem;                    // [2][BM][A_LD]
   _Float16* Bs = smem + 2 * A_TILE;       // [2][BK][B_LD]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int MT = (M + BM - 1) / BM, NT = (N + BN - 1) / BN;      // edge tiles are clamped on the way in and cut on the way out
   int tile = xcd_tile(blockIdx.x, gridDim.x), tm, tn;
   if ((MT % 4 == 0) && (NT % 8 == 0)) {   // 4 x 8 super-tiles, row-major inside and outside
@@ -72,12 +79,12 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
 
   // global -> register staging: 4 chunks of 16 bytes per thread for each operand and stage.  The
   // per-thread part of every address is computed once; a tile only adds a wave-uniform offset.
-  u32x4 ga[2][4], gb[2][4];
-  const _Float16* pa[4];
-  const _Float16* pb[4];
+  u32x4 ga[2][CH], gb[2][CH];
+  const _Float16* pa[CH];
+  const _Float16* pb[CH];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = tid + 256 * i;
+  for (int i = 0; i < CH; ++i) {
+    const int c = tid + NT_ * i;
     // rows past M and columns past N repeat the last valid ones: their products are never stored
     const int arow = tm * BM + (c >> 2), bcol = tn * BN + (c & 31) * 8;
     pa[i] = A + (size_t)(arow < M ? arow : M - 1) * K + (c & 3) * 8;
@@ -88,7 +95,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
     constexpr int S = decltype(tag)::value;
     const size_t oa = (size_t)kt * BK, ob = (size_t)kt * b_step;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < CH; ++i) {
       ga[S][i] = *reinterpret_cast<const u32x4*>(pa[i] + oa);
       gb[S][i] = *reinterpret_cast<const u32x4*>(pb[i] + ob);
     }
@@ -96,18 +103,18 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
   auto store_tiles = [&](int buf, auto tag) {
     constexpr int S = decltype(tag)::value;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + 256 * i;
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + NT_ * i;
       *reinterpret_cast<u32x4*>(As + buf * A_TILE + (c >> 2) * A_LD + (c & 3) * 8) = ga[S][i];
       *reinterpret_cast<u32x4*>(Bs + buf * B_TILE + (c >> 5) * B_LD + (c & 31) * 8) = gb[S][i];
     }
   };
 
-  f16v acc[4][4];
+  f16v acc[4][NJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -116,13 +123,13 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
   const int a_k = (lane >> 5) * 8;                          // + kk*16
   const int s = lane & 15;
   const int b_k = (lane >> 5) * 8 + (s >> 2);               // + kk*16 + r*4
-  const int b_n = wn * 128 + ((lane & 31) >> 4) * 16 + (s & 3) * 4;   // + j*32
+  const int b_n = wn * WCOLS + ((lane & 31) >> 4) * 16 + (s & 3) * 4;   // + j*32
 
-  auto load_frags = [&](h8 (&af)[4], h8 (&bf)[4], const _Float16* as, const _Float16* bs, int kk) {
+  auto load_frags = [&](h8 (&af)[4], h8 (&bf)[NJ], const _Float16* as, const _Float16* bs, int kk) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const h8*>(as + (a_row + i * 32) * A_LD + kk * 16 + a_k);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       const _Float16* p = bs + (kk * 16 + b_k) * B_LD + b_n + j * 32;
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
       const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * B_LD));
@@ -130,11 +137,11 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
       bf[j] = h8{l4[0], l4[1], l4[2], l4[3], h4v[0], h4v[1], h4v[2], h4v[3]};
     }
   };
-  auto mfma_all = [&](const h8 (&af)[4], const h8 (&bf)[4]) {
+  auto mfma_all = [&](const h8 (&af)[4], const h8 (&bf)[NJ]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
   };
 
   const int T = K / BK;
@@ -145,7 +152,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
   store_tiles(0, S0{});
   load_tiles(T > 2 ? 2 : T - 1, S0{});
   art_lds_barrier();
-  h8 af0[4], bf0[4], af1[4], bf1[4];
+  h8 af0[4], bf0[NJ], af1[4], bf1[NJ];
   load_frags(af0, bf0, As, Bs, 0);
   // One tile = two k-steps of 16 MFMAs.  Tile t sits in LDS buffer t & 1.  Register stage `nxt` holds
   // tile t + 1 (requested a tile and a half ago); once it is written to LDS it is refilled with tile
@@ -165,9 +172,9 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
     if (!LAST) store_tiles(buf ^ 1, nxt);
     mfma_all(af0, bf0);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < 4 * NJ; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);                   // 12 reads + 8 writes
+      __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);                   // 12 reads + 8 writes (8 + 4 with 512 threads)
       if (i < 4) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -178,10 +185,10 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
     }
     mfma_all(af1, bf1);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < 4 * NJ; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      if (i < 12) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);      // 12 reads
-      if (i >= 4 && i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      if (NJ == 2 || i < 12) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);      // 12 reads (8 with 512 threads)
+      if (NJ == 4 ? (i >= 4 && i < 12) : (i >= 2 && i < 6)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -199,17 +206,17 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = wm * 128 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        const int col = wn * 128 + j * 32 + (lane & 31);
+        const int col = wn * WCOLS + j * 32 + (lane & 31);
         cs[row * C_LD + col] = (_Float16)acc[i][j][r];
       }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 32; ++i) {
-    const int c = tid + 256 * i;               // 256 rows x 32 chunks of 8 halves
+  for (int i = 0; i < 8192 / NT_; ++i) {
+    const int c = tid + NT_ * i;               // 256 rows x 32 chunks of 8 halves
     const int row = c >> 5, ch = c & 31;
     const int grow = tm * BM + row, gcol = tn * BN + ch * 8;
     if (grow < M && gcol < N)
@@ -220,20 +227,32 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const _Float16* __restric
 }  // namespace
 
 extern "C" int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream) {
+  return art_gemm_f16_tuned(a_dev, b_dev, c_dev, M, N, K, 0, stream);
+}
+
+extern "C" int art_gemm_f16_tuned(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, int threads, void* stream) {
   ART_REQUIRE(a_dev && b_dev && c_dev, "art_gemm_f16: null pointer");
   ART_REQUIRE(M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 64 == 0,
               "art_gemm_f16: N must be a multiple of 8 and K of 64 (M=%d N=%d K=%d)", M, N, K);
   ART_REQUIRE(((uintptr_t)a_dev % 16) == 0 && ((uintptr_t)b_dev % 16) == 0 && ((uintptr_t)c_dev % 16) == 0,
               "art_gemm_f16: operands must be 16-byte aligned");
+  ART_REQUIRE(threads == 0 || threads == 256 || threads == 512, "art_gemm_f16: threads must be 0 (the library's choice), 256 or 512 (got %d)", threads);
   static bool configured = false;
   if (!configured) {
-    ART_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f16_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+    ART_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f16_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)kLdsBytes));
+    ART_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f16_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)kLdsBytes));
     configured = true;
   }
   const int blocks = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  gemm_f16_kernel<<<dim3(blocks), dim3(256), kLdsBytes, (hipStream_t)stream>>>((const _Float16*)a_dev, (const _Float16*)b_dev,
-                                                                                (_Float16*)c_dev, M, N, K);
+  if (threads == 0) threads = 256;       // one wavefront per SIMD measured faster at every benchmark size
+  if (threads == 512)
+    gemm_f16_kernel<4><<<dim3(blocks), dim3(512), kLdsBytes, (hipStream_t)stream>>>((const _Float16*)a_dev, (const _Float16*)b_dev,
+                                                                                    (_Float16*)c_dev, M, N, K);
+  else
+    gemm_f16_kernel<2><<<dim3(blocks), dim3(256), kLdsBytes, (hipStream_t)stream>>>((const _Float16*)a_dev, (const _Float16*)b_dev,
+                                                                                    (_Float16*)c_dev, M, N, K);
   ART_LAUNCH_CHECK();
   return 0;
 }

@@ -161,7 +161,8 @@ class LlamaInt4Decoder:
                     'qzeros': gu['qzeros'][:, :F // 2].contiguous()}
             up = {'qweight': gu['qweight'][:, F:].contiguous(), 'scales': gu['scales'][:, F:].contiguous(),
                   'qzeros': gu['qzeros'][:, F // 2:].contiguous()}
-            layers.append({'qkv': packed(lw['qkv']), 'gate_up': packed(interleave_gate_up(gate, up)), 'down': packed(lw['down'])})
+            layers.append({'qkv': packed(lw['qkv']), 'gate_up': packed(interleave_gate_up(gate, up)), 'down': packed(lw['down']),
+                           'o': packed(lw['o'])})      # used when the attention runs as one block per head
         self.pw = {'layers': layers, 'lm_head': packed(self.w['lm_head'])}
 
     def _ops(self):
@@ -237,7 +238,7 @@ class LlamaInt4Decoder:
             else:
                 ops.attention_rope_f16(self.qkv, self.inv_freq, self.key_cache[l], self.val_cache[l], self.att_f, self.att,
                                        extra=[self.pos])
-                ops.gemv_w4a16_fused(self.att.view(-1), o['qweight'], o['scales'], o['qzeros'], self.x, residual=self.x)
+                gemv(self.att.view(-1), pw['o'], self.x, residual=self.x, shape=(d, d))
             gemv(self.x, pw['gate_up'], self.hb, norm_weight=lw['ffn_norm'], eps=cfg.rms_eps, swiglu_out=True, shape=(d, 2 * F))
             gemv(self.hb, pw['down'], self.x, residual=self.x, shape=(F, d))
         gemv(self.x, self.pw['lm_head'], self.logits, norm_weight=self.w['final_norm'], eps=cfg.rms_eps, shape=(d, cfg.vocab))

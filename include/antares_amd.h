@@ -257,6 +257,9 @@ int art_gemv_gptq(const void* x_dev, const void* qweight_dev, const void* scales
  * Replaces the kernel the reference generates for `C[N,M] +=! A[N,K] * B[K,M]`
  * (AntaresIR.md:115; tiled schedule backends/c-rocm/schedule/standard/algo_tiling.py:35-98). */
 int art_gemm_f16(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, void* stream);
+/* The same with the block shape a tuning run may vary: threads = 256 (2 x 2 wavefronts of 128 x 128 outputs, one per
+ * SIMD) or 512 (2 x 4 wavefronts of 128 x 64, two per SIMD), 0 = the library's choice (256). */
+int art_gemm_f16_tuned(const void* a_dev, const void* b_dev, void* c_dev, int M, int N, int K, int threads, void* stream);
 
 /* fp32 GEMM on the matrix cores (v_mfma_f32_32x32x2_f32): C[M,N] = A[M,K] @ B[K,N], all fp32, row-major; any M,
  * N % 4 == 0, K % 32 == 0; A and B 16-byte aligned, C must not overlap them.

@@ -59,6 +59,34 @@ def test_against_float64_product(gemm, M, N, K):
         assert torch.equal(f(bb.to(dev), eye.to(dev)).cpu(), bb)
 
 
+@pytest.mark.parametrize('threads', [256, 512])
+@pytest.mark.parametrize('M,N,K', [(256, 256, 64), (300, 1000, 192), (1024, 2048, 1024), (4096, 4096, 1024)])
+def test_both_block_shapes_against_float64_product(gemm, threads, M, N, K):
+    """`art_gemm_f16_tuned`: the 256 x 256 tile worked by 2 x 2 wavefronts (256 threads) or by 2 x 4 (512 threads) -
+    the launch parameter `tune:N` searches; the library's own choice is 256 threads."""
+    from ctypes import c_void_p
+    from antares_amd.runtime import capi
+    autort, _ = gemm
+    print(f'[case] art_gemm_f16_tuned threads={threads} {M}x{N}x{K}', flush=True)
+    g = torch.Generator().manual_seed(M + N + K + threads)
+    a = (torch.randn(M, K, generator=g) * 0.02).half()
+    b = (torch.randn(K, N, generator=g) * 0.02).half()
+    dev = autort.device()
+    capi.init(dev.index or 0)
+    ad, bd = a.to(dev), b.to(dev)
+    c = torch.empty(M, N, dtype=torch.float16, device=dev)
+    capi.check(capi.lib().art_gemm_f16_tuned(c_void_p(ad.data_ptr()), c_void_p(bd.data_ptr()), c_void_p(c.data_ptr()), M, N, K, threads,
+                                             c_void_p(torch.cuda.current_stream().cuda_stream)))
+    want = torch.from_numpy(oracle_gemm(a.numpy(), b.numpy()))
+    assert torch.allclose(c.cpu().float(), want.float(), **FP16_TOL)
+    other = torch.empty_like(c)
+    capi.check(capi.lib().art_gemm_f16_tuned(c_void_p(ad.data_ptr()), c_void_p(bd.data_ptr()), c_void_p(other.data_ptr()), M, N, K,
+                                             768 - threads, c_void_p(torch.cuda.current_stream().cuda_stream)))
+    assert torch.equal(c, other)            # same k order per output: the two shapes agree bit for bit
+    assert capi.lib().art_gemm_f16_tuned(c_void_p(ad.data_ptr()), c_void_p(bd.data_ptr()), c_void_p(c.data_ptr()), M, N, K, 128,
+                                         c_void_p(0)) != 0
+
+
 def test_shapes_the_kernel_does_not_take_use_the_generic_lowering(gemm):
     """K % 64 != 0 (or N % 8 != 0) is left to the generic reduce lowering."""
     autort, op = gemm
