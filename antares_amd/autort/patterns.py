@@ -147,14 +147,19 @@ def _w4a16_handler(op, bound, env, stream) -> bool:
     # more go there
     lib = capi.lib()
     gemv = M <= 3
-    entry = lib.art_gemv_w4a16_tuned if gemv else lib.art_gemm_w4a16_tuned
 
     def run(value, t, st=None):
-        capi.check(entry(c_void_p(t[0].data_ptr()), c_void_p(t[1].data_ptr()), c_void_p(t[2].data_ptr()), c_void_p(t[3].data_ptr()),
-                         c_void_p(t[4].data_ptr()), M, K, N, int(value), c_void_p(stream if st is None else st)))
+        args = (c_void_p(t[0].data_ptr()), c_void_p(t[1].data_ptr()), c_void_p(t[2].data_ptr()), c_void_p(t[3].data_ptr()),
+                c_void_p(t[4].data_ptr()), M, K, N)
+        if gemv:         # value = 16 * rows per lane + wavefronts per block (0: the library's choice of both)
+            capi.check(lib.art_gemv_w4a16_knobs(*args, int(value) >> 4, int(value) & 15, c_void_p(stream if st is None else st)))
+        else:
+            capi.check(lib.art_gemm_w4a16_tuned(*args, int(value), c_void_p(stream if st is None else st)))
 
-    # the launch parameter of the kernel that runs: k per block of the GEMV, K-splits of the GEMM
-    key = f"{'gemv_w4a16.k_per_block' if gemv else 'gemm_w4a16.k_splits'}|{M},{K},{N}"
+    # the launch parameters of the kernel that runs: (rows per lane, wavefronts per block) of the GEMV - two factors
+    # searched as a product space, as the reference's tuner walks the factor spaces of a schedule's knobs
+    # (tuner/OpEvo/main.py:154-293) -, (K-splits, rows per block) of the GEMM
+    key = f"{'gemv_w4a16.rows_x16_plus_waves' if gemv else 'gemm_w4a16.k_splits'}|{M},{K},{N}"
     saved = op.tuned.get(key)
     trials = op.config.get('tune')
     if saved is None and isinstance(trials, int) and trials > 0 and not torch.cuda.is_current_stream_capturing():
@@ -162,7 +167,7 @@ def _w4a16_handler(op, bound, env, stream) -> bool:
         copies = max(1, min(8, (256 << 20) // max(per_set, 1)))
         clones = [(x, q.clone(), s.clone(), z.clone(), torch.empty_like(y)) for _ in range(copies)]
         if gemv:
-            cands = [512, 256, 1024] if M == 1 else [512, 256]
+            cands = [16 * rows + waves for rows in (8, 4) for waves in ((4, 8) if M == 1 else (4,))]
         else:
             counts = [v for v in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32) if v <= K // 128]
             # 512 + v: v K-splits over blocks of 64 rows; 256 + v: over blocks of 32 rows (twice the blocks)

@@ -536,6 +536,7 @@ int launch(const void* x, const void* qw, const void* sc, const void* qz, void* 
       if (fused.norm_w != nullptr) ART_GEMV_LAUNCH(1, 8, 8);
       else if (fused.gate_up != nullptr) ART_GEMV_LAUNCH(2, 8, 8);
       else if (fused.att_partial != nullptr) ART_GEMV_LAUNCH(3, 8, 8);
+      else if (rows_per_lane == 4) ART_GEMV_LAUNCH(0, 4, 8);
       else ART_GEMV_LAUNCH(0, 8, 8);
     } else {
       if (fused.norm_w != nullptr && fused.sumsq_in != nullptr) ART_GEMV_LAUNCH(4, 8, 4);
@@ -565,9 +566,19 @@ extern "C" int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, 
                                     void* y_dev, int M, int K, int N, int k_per_block, void* stream) {
   ART_REQUIRE(k_per_block == 0 || k_per_block == 256 || k_per_block == 512 || k_per_block == 1024,
               "art_gemv_w4a16: k_per_block must be 0 (library's choice), 256, 512 or 1024 (got %d)", k_per_block);
-  ART_REQUIRE(k_per_block != 1024 || M == 1, "art_gemv_w4a16: k_per_block = 1024 is for M = 1 (got M = %d)", M);
   // 256: four rows per lane, four wavefronts; 512: eight rows, four wavefronts; 1024: eight rows, eight wavefronts
-  const int rpl = k_per_block == 256 ? 4 : 8, waves = k_per_block == 0 ? 0 : (k_per_block == 1024 ? 8 : 4);
+  const int rpl = k_per_block == 0 ? 0 : (k_per_block == 256 ? 4 : 8), waves = k_per_block == 0 ? 0 : (k_per_block == 1024 ? 8 : 4);
+  return art_gemv_w4a16_knobs(x_dev, qweight_dev, scales_dev, qzeros_dev, y_dev, M, K, N, rpl, waves, stream);
+}
+
+extern "C" int art_gemv_w4a16_knobs(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                                    void* y_dev, int M, int K, int N, int rows_per_lane, int waves_per_block, void* stream) {
+  ART_REQUIRE(rows_per_lane == 0 || rows_per_lane == 4 || rows_per_lane == 8, "art_gemv_w4a16: rows_per_lane must be 0 (library's choice), 4 or 8 (got %d)",
+              rows_per_lane);
+  ART_REQUIRE(waves_per_block == 0 || waves_per_block == 4 || waves_per_block == 8,
+              "art_gemv_w4a16: waves_per_block must be 0 (library's choice), 4 or 8 (got %d)", waves_per_block);
+  ART_REQUIRE(waves_per_block != 8 || M == 1, "art_gemv_w4a16: eight wavefronts per block are for M = 1 (got M = %d)", M);
+  const int rpl = rows_per_lane == 0 ? 8 : rows_per_lane, waves = waves_per_block;
   ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16: null pointer");
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0,

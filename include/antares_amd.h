@@ -23,7 +23,9 @@
  *
  * The first group replaces the reference's header-only `namespace ab` device
  * runtime and its ExecutionModule; the second group are typed entry points for
- * the hand-written kernels that replace generated code on the hot path.
+ * the hand-written kernels that replace generated code on the hot path; the
+ * last group (calibration launches) is measurement tooling, not part of the
+ * drop-in surface.
  */
 #ifndef ANTARES_AMD_H_
 #define ANTARES_AMD_H_
@@ -109,32 +111,6 @@ int art_memcpy_dtoh(void* dst_host, const void* src_dev, size_t bytes, void* str
 /* Device to device, asynchronous on `stream`; replaces ab::memcpyDtoD (backend.hpp:225-227). */
 int art_memcpy_dtod(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
 
-/* Plain device copy kernel (dst, src: 16-byte aligned, bytes % 16 == 0); used
- * as the calibration workload for memory-traffic counters. */
-int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
-
-/* Read-only counterpart: one launch that fetches `bytes` (a multiple of 32768, at most 128 MiB; 16-byte aligned)
- * with the access pattern of the int4 GEMV's weight stream (blocks of 256 threads x eight 16-byte loads, rows of
- * 11008 bytes when bytes is a multiple of 11008 * 256, else of 128 bytes) and computes nothing.  Its duration is the
- * floor of any single launch that has to bring these bytes on chip.  sink_dev: 4096 words of scratch (never
- * written in practice). */
-int art_read_bytes(const void* src_dev, size_t bytes, void* sink_dev, void* stream);
-
-/* Store-only counterpart: one launch that writes `bytes` (a multiple of 16, 16-byte aligned) of the 32-bit `value`
- * with non-temporal 16-byte stores and reads nothing: the floor of a launch that has to write these bytes. */
-int art_fill_bytes(void* dst_dev, size_t bytes, unsigned int value, void* stream);
-
-/* Measurement only, no counterpart in the reference: what a grid-wide meeting inside ONE launch costs on this part,
- * i.e. what a persistent whole-token kernel would pay instead of a dependent launch.  256 resident blocks run `phases`
- * phases over src_dev (phases * phase_bytes bytes, at most src_bytes; phase_bytes a multiple of 32768, at most
- * 24 MiB); in every phase a block fetches its share with the access pattern of art_read_bytes, then all blocks meet
- * through one word per block in the stream's workspace (agent-scope stores and loads, no atomics, no fences, every
- * wait bounded).  mode 0: no loads; 1: a phase's loads follow the previous meeting; 2: the next phase's loads are
- * issued before the meeting.  status_dev: one 32-bit word, zero before the call, 1 afterwards if a block gave up
- * waiting (the chip was not free to hold all 256 blocks).  sink_dev: 256 words of scratch. */
-int art_phase_chain_probe(const void* src_dev, size_t src_bytes, size_t phase_bytes, int phases, int mode, void* sink_dev,
-                          void* status_dev, void* stream);
-
 /* ---------------------------------------------------- hand-written kernels */
 
 /* Weight-only int4 GEMV / skinny GEMM, group size 128 along K:
@@ -164,6 +140,11 @@ int art_gemv_w4a16(const void* x_dev, const void* qweight_dev, const void* scale
  *   max_blocks:    cap on the blocks of the partition, 64..16384 (each walks its span tile by tile). */
 int art_gemv_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                          void* y_dev, int M, int K, int N, int k_per_block, void* stream);
+/* The two factors behind k_per_block as independent knobs: rows_per_lane 4 or 8 (packed rows a lane loads before it
+ * multiplies: 8 or 16 values of k), waves_per_block 4 or 8 (a block's k range is 16 x rows_per_lane x waves_per_block:
+ * 256 .. 1024); 0 = the library's choice for either.  Eight wavefronts need M = 1. */
+int art_gemv_w4a16_knobs(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
+                         void* y_dev, int M, int K, int N, int rows_per_lane, int waves_per_block, void* stream);
 int art_gemm_w4a16_tuned(const void* x_dev, const void* qweight_dev, const void* scales_dev, const void* qzeros_dev,
                          void* y_dev, int M, int K, int N, int k_splits, void* stream);
 int art_partition_even_first_i32_tuned(const void* in_dev, void* out_dev, long long n, int max_blocks, void* stream);
@@ -379,6 +360,40 @@ size_t art_workspace_bytes(void);
  * the graph is alive.  The reference frees nothing either way (its allocation cache never shrinks,
  * backends/c-rocm/include/backend.hpp:78-114). */
 int art_release_stream(void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Calibration launches - NOT part of the drop-in surface.  Nothing in the operator path calls them and a binding
+ * of the reference needs none of them; they exist so that the figures under profiles/ can be reproduced with
+ * committed code (`bench.py --calibrate-copy / --read-floor / --stream-floors / --phase-chain`): a copy of known size
+ * to scale memory-traffic counters, and the floors of one launch that only reads, only writes, or meets inside
+ * itself.  They have no counterpart in the reference.
+ * ------------------------------------------------------------------------------------------------------------ */
+
+/* Plain device copy kernel (dst, src: 16-byte aligned, bytes % 16 == 0); used
+ * as the calibration workload for memory-traffic counters. */
+int art_copy_bytes(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+
+/* Read-only counterpart: one launch that fetches `bytes` (a multiple of 32768, at most 128 MiB; 16-byte aligned)
+ * with the access pattern of the int4 GEMV's weight stream (blocks of 256 threads x eight 16-byte loads, rows of
+ * 11008 bytes when bytes is a multiple of 11008 * 256, else of 128 bytes) and computes nothing.  Its duration is the
+ * floor of any single launch that has to bring these bytes on chip.  sink_dev: 4096 words of scratch (never
+ * written in practice). */
+int art_read_bytes(const void* src_dev, size_t bytes, void* sink_dev, void* stream);
+
+/* Store-only counterpart: one launch that writes `bytes` (a multiple of 16, 16-byte aligned) of the 32-bit `value`
+ * with non-temporal 16-byte stores and reads nothing: the floor of a launch that has to write these bytes. */
+int art_fill_bytes(void* dst_dev, size_t bytes, unsigned int value, void* stream);
+
+/* Measurement only, no counterpart in the reference: what a grid-wide meeting inside ONE launch costs on this part,
+ * i.e. what a persistent whole-token kernel would pay instead of a dependent launch.  256 resident blocks run `phases`
+ * phases over src_dev (phases * phase_bytes bytes, at most src_bytes; phase_bytes a multiple of 32768, at most
+ * 24 MiB); in every phase a block fetches its share with the access pattern of art_read_bytes, then all blocks meet
+ * through one word per block in the stream's workspace (agent-scope stores and loads, no atomics, no fences, every
+ * wait bounded).  mode 0: no loads; 1: a phase's loads follow the previous meeting; 2: the next phase's loads are
+ * issued before the meeting.  status_dev: one 32-bit word, zero before the call, 1 afterwards if a block gave up
+ * waiting (the chip was not free to hold all 256 blocks).  sink_dev: 256 words of scratch. */
+int art_phase_chain_probe(const void* src_dev, size_t src_bytes, size_t phase_bytes, int phases, int mode, void* sink_dev,
+                          void* status_dev, void* stream);
 
 #ifdef __cplusplus
 }

@@ -141,8 +141,8 @@ def test_tune_config_times_candidates_and_keeps_the_winner(ops_dir):
 
 @pytest.mark.gpu
 def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
-    """config="tune:N" on a program that runs on a hand-written kernel searches that kernel's launch parameter (rows
-    per lane of the int4 GEMV, K-splits and rows per block of the int4 GEMM) for the shape of the call, keeps the winner in the module
+    """config="tune:N" on a program that runs on a hand-written kernel searches that kernel's launch parameters (rows
+    per lane x wavefronts per block of the int4 GEMV, K-splits x rows per block of the int4 GEMM) for the shape of the call, keeps the winner in the module
     file, and the tuned operator - like every value of the parameter - matches the oracle."""
     import subprocess
     from ctypes import c_void_p
@@ -156,25 +156,28 @@ def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
     f = autort.export(ir=patterns.W4A16_IR, inputs=patterns.W4A16_INPUTS, name='w4a16_tuned', config='tune:8')
     lib = capi.lib()
     for M, K, N, key, entry, values in [
-            (1, 4096, 4096, 'gemv_w4a16.k_per_block|1,4096,4096', lib.art_gemv_w4a16_tuned, (0, 256, 512, 1024)),
-            (1, 11008, 528, 'gemv_w4a16.k_per_block|1,11008,528', lib.art_gemv_w4a16_tuned, (256, 512, 1024)),
-            (2, 1024, 1040, 'gemv_w4a16.k_per_block|2,1024,1040', lib.art_gemv_w4a16_tuned, (256, 512)),
+            (1, 4096, 4096, 'gemv_w4a16.rows_x16_plus_waves|1,4096,4096', lib.art_gemv_w4a16_knobs, ((0, 0), (8, 4), (4, 4), (8, 8), (4, 8), (0, 8), (4, 0))),
+            (1, 11008, 528, 'gemv_w4a16.rows_x16_plus_waves|1,11008,528', lib.art_gemv_w4a16_knobs, ((8, 4), (4, 4), (8, 8), (4, 8))),
+            (2, 1024, 1040, 'gemv_w4a16.rows_x16_plus_waves|2,1024,1040', lib.art_gemv_w4a16_knobs, ((8, 4), (4, 4))),
             (64, 4096, 4096, 'gemm_w4a16.k_splits|64,4096,4096', lib.art_gemm_w4a16_tuned, (0, 1, 3, 8, 32, 255, 256 + 2, 256 + 8, 256, 512 + 3))]:
         print(f'[case] tuned int4 product M={M} K={K} N={N}', flush=True)
         p = workloads.w4_problem(M + K + N, M, K, N)
         want = hot_ops.gemm_w4a16(p['x'].numpy(), p['qweight'].numpy(), p['scales'].numpy(), p['qzeros'].numpy()).astype(np.float32)
         d = [p[k].to(dev) for k in ('x', 'qweight', 'scales', 'qzeros')]
+        if (M, K, N) == (1, 4096, 4096):
+            d1, want1 = d, want
         got = f(*d)
         assert np.allclose(got.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
         choice = f.tuned[key]
-        assert choice['us'] > 0 and (choice['value'] in (256, 512, 1024) if 'gemv' in key
+        assert choice['us'] > 0 and (choice['value'] in (8 * 16 + 4, 4 * 16 + 4, 8 * 16 + 8, 4 * 16 + 8) if 'gemv' in key
                                     else (choice['value'] & 255) <= K // 128 and choice['value'] >> 8 in (0, 1, 2))
         assert store.load('w4a16_tuned')['tuned'][key] == choice
         assert torch.equal(f(*d), got)                              # the stored choice is used again, no new search
         for v in values:                                            # every value of the parameter gives the oracle's result
             y = torch.full((M, N), float('nan'), dtype=torch.float16, device=dev)
+            knobs = v if isinstance(v, tuple) else (v,)
             capi.check(entry(c_void_p(d[0].data_ptr()), c_void_p(d[1].data_ptr()), c_void_p(d[2].data_ptr()), c_void_p(d[3].data_ptr()),
-                             c_void_p(y.data_ptr()), M, K, N, v, None))
+                             c_void_p(y.data_ptr()), M, K, N, *knobs, None))
             torch.cuda.synchronize()
             assert np.allclose(y.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2), v
     # a later session finds the choices
@@ -183,6 +186,13 @@ def test_tune_config_searches_the_hand_kernels_launch_parameters(ops_dir):
     # a value outside the parameter's range is refused
     assert lib.art_gemv_w4a16_tuned(None, None, None, None, None, 1, 4096, 4096, 5, None) != 0
     assert b'k_per_block' in lib.art_last_error()
+    for k_per_block in (256, 512, 1024):                            # the older single knob still names three of the four combinations
+        y = torch.full((1, 4096), float('nan'), dtype=torch.float16, device=dev)
+        capi.check(lib.art_gemv_w4a16_tuned(c_void_p(d1[0].data_ptr()), c_void_p(d1[1].data_ptr()), c_void_p(d1[2].data_ptr()),
+                                            c_void_p(d1[3].data_ptr()), c_void_p(y.data_ptr()), 1, 4096, 4096, k_per_block, None))
+        assert np.allclose(y.float().cpu().numpy(), want1, rtol=1e-2, atol=1e-2), k_per_block
+    assert lib.art_gemv_w4a16_knobs(None, None, None, None, None, 1, 4096, 4096, 5, 4, None) != 0 and b'rows_per_lane' in lib.art_last_error()
+    assert lib.art_gemv_w4a16_knobs(None, None, None, None, None, 2, 4096, 4096, 8, 8, None) != 0 and b'M = 1' in lib.art_last_error()
     assert lib.art_gemm_w4a16_tuned(None, None, None, None, None, 64, 4096, 4096, 0x300, None) != 0
     assert b'rows-per-block' in lib.art_last_error()
 
@@ -218,3 +228,24 @@ def test_partition_tuning_keeps_results_bit_exact(ops_dir):
     assert np.array_equal(op(xd).cpu().numpy(), want)
     fresh = PartitionEvenFirst()
     assert np.array_equal(fresh(xd).cpu().numpy(), want) and fresh.tuned[str(n)] == rec
+
+
+@pytest.mark.gpu
+def test_tune_config_searches_the_fp16_gemm_block_shape(ops_dir):
+    """config="tune:N" on the fp16 matrix product times both block shapes of `art_gemm_f16_tuned` (256 or 512
+    threads per 256 x 256 tile) for the shape of the call and keeps the faster one; the result is the fp64 product
+    either way."""
+    import autort
+    from antares_amd.autort import patterns, store
+    dev = autort.device()
+    f = autort.export(ir=patterns.GEMM_F16_IR, inputs=patterns.GEMM_F16_INPUTS, name='gemm_f16_tuned', config='tune:2')
+    g = torch.Generator().manual_seed(9)
+    a = (torch.randn(1024, 512, generator=g) * 0.05).half()
+    b = (torch.randn(512, 768, generator=g) * 0.05).half()
+    got = f(a.to(dev), b.to(dev))
+    want = (a.double() @ b.double()).float()
+    assert torch.allclose(got.float().cpu(), want, rtol=1e-2, atol=1e-2)
+    choice = f.tuned['gemm_f16.threads|1024,512,768']
+    assert choice['value'] in (256, 512) and choice['us'] > 0
+    assert store.load('gemm_f16_tuned')['tuned']['gemm_f16.threads|1024,512,768'] == choice
+    assert torch.equal(f(a.to(dev), b.to(dev)), got)
