@@ -26,6 +26,7 @@
 // A block is one wavefront per record (4 for K = 4096, 11 for K = 11008).  The 8 lanes of a group meet by the
 // reduce-scatter of art_gemv_w4.hip (lane bits 5, 4, 3; afterwards a lane holds two columns of its group), apply
 // scale and zero point, the 8 groups of the wavefront meet by three DPP steps and the wavefronts of the block in LDS.
+// (For K of 2049 .. 4096 a second form further down lets a wavefront own four columns over all of K.)
 // One tile per block: the kernel needs about 60 registers per lane, so up to eight blocks of a compute unit have their
 // loads in flight while others multiply (blocks that walk several tiles with a second register set measured 10-25 %
 // slower on every decode shape).
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_w4p_kernel(Args a, Magic 
   const unsigned char* lane_base = a.packed + (size_t)wave * kChunkBytes;
   auto issue = [&](int tile, u32x4 (&w)[8], unsigned int& sc2, unsigned int& zb, _Float16& res) {
     const unsigned char* wp = lane_base + (size_t)tile * a.tile_stride;
-    if (EPI == 1 && tid < kTileCols) res = a.residual[tile * kTileCols + tid];      // fetched with the tile, not behind its reduction
+    if constexpr (EPI == 1) res = a.residual[tile * kTileCols + (tid & 15)];      // fetched with the tile, not behind its reduction (by every lane: no divergent branch around a load)
 #pragma unroll
     for (int i = 0; i < 8; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + i * 1024 + lane * 16));
     sc2 = __builtin_nontemporal_load(reinterpret_cast<const unsigned int*>(wp + kScaleOff + (gi * 16 + 2 * sb) * 2));
@@ -280,8 +281,190 @@ __global__ __launch_bounds__(256) void w4_prepack_kernel(const unsigned char* __
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// K of 2049 .. 4096 (the hidden size of the decode step): a wavefront owns FOUR columns over all of K, so the four
+// wavefronts of a block never meet - no LDS meeting, no barrier behind the stream, every wavefront stores its own
+// four results - and a block is launched with 256 threads whatever K is.  ("Column quads"; the general form above
+// keeps 16 columns per wavefront and 1024 values of k.)
+//
+// Packed form: N/16 tiles of four records (wavefront w: columns 2w, 2w+1, 8+2w, 8+2w+1 of the tile - two from each
+// half, so that with gate | up interleaved in blocks of 8 a wavefront holds matching gate and up columns):
+//   [0, 8192)     lane l owns the 64 values of k from 64 l (quantisation group l / 2); load i (0..7) is the 16 bytes at
+//                 i*1024 + l*16: the 8 values of k from 8i of those, one 32-bit word per column, nibbles in the order
+//                 k0 k2 k4 k6 k1 k3 k5 k7 as above;
+//   [8192, 8448)  fp16 scales, lane l: group l / 2, the wavefront's columns 2 (l % 2) and 2 (l % 2) + 1 - the two a lane
+//                 holds once the two lanes of a group have met;
+//   [8448, 8512)  zero points of the same two columns, one byte per lane;  [8512, 8576) padding.
+// x goes through LDS once (thread t prepares x[16t .. 16t+15], normalised if asked, and the four threads of a lane's 64
+// values leave the two sums that go with the 1024 / 64 offsets and the zero point); a lane reads its x from there
+// while its weights are in flight.
+constexpr int kQuadMaxK = 4096, kQuadRecords = 4, kXChunkBytes = 144;   // 64 values of x + 16 bytes: neighbouring chunks lie on different banks
+
+__device__ __forceinline__ int quad_column(int wave, int c) { return (c >> 1) * 8 + 2 * wave + (c & 1); }
+
+template <bool NORM, int EPI>
+__global__ __launch_bounds__(256) void gemv_w4q_kernel(Args a, Magic magic) {
+  __shared__ __align__(16) unsigned char xs[64 * kXChunkBytes];
+  __shared__ __align__(8) float corr[64][2];                // per 64 values of k: 1024 * sum(low positions) + 64 * sum(high positions), sum(x)
+  __shared__ float s_ss[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  // ---- x: thread t prepares x[16t .. 16t+15]; past the end of K it is zero (the weights there are zeros too)
+  const bool k_ok = 16 * tid < a.K;
+  const int k0 = k_ok ? 16 * tid : 0;
+  const u32x4* xp = reinterpret_cast<const u32x4*>(a.x + k0);
+  u32x4 xv0 = xp[0], xv1 = xp[1];
+  u32x4 n0v = {0, 0, 0, 0}, n1v = {0, 0, 0, 0};
+  if constexpr (NORM) {
+    const u32x4* np = reinterpret_cast<const u32x4*>(a.norm_w + k0);
+    n0v = np[0];
+    n1v = np[1];
+  }
+  const int tile = blockIdx.x;
+  const unsigned char* wp = a.packed + (size_t)tile * a.tile_stride + (size_t)wave * kChunkBytes;
+  u32x4 w[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + i * 1024 + lane * 16));
+  const unsigned int sc2 = __builtin_nontemporal_load(reinterpret_cast<const unsigned int*>(wp + kScaleOff + lane * 4));
+  const unsigned int zb = __builtin_nontemporal_load(wp + kZeroOff + lane);
+  // after the reductions lane l < 4 holds the wavefront's column 2 (l % 2) + (l / 2): its residual comes with the tile
+  const int out_col = quad_column(wave, 2 * (lane & 1) + ((lane >> 1) & 1));
+  // (every lane loads it - the column repeats every four lanes: a load inside a divergent branch makes the compiler
+  // wait there for every load in flight)
+  _Float16 res = (_Float16)0;
+  if constexpr (EPI == 1) res = a.residual[tile * kTileCols + out_col];
+  __builtin_amdgcn_sched_barrier(0);                        // nothing below moves above the loads
+
+  if (!k_ok) { xv0 = u32x4{0, 0, 0, 0}; xv1 = u32x4{0, 0, 0, 0}; }
+  unsigned int xw[8] = {xv0[0], xv0[1], xv0[2], xv0[3], xv1[0], xv1[1], xv1[2], xv1[3]};
+  if constexpr (NORM) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const half2_t h = as_h2(xw[j]);
+      ss = fmaf((float)h.x, (float)h.x, ss);
+      ss = fmaf((float)h.y, (float)h.y, ss);
+    }
+    ss = wave_sum_all(ss);
+    if (lane == 0) s_ss[wave] = ss;
+    art_lds_barrier();                                      // LDS only: the weight loads stay in flight
+    const float r = __builtin_amdgcn_rsqf(((s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3])) * a.inv_n + a.eps);
+    const unsigned int nw[8] = {n0v[0], n0v[1], n0v[2], n0v[3], n1v[0], n1v[1], n1v[2], n1v[3]};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const half2_t xh = as_h2(xw[j]), wh = as_h2(nw[j]);
+      const half2_t o = {(_Float16)fmaf(fmaf((float)xh.x, r, 0.f), (float)wh.x, 0.f), (_Float16)fmaf(fmaf((float)xh.y, r, 0.f), (float)wh.y, 0.f)};
+      xw[j] = __builtin_bit_cast(unsigned int, o);
+    }
+  }
+  {
+    const half2_t ones = {(_Float16)1, (_Float16)1};
+    float se = 0.f, so = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      se = __builtin_amdgcn_fdot2(as_h2(xw[j]), ones, se, false);
+      so = __builtin_amdgcn_fdot2(as_h2(xw[j + 1]), ones, so, false);
+    }
+    se += ART_DPP_F(se, 0xB1); se += ART_DPP_F(se, 0x4E);  // the four threads of 64 values of k are a quad
+    so += ART_DPP_F(so, 0xB1); so += ART_DPP_F(so, 0x4E);
+    if ((tid & 3) == 0) *reinterpret_cast<f32x2*>(&corr[tid >> 2][0]) = f32x2{1024.f * se + 64.f * so, se + so};
+    unsigned char* dst = xs + (tid >> 2) * kXChunkBytes + (tid & 3) * 32;
+    *reinterpret_cast<u32x4*>(dst) = u32x4{xw[0], xw[1], xw[2], xw[3]};
+    *reinterpret_cast<u32x4*>(dst + 16) = u32x4{xw[4], xw[5], xw[6], xw[7]};
+  }
+  art_lds_barrier();
+
+  // ---- multiply: the lane's 64 values of k, 8 at a time as the loads arrive, against its x from LDS
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const unsigned char* xsrc = xs + lane * kXChunkBytes;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const u32x4 xq = *reinterpret_cast<const u32x4*>(xsrc + 16 * i);
+    const unsigned int xo[4] = {xq[0], xq[1], xq[2], xq[3]};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = mac_word(w[i][c], xo, acc[c], magic);
+  }
+  // ---- the two lanes of a group meet (lane bit 0): the even lane keeps columns 0, 1, the odd one 2, 3; so do their sums of x
+  // (the two sums are copied out of the loaded register pair before they go through DPP: with the pair's second
+  // half as a DPP source the compiler's DPP combiner picks the first half)
+  float c0 = corr[lane][0], c1 = corr[lane][1];
+  asm volatile("" : "+v"(c0), "+v"(c1));
+  const bool odd = (lane & 1) != 0;
+  const float v0 = (odd ? acc[2] : acc[0]) + ART_DPP_F(odd ? acc[0] : acc[2], 0xB1);
+  const float v1 = (odd ? acc[3] : acc[1]) + ART_DPP_F(odd ? acc[1] : acc[3], 0xB1);
+  const float a0 = c0 + ART_DPP_F(c0, 0xB1), a1 = c1 + ART_DPP_F(c1, 0xB1);
+  const half2_t s2 = as_h2(sc2);
+  const float z0 = (float)(zb & 15), z1 = (float)(zb >> 4);
+  const float r0 = (float)s2.x * (v0 - a0 - z0 * a1), r1 = (float)s2.y * (v1 - a0 - z1 * a1);
+  // ---- the 32 groups meet: lane bit 1 splits the two columns, bits 2..5 are summed (rotations inside a row of 16
+  // lanes, swaps between rows); lane l < 4 then holds column 2 (l % 2) + (l / 2) of the wavefront
+  const bool b1 = (lane & 2) != 0;
+  float r = (b1 ? r1 : r0) + ART_DPP_F(b1 ? r0 : r1, 0x4E);
+  r += ART_DPP_F(r, 0x124);                                 // row_ror:4
+  r += ART_DPP_F(r, 0x128);                                 // row_ror:8
+  r = swap16_add(r, r);
+  r = swap32_add(r, r);
+  if constexpr (EPI == 2) {
+    // the wavefront's columns are gate 2w, gate 2w+1, up 2w, up 2w+1 of the tile: the up value sits in the neighbouring lane
+    const float up = ART_DPP_F(r, 0xB1);
+    if (lane < 4 && !odd) {
+      const float gf = (float)(_Float16)r, uf = (float)(_Float16)up;
+      a.y[tile * 8 + 2 * wave + (lane >> 1)] = (_Float16)(gf / (1.0f + expf(0.0f - gf)) * uf);
+    }
+  } else if (lane < 4) {
+    _Float16 o = (_Float16)r;
+    if constexpr (EPI == 1) o = (_Float16)((float)o + (float)res);
+    a.y[tile * kTileCols + out_col] = o;
+  }
+}
+
+// Repack for the column-quad form: one block per (tile, wavefront record).
+__global__ __launch_bounds__(256) void w4_prepack_quad_kernel(const unsigned char* __restrict__ qweight, const _Float16* __restrict__ scales,
+                                                               const unsigned char* __restrict__ qzeros, unsigned char* __restrict__ packed,
+                                                               int K, int N, unsigned int tile_stride) {
+  const int tile = blockIdx.x, wave = blockIdx.y, tid = threadIdx.x;
+  const int groups = K >> 7;
+  unsigned char* rec = packed + (size_t)tile * tile_stride + (size_t)wave * kChunkBytes;
+  for (int wi = tid; wi < 2048; wi += 256) {
+    const int i = wi >> 8, l = (wi >> 2) & 63, c = wi & 3;
+    const int kb = 64 * l + 8 * i;                          // first of the word's 8 values of k
+    unsigned int word = 0;
+    if ((kb >> 7) < groups) {
+      const unsigned char* src = qweight + (size_t)(kb >> 1) * N + tile * kTileCols + quad_column(wave, c);
+      const unsigned int b0 = src[0], b1 = src[(size_t)N], b2 = src[(size_t)2 * N], b3 = src[(size_t)3 * N];
+      word = (b0 & 15u) | ((b1 & 15u) << 4) | ((b2 & 15u) << 8) | ((b3 & 15u) << 12) |
+             ((b0 >> 4) << 16) | ((b1 >> 4) << 20) | ((b2 >> 4) << 24) | ((b3 >> 4) << 28);
+    }
+    reinterpret_cast<unsigned int*>(rec)[wi] = word;
+  }
+  if (tid < 64) {                                           // lane tid: group tid / 2, the two columns it keeps
+    const int g = tid >> 1;
+    _Float16 s0 = (_Float16)0, s1 = (_Float16)0;
+    unsigned int z = 0;
+    if (g < groups) {
+      const int c0 = tile * kTileCols + quad_column(wave, 2 * (tid & 1)), c1 = c0 + 1;
+      s0 = scales[(size_t)g * N + c0];
+      s1 = scales[(size_t)g * N + c1];
+      const unsigned int zbyte = qzeros[(size_t)g * (N >> 1) + (c0 >> 1)];      // c0 is even: both columns in one byte
+      z = zbyte;
+    }
+    reinterpret_cast<_Float16*>(rec + kScaleOff)[2 * tid] = s0;
+    reinterpret_cast<_Float16*>(rec + kScaleOff)[2 * tid + 1] = s1;
+    rec[kZeroOff + tid] = (unsigned char)z;
+  } else if (tid < 128) {
+    rec[kZeroOff + tid] = 0;                                // padding
+  }
+  if (wave == 0) {
+    const unsigned int used = kQuadRecords * kChunkBytes;
+    for (unsigned int o = used + tid; o < tile_stride; o += 256) packed[(size_t)tile * tile_stride + o] = 0;
+  }
+}
+
+inline bool quad_form(int K) { return K > kQuadMaxK / 2 && K <= kQuadMaxK; }
 inline int chunks_of(int K) { return (K + kChunkK - 1) / kChunkK; }
-inline size_t tile_stride_of(int K) { return (((size_t)chunks_of(K) * kChunkBytes) + 255) & ~(size_t)255; }
+inline int records_of(int K) { return quad_form(K) ? kQuadRecords : chunks_of(K); }
+inline size_t tile_stride_of(int K) { return (((size_t)records_of(K) * kChunkBytes) + 255) & ~(size_t)255; }
 
 int check_shape(const char* who, int K, int N) {
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "%s: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", who, K, N);
@@ -309,7 +492,11 @@ extern "C" int art_w4_prepack(const void* qweight_dev, const void* scales_dev, c
                   !art::overlaps(packed_dev, bytes, qzeros_dev, (size_t)(K / 128) * (N / 2)),
               "art_w4_prepack: the packed buffer must not overlap the inputs");
   ART_REQUIRE(stride <= 0xffffffffu, "art_w4_prepack: K too large");
-  const dim3 grid(N / kTileCols, chunks_of(K));
+  const dim3 grid(N / kTileCols, records_of(K));
+  if (quad_form(K))
+    w4_prepack_quad_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
+                                                                 (const unsigned char*)qzeros_dev, (unsigned char*)packed_dev, K, N, (unsigned int)stride);
+  else
   w4_prepack_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const unsigned char*)qweight_dev, (const _Float16*)scales_dev,
                                                           (const unsigned char*)qzeros_dev, (unsigned char*)packed_dev, K, N, (unsigned int)stride);
   ART_LAUNCH_CHECK();
@@ -334,7 +521,11 @@ extern "C" int art_gemv_w4p(const void* x_dev, const void* packed_dev, void* y_d
   const Magic magic{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
   const dim3 grid(blocks), block(64 * waves);
   hipStream_t st = (hipStream_t)stream;
-#define ART_W4P_LAUNCH(NORM, EPI) gemv_w4p_kernel<NORM, EPI><<<grid, block, 0, st>>>(a, magic)
+#define ART_W4P_LAUNCH(NORM, EPI)                                                          \
+  do {                                                                                    \
+    if (quad_form(K)) gemv_w4q_kernel<NORM, EPI><<<grid, dim3(256), 0, st>>>(a, magic);    \
+    else gemv_w4p_kernel<NORM, EPI><<<grid, block, 0, st>>>(a, magic);                     \
+  } while (0)
   if (norm_weight_dev != nullptr) {
     if (swiglu_out) ART_W4P_LAUNCH(true, 2);
     else if (residual_dev != nullptr) ART_W4P_LAUNCH(true, 1);
