@@ -13,6 +13,8 @@
 // over the data, 128-bit loads, fp32 math, wavefront reductions through DPP.
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "art_common.h"
 
 namespace {
@@ -136,15 +138,25 @@ constexpr int kAttGroups = kAttThreads / 8;   // 64 position groups per block
 constexpr int kAttWaves = kAttThreads / 64;
 constexpr int kAttPartialStride = 132;        // floats per (head, part) record: acc[128], max, sum, 2 of padding (16-byte rows)
 
-// Merge the online-softmax state of the lane `mask` away (same dims, other positions) into this lane's.
-__device__ __forceinline__ void att_merge_lane(float& m, float& l, float (&acc)[16], int mask) {
-  const float m2 = __shfl_xor(m, mask), l2 = __shfl_xor(l, mask);
-  const float mn = fmaxf(m, m2);
-  const float c1 = (m == -INFINITY) ? 0.f : __expf(m - mn), c2 = (m2 == -INFINITY) ? 0.f : __expf(m2 - mn);
-  l = l * c1 + l2 * c2;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = acc[i] * c1 + __shfl_xor(acc[i], mask) * c2;
-  m = mn;
+// Lane exchanges between the eight position groups of a wavefront (lanes that differ in bits 3, 4, 5).
+__device__ __forceinline__ float att_ror8(float v) {      // the value of lane ^ 8 (row_ror:8)
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+}
+// One step of a reduce-scatter between lanes l and l ^ 16 (l ^ 32): the lower lane of a pair keeps `a`, the upper one
+// keeps `b`; the swap exchanges the upper lanes' `a` with the lower lanes' `b`, so both results are the kept quantity.
+template <class F> __device__ __forceinline__ float att_swap16(float a, float b, F op) {
+  auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned int, a), __builtin_bit_cast(unsigned int, b), false, false);
+  return op(__builtin_bit_cast(float, (unsigned int)r[0]), __builtin_bit_cast(float, (unsigned int)r[1]));
+}
+template <class F> __device__ __forceinline__ float att_swap32(float a, float b, F op) {
+  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned int, a), __builtin_bit_cast(unsigned int, b), false, false);
+  return op(__builtin_bit_cast(float, (unsigned int)r[0]), __builtin_bit_cast(float, (unsigned int)r[1]));
+}
+// `op` over the eight groups; every lane gets the result.
+template <class F> __device__ __forceinline__ float att_over_groups(float v, F op) {
+  v = op(v, att_ror8(v));
+  v = att_swap16(v, v, op);
+  return att_swap32(v, v, op);
 }
 
 // ROPE = true: the block first rotates its head's q and k (rotate-half form) from the token's q|k|v vector,
@@ -163,8 +175,26 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
   __shared__ float s_acc[kAttWaves][D];
   __shared__ float s_q[D];
   __shared__ float s_k[D], s_v[D];
-  const int S = len_dev ? (*len_dev + 1) : len_host;     // device form carries the position, length = pos + 1
   const int h = blockIdx.x / parts, part = blockIdx.x % parts, tid = threadIdx.x;
+  const int sub = tid & 7, group = tid >> 3, wave = tid >> 6, lane = tid & 63;
+  const size_t row = (size_t)heads * D;
+  // From here to the first use of a cache row the code is one straight line for every lane: all loads are issued
+  // unconditionally (lanes without work re-read a valid address) and kept as loaded.  A load inside a divergent branch,
+  // or a branch join between a load and its use, makes the compiler wait for every outstanding load on the spot, which
+  // would put the trips to memory for the position, the token's vector and the cache rows one after another.
+  QT xa = (QT)0.f, xb = (QT)0.f, xv = (QT)0.f;
+  _Float16 freq = (_Float16)0.f;
+  if constexpr (ROPE) {                                   // wavefront 0 rotates q, wavefront 1 rotates k, 2 and 3 carry v
+    const int dim = heads * D;
+    const QT* src = q_or_qkv + (wave == 1 ? dim : 0) + (size_t)h * D;
+    xa = src[lane];
+    xb = src[lane + 64];
+    xv = q_or_qkv[2 * (size_t)dim + (size_t)h * D + (tid & 127)];
+    freq = inv_freq[lane];
+  }
+  const float scale = att_f[0];
+  int S;                                                  // device form carries the position, length = pos + 1
+  if constexpr (ROPE) S = *len_dev + 1; else S = len_dev ? (*len_dev + 1) : len_host;
   if (len_dev && (S < 1 || S > len_host)) {
     // The position read on the device is past the end of the cache (len_host rows): touch no cache row and
     // hand on NaN, which every consumer propagates, instead of running off the allocation.
@@ -180,76 +210,14 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
     }
     return;
   }
-  const int sub = tid & 7, group = tid >> 3;
-  const float scale = att_f[0];
-  const size_t row = (size_t)heads * D;
   // With ROPE the newest position is served from LDS: the block does not wait for its own cache write.
   const int cached = ROPE ? S - 1 : S;                    // positions read from the cache
   const int span = (cached + parts - 1) / parts;          // ... of which this block takes [s_first, Sc)
   const int s_first = part * span < cached ? part * span : cached;
   const int Sc = s_first + span < cached ? s_first + span : cached;
+  const int s_safe = Sc > 0 ? Sc - 1 : 0;                 // a row that exists, for lanes past the end (weight 0 below)
   const bool newest_here = ROPE && part == 0;             // one block of the head writes the cache row and attends to it
-
-  // this thread's share of the token's q|k|v, requested before anything else
-  float xa = 0.f, xb = 0.f, xv = 0.f;
-  if (ROPE) {
-    const int dim = heads * D;
-    if (tid < 128) {                                      // 64 pairs of q, 64 pairs of k
-      const QT* src = q_or_qkv + (tid >= 64 ? dim : 0) + (size_t)h * D;
-      xa = ld(src, tid & 63);
-      xb = ld(src, (tid & 63) + 64);
-    } else if (tid < 256) {
-      xv = ld(q_or_qkv, 2 * (size_t)dim + (size_t)h * D + (tid - 128));
-    }
-  }
-  // U positions per group are requested before the first is used, and the first round is requested
-  // before the rotary phase, which does not depend on it
-  typename Row16<KT>::Raw kf[U], vf[U];
-  auto request = [&](int s0) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int s = s0 + u * kAttGroups;
-      const int sc = s < Sc ? s : s0;                     // past the end: re-read a valid row, weight 0 below
-      Row16<KT>::load(k + (size_t)sc * row + (size_t)h * D + sub * 16, kf[u]);
-      Row16<KT>::load(v + (size_t)sc * row + (size_t)h * D + sub * 16, vf[u]);
-    }
-  };
   const int s_start = s_first + group;
-  if (s_start < Sc) request(s_start);
-
-  float qf[16];
-  if (ROPE) {
-    const int pos = S - 1;
-    if (tid < 128) {
-      const bool is_k = tid >= 64;
-      const int j = tid & 63;
-      float sn, cs;
-      sincosf((float)pos * (float)inv_freq[j], &sn, &cs);
-      const float ra = xa * cs - xb * sn, rb = xb * cs + xa * sn;
-      if (is_k) {                                         // the cache gets the rounded value, and so does this step
-        if (newest_here) {
-          KT* dst = k + (size_t)pos * row + (size_t)h * D;
-          st(dst, j, ra);
-          st(dst, j + 64, rb);
-          s_k[j] = (float)(KT)ra;
-          s_k[j + 64] = (float)(KT)rb;
-        }
-      } else {                                            // q goes through the output dtype like the separate operator
-        s_q[j] = (float)(QT)ra;
-        s_q[j + 64] = (float)(QT)rb;
-      }
-    } else if (tid < 256 && newest_here) {
-      const int e = tid - 128;
-      v[(size_t)pos * row + (size_t)h * D + e] = (KT)xv;
-      s_v[e] = (float)(KT)xv;
-    }
-    art_lds_barrier();
-#pragma unroll
-    for (int i = 0; i < 16; ++i) qf[i] = s_q[sub * 16 + i] * scale;
-  } else {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) qf[i] = ld(q_or_qkv, (size_t)h * D + sub * 16 + i) * scale;
-  }
 
   float m = -INFINITY, l = 0.f, acc[16];
 #pragma unroll
@@ -268,38 +236,106 @@ __global__ __launch_bounds__(kAttThreads) void attention_kernel(const QT* __rest
     for (int i = 0; i < 16; ++i) acc[i] = fmaf(acc[i], corr, p * value(i));
     m = mn;
   };
-  for (int s0 = s_start; s0 < Sc; s0 += kAttGroups * U) {
-    if (s0 != s_start) request(s0);
+  // The cached positions of this block, UU per group in flight: requested first, then the rotary phase (which does
+  // not depend on them), then the online softmax.
+  auto stream = [&](auto in_flight) {
+    constexpr int UU = decltype(in_flight)::value;
+    typename Row16<KT>::Raw kf[UU], vf[UU];
+    auto request = [&](int s0) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
+      for (int u = 0; u < UU; ++u) {
+        const int s = s0 + u * kAttGroups;
+        const int sc = s < Sc ? s : s_safe;
+        Row16<KT>::load(k + (size_t)sc * row + (size_t)h * D + sub * 16, kf[u]);
+        Row16<KT>::load(v + (size_t)sc * row + (size_t)h * D + sub * 16, vf[u]);
+      }
+    };
+    request(s_start);
+    float qf[16];
+    if constexpr (ROPE) {
+      const int pos = S - 1;
+      if (tid < 128) {
+        float sn, cs;
+        sincosf((float)pos * (float)freq, &sn, &cs);
+        const float fa = (float)xa, fb = (float)xb;
+        const float ra = fa * cs - fb * sn, rb = fb * cs + fa * sn;
+        if (wave == 1) {                                  // the cache gets the rounded value, and so does this step
+          if (newest_here) {
+            KT* dst = k + (size_t)pos * row + (size_t)h * D;
+            st(dst, lane, ra);
+            st(dst, lane + 64, rb);
+            s_k[lane] = (float)(KT)ra;
+            s_k[lane + 64] = (float)(KT)rb;
+          }
+        } else {                                          // q goes through the output dtype like the separate operator
+          s_q[lane] = (float)(QT)ra;
+          s_q[lane + 64] = (float)(QT)rb;
+        }
+      } else if (tid < 256 && newest_here) {
+        const int e = tid - 128;
+        v[(size_t)pos * row + (size_t)h * D + e] = (KT)(float)xv;
+        s_v[e] = (float)(KT)(float)xv;
+      }
+      art_lds_barrier();
+#pragma unroll
+      for (int i = 0; i < 16; ++i) qf[i] = s_q[sub * 16 + i] * scale;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) qf[i] = ld(q_or_qkv, (size_t)h * D + sub * 16 + i) * scale;
+    }
+    for (int s0 = s_start; s0 < Sc; s0 += kAttGroups * UU) {
+      if (s0 != s_start) request(s0);
+#pragma unroll
+      for (int u = 0; u < UU; ++u) {
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) d = fmaf(qf[i], Row16<KT>::at(kf[u], i), d);
+        d = group_sum(d);
+        if (s0 + u * kAttGroups < Sc) absorb(d, [&](int i) { return Row16<KT>::at(vf[u], i); });
+      }
+    }
+    if (newest_here) {                                    // the newest position, from LDS, joins group 0
+      float kn[16], vn[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        kn[i] = s_k[sub * 16 + i];
+        vn[i] = s_v[sub * 16 + i];
+      }
       float d = 0.f;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) d = fmaf(qf[i], Row16<KT>::at(kf[u], i), d);
+      for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kn[i], d);
       d = group_sum(d);
-      if (s0 + u * kAttGroups < Sc) absorb(d, [&](int i) { return Row16<KT>::at(vf[u], i); });
+      if (group == 0) absorb(d, [&](int i) { return vn[i]; });
     }
-  }
-  if (newest_here) {                                      // the newest position, from LDS, joins group 0
-    float kn[16], vn[16];
+  };
+  // A block with at most one position per group (the usual case when several blocks share a head) keeps one row per
+  // group in flight: every further one would be a second copy of the same row, and a wavefront's 16-byte load
+  // occupies the compute unit's load path for 16 cycles whether it hits or not.
+  if (Sc - s_first <= kAttGroups) stream(std::integral_constant<int, 1>()); else stream(std::integral_constant<int, U>());
+  // The eight groups of a wavefront become one state: a common maximum, then the weighted sums.  The 16 outputs per
+  // lane are summed over the groups by a reduce-scatter over lane bits 3, 4, 5 (16 -> 8 -> 4 -> 2 dims per lane, 14
+  // exchanges instead of one per output and level), which leaves every lane with two dims of the wavefront's total.
+  {
+    const auto vmax = [](float a, float b) { return fmaxf(a, b); };
+    const auto vadd = [](float a, float b) { return a + b; };
+    const float mw = att_over_groups(m, vmax);
+    const float wgt = (m == -INFINITY) ? 0.f : __expf(m - mw);
+    const float lw = att_over_groups(l * wgt, vadd);
+    const bool up = lane & 8;
+    float r8[8], r4[4], r2[2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      kn[i] = s_k[sub * 16 + i];
-      vn[i] = s_v[sub * 16 + i];
+    for (int i = 0; i < 8; ++i) {
+      const float lo = acc[i] * wgt, hi = acc[8 + i] * wgt;
+      r8[i] = (up ? hi : lo) + att_ror8(up ? lo : hi);
     }
-    float d = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) d = fmaf(qf[i], kn[i], d);
-    d = group_sum(d);
-    if (group == 0) absorb(d, [&](int i) { return vn[i]; });
-  }
-  att_merge_lane(m, l, acc, 8);       // the eight groups of a wavefront: lanes that differ in bits 3..5
-  att_merge_lane(m, l, acc, 16);
-  att_merge_lane(m, l, acc, 32);
-  const int wave = tid >> 6;
-  if ((tid & 63) < 8) {
-    if (sub == 0) { s_m[wave] = m; s_l[wave] = l; }
+    for (int i = 0; i < 4; ++i) r4[i] = att_swap16(r8[i], r8[i + 4], vadd);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) s_acc[wave][sub * 16 + i] = acc[i];
+    for (int i = 0; i < 2; ++i) r2[i] = att_swap32(r4[i], r4[i + 2], vadd);
+    const int dim0 = sub * 16 + (lane & 8) + ((lane & 16) >> 2) + ((lane & 32) >> 4);
+    s_acc[wave][dim0] = r2[0];
+    s_acc[wave][dim0 + 1] = r2[1];
+    if (lane == 0) { s_m[wave] = mw; s_l[wave] = lw; }
   }
   art_lds_barrier();                  // LDS only: the cache-row stores above need not have landed
   if (tid < D) {

@@ -6,6 +6,7 @@
     python bench.py --read-floor                      # only the read-only launch over the headline's weight bytes
     python bench.py --stream-floors                   # read-only, store-only and copy launches over 22.5 / 67 MB
     python bench.py --phase-chain                     # phases that meet inside ONE launch against dependent launches
+    python bench.py --attention                       # only the decode attention at positions 0 / 127 / 255 / 383
 
 Headline workload (BASELINE.json: "int4-GEMV HBM GB/s"): the int4 group-128
 GEMV y[1,11008] = x[1,4096] @ dequant(W), through ``autort.export`` and the
@@ -73,6 +74,8 @@ def parse_args():
                     help='run only the read-only, store-only and copy launches (what one launch needs to move bytes), and exit')
     ap.add_argument('--lowering', action='store_true',
                     help='run only the generic lowering on a set of programs (products, convolutions, reductions, rows, copies), one JSON line each, and exit')
+    ap.add_argument('--attention', action='store_true',
+                    help='run only the decode attention (rotary + cache write + attention over 8 blocks per head) at several positions, and exit')
     ap.add_argument('--phase-chain', action='store_true',
                     help='run only the probe of phases meeting inside one launch (a persistent kernel against dependent launches), and exit')
     return ap.parse_args()
@@ -309,6 +312,34 @@ def bench_phase_chain(torch, capi, phases=32, nbytes=2048 * 11008, runs=5):
             capi.check(lib.art_read_bytes(c_void_p(src.data_ptr() + i * nbytes), nbytes, c_void_p(sink.data_ptr()), c_void_p(st)))
     out['dependent_launches_us_per_phase'] = round(time_graph(torch, capi, launches, 20, 3) / phases * 1e6, 3)
     return out
+
+
+def bench_attention(torch, autort, capi, steps, warmup, layers=LAYERS, heads=32, head_dim=128, max_seq=384, parts=8):
+    """The decode attention of one step by itself: `attention_rope_split_f16` (rotary of q and k, both cache writes,
+    attention over rows 0..pos in `parts` blocks per head) on `layers` distinct caches per replayed graph, at several
+    positions.  Bytes per launch: the K and V rows it reads (2 * (pos + 1) * heads * head_dim fp16) plus q|k|v."""
+    dev = autort.device()
+    d = heads * head_dim
+    g = torch.Generator().manual_seed(3)
+    keys = (torch.randn(layers, max_seq, d, generator=g) * 0.5).half().to(dev)
+    vals = (torch.randn(layers, max_seq, d, generator=g) * 0.5).half().to(dev)
+    qkv = [(torch.randn(3 * d, generator=g)).half().to(dev) for _ in range(layers)]
+    inv = (1.0 / (10000.0 ** (torch.arange(0, head_dim, 2).float() / head_dim))).half()
+    inv_freq = torch.cat([inv, inv]).to(dev)
+    att_f = torch.tensor([head_dim ** -0.5], dtype=torch.float32, device=dev)
+    partial = [torch.zeros(heads, parts, 132, dtype=torch.float32, device=dev) for _ in range(layers)]
+    pos = torch.zeros(1, dtype=torch.int32, device=dev)
+    out = []
+    for p in (0, 127, 255, 383):
+        pos.fill_(p)
+
+        def one_pass():
+            for l in range(layers):
+                autort.ops.attention_rope_split_f16(qkv[l], inv_freq, keys[l], vals[l], att_f, partial[l], extra=[pos])
+        sec = time_graph(torch, capi, one_pass, steps, warmup) / layers
+        nbytes = 2 * (p + 1) * d * 2 + 3 * d * 2
+        out.append({'pos': p, 'us_per_launch': round(sec * 1e6, 3), 'kv_bytes_per_launch': nbytes, 'gbps': round(nbytes / sec / 1e9, 1)})
+    return {'kernel': 'attention_kernel<f16, rotary + cache write>', 'blocks_per_head': parts, 'heads': heads, 'positions': out}
 
 
 _SIDE_STREAM = None
@@ -656,6 +687,9 @@ def main():
         return
     if args.phase_chain:
         print(json.dumps(bench_phase_chain(torch, capi)), flush=True)
+        return
+    if args.attention:
+        print(json.dumps(bench_attention(torch, autort, capi, args.steps, args.warmup)), flush=True)
         return
     if args.lowering:
         bench_lowering(torch, autort, capi, args.steps, args.warmup)
