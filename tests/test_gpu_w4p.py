@@ -30,7 +30,8 @@ def to_dev(p, dev):
 # ragged sizes: one quantisation group, K below / not a multiple of a wavefront's 1024 values, a single tile,
 # the largest K; then the benchmark's four shapes and the two fused projections of the decode step
 @pytest.mark.parametrize('K,N', [(128, 16), (256, 64), (384, 144), (1152, 1040), (2048, 16), (16384, 48),
-                                 (4096, 4096), (4096, 11008), (11008, 4096), (4096, 32000), (4096, 12288), (4096, 22016)])
+                                 (4096, 4096), (4096, 11008), (11008, 4096), (4096, 32000), (4096, 12288), (4096, 22016),
+                                 (2176, 16400), (3968, 16400)])      # 1025 tiles: two tiles per block, the last block half empty
 def test_packed_gemv_matches_oracle(autort, K, N):
     from oracle import hot_ops
     note(f'gemv_w4p K={K} N={N}')
@@ -84,7 +85,7 @@ def test_packed_layout_pins_nibble_group_and_column_order(autort):
         assert torch.equal(y, want), (g, n)
 
 
-@pytest.mark.parametrize('K,N', [(512, 256), (1152, 48), (4096, 4096), (4096, 12288), (11008, 4096), (4096, 32000)])
+@pytest.mark.parametrize('K,N', [(512, 256), (1152, 48), (4096, 4096), (4096, 12288), (11008, 4096), (4096, 32000), (3968, 16400)])
 def test_packed_gemv_with_rmsnorm_and_residual(autort, K, N):
     """norm_weight / residual folded in, against rmsnorm -> gemv -> add of the oracle, and in place on the residual."""
     from oracle import hot_ops
@@ -118,7 +119,7 @@ def test_packed_gemv_with_rmsnorm_and_residual(autort, K, N):
     assert torch.allclose(got.float(), other.float(), rtol=4e-3, atol=4e-3)
 
 
-@pytest.mark.parametrize('K,F', [(512, 1024), (1152, 24), (4096, 11008)])
+@pytest.mark.parametrize('K,F', [(512, 1024), (1152, 24), (4096, 11008), (2304, 8200)])
 def test_packed_gate_up_with_swiglu_output(autort, K, F):
     """gate | up interleaved in blocks of 8 columns, RMSNorm in, SwiGLU out: against the oracle's two projections and
     silu(gate) * up as the decode step of the oracle computes it."""
