@@ -299,66 +299,49 @@ __global__ __launch_bounds__(256) void w4_prepack_kernel(const unsigned char* __
 // x goes through LDS once (thread t prepares x[16t .. 16t+15], normalised if asked, and the four threads of a lane's 64
 // values leave the two sums that go with the 1024 / 64 offsets and the zero point); a lane reads its x from there
 // while its weights are in flight.
-// With the RMSNorm in front (x and the norm weights are read by every block), two tiles per block from this many tiles
-// on: 4096 x 22016 with norm and SwiGLU 10.3 -> 10.1 us, 4096 x 32000 with norm 13.0 -> 12.9; without the norm the
-// larger blocks lose what the shared x saves (9.2 -> 9.4 us), and fewer tiles leave compute units with one block
-// where others have two.
-constexpr int kTwoTileBlocksFrom = 1024;
 constexpr int kQuadMaxK = 4096, kQuadRecords = 4, kXChunkBytes = 144;   // 64 values of x + 16 bytes: neighbouring chunks lie on different banks
 
 __device__ __forceinline__ int quad_column(int wave, int c) { return (c >> 1) * 8 + 2 * wave + (c & 1); }
 
-// WPB wavefronts per block: 4 (one tile) or 8 (two neighbouring tiles that share the block's copy of x: every block
-// reads all of x, and the norm weights with it, so on the widest shapes that side of the load path is worth halving).
-template <bool NORM, int EPI, int WPB>
-__global__ __launch_bounds__(64 * WPB) void gemv_w4q_kernel(Args a, Magic magic) {
-  constexpr int VPT = kQuadMaxK / (64 * WPB);               // values of x a thread prepares: 16 or 8
-  constexpr int TPC = 64 / VPT;                             // threads per 64 values of k: 4 or 8
+template <bool NORM, int EPI>
+__global__ __launch_bounds__(256) void gemv_w4q_kernel(Args a, Magic magic) {
   __shared__ __align__(16) unsigned char xs[64 * kXChunkBytes];
   __shared__ __align__(8) float corr[64][2];                // per 64 values of k: 1024 * sum(low positions) + 64 * sum(high positions), sum(x)
-  __shared__ float s_ss[WPB];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rec = wave & 3;
+  __shared__ float s_ss[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-  // ---- x: thread t prepares x[VPT t .. VPT t + VPT - 1]; past the end of K it is zero (the weights there are zeros too)
-  const bool k_ok = VPT * tid < a.K;
-  const int k0 = k_ok ? VPT * tid : 0;
+  // ---- x: thread t prepares x[16t .. 16t+15]; past the end of K it is zero (the weights there are zeros too)
+  const bool k_ok = 16 * tid < a.K;
+  const int k0 = k_ok ? 16 * tid : 0;
   const u32x4* xp = reinterpret_cast<const u32x4*>(a.x + k0);
-  u32x4 xv[VPT / 8], nv[VPT / 8];
-#pragma unroll
-  for (int i = 0; i < VPT / 8; ++i) {
-    xv[i] = xp[i];
-    nv[i] = u32x4{0, 0, 0, 0};
-  }
+  u32x4 xv0 = xp[0], xv1 = xp[1];
+  u32x4 n0v = {0, 0, 0, 0}, n1v = {0, 0, 0, 0};
   if constexpr (NORM) {
     const u32x4* np = reinterpret_cast<const u32x4*>(a.norm_w + k0);
-#pragma unroll
-    for (int i = 0; i < VPT / 8; ++i) nv[i] = np[i];
+    n0v = np[0];
+    n1v = np[1];
   }
-  // a block's last wavefronts may lie past the last tile: they fetch the last tile again and store nothing
-  const int tile_of_wave = blockIdx.x * (WPB / 4) + (wave >> 2);
-  const bool tile_ok = tile_of_wave < a.tiles;
-  const int tile = tile_ok ? tile_of_wave : a.tiles - 1;
-  const unsigned char* wp = a.packed + (size_t)tile * a.tile_stride + (size_t)rec * kChunkBytes;
+  const int tile = blockIdx.x;
+  const unsigned char* wp = a.packed + (size_t)tile * a.tile_stride + (size_t)wave * kChunkBytes;
   u32x4 w[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + i * 1024 + lane * 16));
   const unsigned int sc2 = __builtin_nontemporal_load(reinterpret_cast<const unsigned int*>(wp + kScaleOff + lane * 4));
   const unsigned int zb = __builtin_nontemporal_load(wp + kZeroOff + lane);
   // after the reductions lane l < 4 holds the wavefront's column 2 (l % 2) + (l / 2): its residual comes with the tile
-  const int out_col = quad_column(rec, 2 * (lane & 1) + ((lane >> 1) & 1));
+  const int out_col = quad_column(wave, 2 * (lane & 1) + ((lane >> 1) & 1));
   // (every lane loads it - the column repeats every four lanes: a load inside a divergent branch makes the compiler
   // wait there for every load in flight)
   _Float16 res = (_Float16)0;
   if constexpr (EPI == 1) res = a.residual[tile * kTileCols + out_col];
   __builtin_amdgcn_sched_barrier(0);                        // nothing below moves above the loads
 
-  unsigned int xw[VPT / 2];
-#pragma unroll
-  for (int j = 0; j < VPT / 2; ++j) xw[j] = k_ok ? xv[j / 4][j % 4] : 0u;
+  if (!k_ok) { xv0 = u32x4{0, 0, 0, 0}; xv1 = u32x4{0, 0, 0, 0}; }
+  unsigned int xw[8] = {xv0[0], xv0[1], xv0[2], xv0[3], xv1[0], xv1[1], xv1[2], xv1[3]};
   if constexpr (NORM) {
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < VPT / 2; ++j) {
+    for (int j = 0; j < 8; ++j) {
       const half2_t h = as_h2(xw[j]);
       ss = fmaf((float)h.x, (float)h.x, ss);
       ss = fmaf((float)h.y, (float)h.y, ss);
@@ -366,12 +349,11 @@ __global__ __launch_bounds__(64 * WPB) void gemv_w4q_kernel(Args a, Magic magic)
     ss = wave_sum_all(ss);
     if (lane == 0) s_ss[wave] = ss;
     art_lds_barrier();                                      // LDS only: the weight loads stay in flight
-    float ss_all = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
-    if constexpr (WPB == 8) ss_all += (s_ss[4] + s_ss[5]) + (s_ss[6] + s_ss[7]);
-    const float r = __builtin_amdgcn_rsqf(ss_all * a.inv_n + a.eps);
+    const float r = __builtin_amdgcn_rsqf(((s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3])) * a.inv_n + a.eps);
+    const unsigned int nw[8] = {n0v[0], n0v[1], n0v[2], n0v[3], n1v[0], n1v[1], n1v[2], n1v[3]};
 #pragma unroll
-    for (int j = 0; j < VPT / 2; ++j) {
-      const half2_t xh = as_h2(xw[j]), wh = as_h2(nv[j / 4][j % 4]);
+    for (int j = 0; j < 8; ++j) {
+      const half2_t xh = as_h2(xw[j]), wh = as_h2(nw[j]);
       const half2_t o = {(_Float16)fmaf(fmaf((float)xh.x, r, 0.f), (float)wh.x, 0.f), (_Float16)fmaf(fmaf((float)xh.y, r, 0.f), (float)wh.y, 0.f)};
       xw[j] = __builtin_bit_cast(unsigned int, o);
     }
@@ -380,20 +362,16 @@ __global__ __launch_bounds__(64 * WPB) void gemv_w4q_kernel(Args a, Magic magic)
     const half2_t ones = {(_Float16)1, (_Float16)1};
     float se = 0.f, so = 0.f;
 #pragma unroll
-    for (int j = 0; j < VPT / 2; j += 2) {
+    for (int j = 0; j < 8; j += 2) {
       se = __builtin_amdgcn_fdot2(as_h2(xw[j]), ones, se, false);
       so = __builtin_amdgcn_fdot2(as_h2(xw[j + 1]), ones, so, false);
     }
-    se += ART_DPP_F(se, 0xB1); se += ART_DPP_F(se, 0x4E);  // the TPC threads of 64 values of k are neighbours: a quad,
+    se += ART_DPP_F(se, 0xB1); se += ART_DPP_F(se, 0x4E);  // the four threads of 64 values of k are a quad
     so += ART_DPP_F(so, 0xB1); so += ART_DPP_F(so, 0x4E);
-    if constexpr (TPC == 8) {                               // ... or two quads (row_half_mirror brings the other quad's sum)
-      se += ART_DPP_F(se, 0x141);
-      so += ART_DPP_F(so, 0x141);
-    }
-    if ((tid & (TPC - 1)) == 0) *reinterpret_cast<f32x2*>(&corr[tid / TPC][0]) = f32x2{1024.f * se + 64.f * so, se + so};
-    unsigned char* dst = xs + (tid / TPC) * kXChunkBytes + (tid & (TPC - 1)) * (2 * VPT);
-#pragma unroll
-    for (int i = 0; i < VPT / 8; ++i) *reinterpret_cast<u32x4*>(dst + 16 * i) = u32x4{xw[4 * i], xw[4 * i + 1], xw[4 * i + 2], xw[4 * i + 3]};
+    if ((tid & 3) == 0) *reinterpret_cast<f32x2*>(&corr[tid >> 2][0]) = f32x2{1024.f * se + 64.f * so, se + so};
+    unsigned char* dst = xs + (tid >> 2) * kXChunkBytes + (tid & 3) * 32;
+    *reinterpret_cast<u32x4*>(dst) = u32x4{xw[0], xw[1], xw[2], xw[3]};
+    *reinterpret_cast<u32x4*>(dst + 16) = u32x4{xw[4], xw[5], xw[6], xw[7]};
   }
   art_lds_barrier();
 
@@ -430,11 +408,11 @@ __global__ __launch_bounds__(64 * WPB) void gemv_w4q_kernel(Args a, Magic magic)
   if constexpr (EPI == 2) {
     // the wavefront's columns are gate 2w, gate 2w+1, up 2w, up 2w+1 of the tile: the up value sits in the neighbouring lane
     const float up = ART_DPP_F(r, 0xB1);
-    if (lane < 4 && !odd && tile_ok) {
+    if (lane < 4 && !odd) {
       const float gf = (float)(_Float16)r, uf = (float)(_Float16)up;
-      a.y[tile * 8 + 2 * rec + (lane >> 1)] = (_Float16)(gf / (1.0f + expf(0.0f - gf)) * uf);
+      a.y[tile * 8 + 2 * wave + (lane >> 1)] = (_Float16)(gf / (1.0f + expf(0.0f - gf)) * uf);
     }
-  } else if (lane < 4 && tile_ok) {
+  } else if (lane < 4) {
     _Float16 o = (_Float16)r;
     if constexpr (EPI == 1) o = (_Float16)((float)o + (float)res);
     a.y[tile * kTileCols + out_col] = o;
@@ -545,9 +523,7 @@ extern "C" int art_gemv_w4p(const void* x_dev, const void* packed_dev, void* y_d
   hipStream_t st = (hipStream_t)stream;
 #define ART_W4P_LAUNCH(NORM, EPI)                                                          \
   do {                                                                                    \
-    if (quad_form(K) && NORM && tiles >= kTwoTileBlocksFrom)                               \
-      gemv_w4q_kernel<NORM, EPI, 8><<<dim3((tiles + 1) / 2), dim3(512), 0, st>>>(a, magic); \
-    else if (quad_form(K)) gemv_w4q_kernel<NORM, EPI, 4><<<grid, dim3(256), 0, st>>>(a, magic); \
+    if (quad_form(K)) gemv_w4q_kernel<NORM, EPI><<<grid, dim3(256), 0, st>>>(a, magic);    \
     else gemv_w4p_kernel<NORM, EPI><<<grid, block, 0, st>>>(a, magic);                     \
   } while (0)
   if (norm_weight_dev != nullptr) {

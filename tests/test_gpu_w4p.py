@@ -31,7 +31,7 @@ def to_dev(p, dev):
 # the largest K; then the benchmark's four shapes and the two fused projections of the decode step
 @pytest.mark.parametrize('K,N', [(128, 16), (256, 64), (384, 144), (1152, 1040), (2048, 16), (16384, 48),
                                  (4096, 4096), (4096, 11008), (11008, 4096), (4096, 32000), (4096, 12288), (4096, 22016),
-                                 (2176, 16400), (3968, 16400)])      # 1025 tiles: two tiles per block, the last block half empty
+                                 (2176, 16400), (3968, 16400)])      # an odd number of tiles (1025)
 def test_packed_gemv_matches_oracle(autort, K, N):
     from oracle import hot_ops
     note(f'gemv_w4p K={K} N={N}')
