@@ -466,11 +466,17 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 4))) 
 #pragma unroll
       for (int m = 0; m < M; ++m)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          mine[m][j] = (1LL << 56) + to_fixed(r[m][j], splits);
+        for (int j = 0; j < 2; ++j) mine[m][j] = (1LL << 56) + to_fixed(r[m][j], splits);
+      // (pinned: left alone, the scheduler moves the first use of one atomic's result - and with it the wait for
+      // that result - in front of the next atomic, and the lane pays one round trip per atomic)
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
           old[m][j] = (long long)__hip_atomic_fetch_add(slots + (size_t)m * N + col + j, (unsigned long long)mine[m][j], __ATOMIC_RELAXED,
                                                         __HIP_MEMORY_SCOPE_AGENT);
-        }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int m = 0; m < M; ++m)
 #pragma unroll
