@@ -584,7 +584,15 @@ extern "C" int art_gemv_w4a16_knobs(const void* x_dev, const void* qweight_dev, 
   ART_REQUIRE(waves_per_block == 0 || waves_per_block == 4 || waves_per_block == 8,
               "art_gemv_w4a16: waves_per_block must be 0 (library's choice), 4 or 8 (got %d)", waves_per_block);
   ART_REQUIRE(waves_per_block != 8 || M == 1, "art_gemv_w4a16: eight wavefronts per block are for M = 1 (got M = %d)", M);
-  const int rpl = rows_per_lane == 0 ? 8 : rows_per_lane, waves = waves_per_block;
+  // The library's choice: eight rows per lane, except where that many-row blocks need more than one and a half rounds
+  // of the chip (four blocks per compute unit at a time) - there blocks of half the rows fill the rounds better
+  // (M = 1, 4096 x 32000: 16.2 us against 16.9 on MI355X; the narrower benchmark shapes lose 0.1 - 1 us with them).
+  int rpl = rows_per_lane == 0 ? 8 : rows_per_lane;
+  if (rows_per_lane == 0 && M == 1) {
+    const long long blocks = (long long)((N + 127) / 128) * ((K + 511) / 512);
+    if (blocks > 6LL * art::compute_units()) rpl = 4;
+  }
+  const int waves = waves_per_block;
   ART_REQUIRE(x_dev && qweight_dev && scales_dev && qzeros_dev && y_dev, "art_gemv_w4a16: null pointer");
   ART_REQUIRE(K > 0 && N > 0 && K % 128 == 0 && N % 16 == 0, "art_gemv_w4a16: need K %% 128 == 0 and N %% 16 == 0 (K=%d N=%d)", K, N);
   ART_REQUIRE(((uintptr_t)qweight_dev % 16) == 0 && ((uintptr_t)x_dev % 16) == 0,
