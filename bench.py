@@ -7,6 +7,7 @@
     python bench.py --stream-floors                   # read-only, store-only and copy launches over 22.5 / 67 MB
     python bench.py --phase-chain                     # phases that meet inside ONE launch against dependent launches
     python bench.py --attention                       # only the decode attention at positions 0 / 127 / 255 / 383
+    python bench.py --gemv-knobs                      # only the split-K int4 GEMV with each of its launch shapes
 
 Headline workload (BASELINE.json: "int4-GEMV HBM GB/s"): the int4 group-128
 GEMV y[1,11008] = x[1,4096] @ dequant(W), through ``autort.export`` and the
@@ -76,6 +77,8 @@ def parse_args():
                     help='run only the generic lowering on a set of programs (products, convolutions, reductions, rows, copies), one JSON line each, and exit')
     ap.add_argument('--attention', action='store_true',
                     help='run only the decode attention (rotary + cache write + attention over 8 blocks per head) at several positions, and exit')
+    ap.add_argument('--gemv-knobs', action='store_true',
+                    help='run only the split-K int4 GEMV at the four benchmark shapes with every (rows per lane, wavefronts per block), and exit')
     ap.add_argument('--phase-chain', action='store_true',
                     help='run only the probe of phases meeting inside one launch (a persistent kernel against dependent launches), and exit')
     return ap.parse_args()
@@ -340,6 +343,34 @@ def bench_attention(torch, autort, capi, steps, warmup, layers=LAYERS, heads=32,
         nbytes = 2 * (p + 1) * d * 2 + 3 * d * 2
         out.append({'pos': p, 'us_per_launch': round(sec * 1e6, 3), 'kv_bytes_per_launch': nbytes, 'gbps': round(nbytes / sec / 1e9, 1)})
     return {'kernel': 'attention_kernel<f16, rotary + cache write>', 'blocks_per_head': parts, 'heads': heads, 'positions': out}
+
+
+def bench_gemv_knobs(torch, autort, capi, workloads, steps, warmup, layers=16):
+    """The split-K int4 GEMV (M = 1, benchmark layout) through `art_gemv_w4a16_knobs` with each of its four launch
+    shapes - (rows per lane, wavefronts per block) in (8, 4), (4, 4), (8, 8), (4, 8) - and with the library's own
+    choice (0, 0), `layers` rotating weight sets per replayed graph: what `tune:N` searches, and what the library's
+    rule is set by."""
+    from ctypes import c_void_p
+    dev = autort.device()
+    lib = capi.lib()
+    rows = []
+    for K, N in ((4096, 4096), (4096, 11008), (11008, 4096), (4096, 32000)):
+        sets = [{k: v.to(dev) for k, v in workloads.w4_problem(100 + i, 1, K, N).items()} for i in range(layers)]
+        y = torch.empty(1, N, dtype=torch.float16, device=dev)
+        row = {'workload': f'int4 g128 GEMV M=1 K={K} N={N}, benchmark layout', 'us_per_launch': {}}
+        for n_th, (r, w) in enumerate(((8, 4), (8, 4), (4, 4), (8, 8), (4, 8), (0, 0))):      # the first pass is not reported
+            def one_pass():
+                st = c_void_p(torch.cuda.current_stream().cuda_stream)
+                for d in sets:
+                    capi.check(lib.art_gemv_w4a16_knobs(c_void_p(d['x'].data_ptr()), c_void_p(d['qweight'].data_ptr()),
+                                                        c_void_p(d['scales'].data_ptr()), c_void_p(d['qzeros'].data_ptr()),
+                                                        c_void_p(y.data_ptr()), 1, K, N, r, w, st))
+            sec = time_graph(torch, capi, one_pass, steps, warmup) / layers
+            if n_th > 0:
+                row['us_per_launch']["library's choice" if r == 0 else f'{r} x {w}'] = round(sec * 1e6, 2)
+        rows.append(row)
+        del sets
+    return {'kernel': 'gemv_w4a16_kernel<M=1, plain>', 'launch_shapes': 'rows per lane x wavefronts per block', 'shapes': rows}
 
 
 _SIDE_STREAM = None
@@ -690,6 +721,9 @@ def main():
         return
     if args.attention:
         print(json.dumps(bench_attention(torch, autort, capi, args.steps, args.warmup)), flush=True)
+        return
+    if args.gemv_knobs:
+        print(json.dumps(bench_gemv_knobs(torch, autort, capi, workloads, args.steps, args.warmup)), flush=True)
         return
     if args.lowering:
         bench_lowering(torch, autort, capi, args.steps, args.warmup)

@@ -16,5 +16,5 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 def test_help_lists_the_stand_alone_legs():
     r = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--help'], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0
-    for flag in ('--read-floor', '--stream-floors', '--phase-chain', '--attention', '--lowering', '--calibrate-copy', '--no-cpu'):
+    for flag in ('--read-floor', '--stream-floors', '--phase-chain', '--attention', '--gemv-knobs', '--lowering', '--calibrate-copy', '--no-cpu'):
         assert flag in r.stdout, flag
